@@ -1,0 +1,124 @@
+"""ctypes binding of ``libneox_fused.so`` (the C-ABI declared in ``include/neox_fused.h``).
+
+The library is built in-tree by ``make -C gpt-neox_amd/csrc`` (see :func:`build`).
+There is no CPU or eager fallback behind these calls: if the shared object is
+missing or cannot be loaded, :func:`lib` raises ``ImportError``; if a tensor is
+not on the GPU, the wrappers raise ``RuntimeError``.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+import torch
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libneox_fused.so")
+ABI_VERSION = 1
+
+NEOX_F16, NEOX_BF16, NEOX_F32 = 0, 1, 2
+_DTYPE_CODE = {torch.float16: NEOX_F16, torch.bfloat16: NEOX_BF16, torch.float32: NEOX_F32}
+
+_c_i64p = ctypes.POINTER(ctypes.c_int64)
+_vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
+
+# name -> (restype, argtypes); one entry per declaration of include/neox_fused.h
+SIGNATURES = {
+    "neox_fused_abi_version": (ctypes.c_int, []),
+    "neox_fused_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "neox_fused_last_error": (ctypes.c_char_p, []),
+    "neox_causal_softmax_fwd": (ctypes.c_int, [_vp, _vp, _f32, _i64, _i32, _i32, _i32, _vp]),
+    "neox_causal_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _i32, _vp]),
+    "neox_masked_softmax_fwd": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+    ),
+    "neox_masked_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _vp]),
+    "neox_get_batch_per_block": (ctypes.c_int, [_i32, _i32, _i32, _i32]),
+    "neox_rope_apply": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _c_i64p, _c_i64p, _c_i64p,
+         _c_i64p, _i64, _i32, _i32, _i32, _i32, _vp],
+    ),
+    "neox_copy_bytes": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+def build(verbose=False):
+    """Compile ``libneox_fused.so`` for gfx950 with hipcc (works without a GPU)."""
+    cmd = ["make", "-C", _CSRC, "-j4", "-B"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or res.returncode != 0:
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("building libneox_fused.so failed (see output above)")
+    return LIB_PATH
+
+
+def lib():
+    """Return the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: the fused kernels are not built. "
+                "Run `make -C gpt-neox_amd/csrc` (or __graft_entry__.build())."
+            )
+        try:
+            handle = ctypes.CDLL(LIB_PATH)
+        except OSError as exc:  # unresolved HIP runtime, wrong arch, ...
+            raise ImportError(f"cannot load {LIB_PATH}: {exc}") from exc
+        for name, (restype, argtypes) in SIGNATURES.items():
+            try:
+                fn = getattr(handle, name)
+            except AttributeError as exc:
+                raise ImportError(f"{LIB_PATH} does not export {name}") from exc
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = handle.neox_fused_abi_version()
+        if got != ABI_VERSION:
+            raise ImportError(f"{LIB_PATH}: ABI version {got}, expected {ABI_VERSION}")
+        _lib = handle
+    return _lib
+
+
+def check(status):
+    """Turn a negative neox_status into ``RuntimeError`` (as torch's checks do)."""
+    if status != 0:
+        handle = lib()
+        msg = handle.neox_fused_last_error().decode() or handle.neox_fused_strerror(status).decode()
+        raise RuntimeError(msg)
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError("Only fp16 and bf16 are supported") from None
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "fused kernels need GPU tensors (got a tensor on %s); there is no CPU fallback"
+                % t.device
+            )
+
+
+def current_stream(tensor):
+    """hipStream_t of torch's current stream on the tensor's device, as an integer."""
+    return torch.cuda.current_stream(tensor.device).cuda_stream
+
+
+def strides3(t):
+    """First three element strides of a 4-D tensor as a C int64[3]."""
+    s = t.stride()
+    return (ctypes.c_int64 * 3)(s[0], s[1], s[2])

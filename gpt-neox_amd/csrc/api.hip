@@ -1,0 +1,293 @@
+// extern "C" entry points of libneox_fused.so: argument validation, error
+// reporting and hand-off to the launchers.  Validation finishes before the
+// first HIP call, so it behaves the same on a host without a GPU.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "internal.hpp"
+
+namespace neox {
+
+static thread_local char g_last_error[256] = {0};
+
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+static inline bool aligned(const void* p, uintptr_t n) {
+    return (reinterpret_cast<uintptr_t>(p) & (n - 1)) == 0;
+}
+
+static int check_launch(hipError_t e, const char* what) {
+    if (e == hipSuccess) return NEOX_OK;
+    return fail(NEOX_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+}
+
+static int check_dtype(int dtype, const char* what) {
+    if (dtype == NEOX_F16 || dtype == NEOX_BF16) return NEOX_OK;
+    return fail(NEOX_ERR_BAD_DTYPE, "%s: Only fp16 and bf16 are supported (dtype code %d)", what,
+                dtype);
+}
+
+// rows of a [.., sq, sk] score tensor must be countable in 31 bits
+static int check_rows(int64_t rows, int sq, int sk, const char* what) {
+    if (sq < 1 || sk < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: sq=%d sk=%d must be >= 1", what, sq, sk);
+    if (rows < 1 || rows > 0x7fffffffLL)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: row count %lld outside [1, 2^31)", what,
+                    (long long)rows);
+    return NEOX_OK;
+}
+
+// Plain copy with the same access shape (measurement aid).
+__global__ __launch_bounds__(256) void copy_kernel(u32x4* dst, const u32x4* src, size_t n16) {
+    size_t idx = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    u32x4 r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (idx + k * 256 < n16) r[k] = ld128(src + idx + k * 256);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (idx + k * 256 < n16) st128(dst + idx + k * 256, r[k]);
+}
+
+}  // namespace neox
+
+using namespace neox;
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+int neox_fused_abi_version(void) { return NEOX_FUSED_ABI_VERSION; }
+
+const char* neox_fused_strerror(int status) {
+    switch (status) {
+        case NEOX_OK: return "success";
+        case NEOX_ERR_NULL_POINTER: return "null pointer";
+        case NEOX_ERR_BAD_DTYPE: return "Only fp16 and bf16 are supported";
+        case NEOX_ERR_BAD_SHAPE: return "unsupported shape";
+        case NEOX_ERR_BAD_STRIDE: return "unsupported stride";
+        case NEOX_ERR_MISALIGNED: return "pointer not aligned to the element size";
+        case NEOX_ERR_LAUNCH: return "kernel launch failed";
+        default: return "unknown status";
+    }
+}
+
+const char* neox_fused_last_error(void) { return g_last_error; }
+
+int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int32_t sq,
+                            int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_causal_softmax_fwd";
+    if (!y || !x) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
+    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    a.out = y;
+    a.in0 = x;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)(batches * sq);
+    a.sq = sq;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
+                            int32_t sq, int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_causal_softmax_bwd";
+    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
+    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
+    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    a.out = dx;
+    a.in0 = dy;
+    a.in1 = y;
+    a.scale = scale;
+    a.rows = (uint32_t)(batches * sq);
+    a.sq = sq;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_bwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
+                            int32_t np, int32_t sq, int32_t sk, int32_t mask_b, int32_t dtype,
+                            void* stream) {
+    static const char* what = "neox_masked_softmax_fwd";
+    if (!y || !x || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+    if (mask_b != 1 && mask_b != b)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
+    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    a.out = y;
+    a.in0 = x;
+    a.mask = mask;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)((int64_t)b * np * sq);
+    a.sq = sq;
+    a.sk = sk;
+    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
+    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(mask, 8);
+    return check_launch(launch_softmax_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows,
+                            int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_masked_softmax_bwd";
+    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (int e = check_rows(rows, 1, sk, what)) return e;
+    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    a.out = dx;
+    a.in0 = dy;
+    a.in1 = y;
+    a.scale = scale;
+    a.rows = (uint32_t)rows;
+    a.sq = 1;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np) {
+    (void)sq;
+    (void)b;
+    (void)np;
+    if (sk < 1) return fail(NEOX_ERR_BAD_SHAPE, "neox_get_batch_per_block: sk=%d must be >= 1", sk);
+    int log2_elements = 0;
+    while ((1LL << log2_elements) < sk) ++log2_elements;
+    const long long next_pow2 = 1LL << log2_elements;
+    const int wave = (next_pow2 < kWave) ? (int)next_pow2 : kWave;
+    const int rows_per_wave = (next_pow2 <= 128) ? 2 : 1;
+    const int waves_per_block = 128 / wave;
+    return waves_per_block * rows_per_wave;
+}
+
+static int check_rope_strides(const int64_t* st, const char* what, const char* name) {
+    if (!st) return fail(NEOX_ERR_NULL_POINTER, "%s: %s strides are null", what, name);
+    for (int i = 0; i < 3; ++i)
+        if (st[i] < 0) return fail(NEOX_ERR_BAD_STRIDE, "%s: %s stride[%d]=%lld is negative", what, name, i, (long long)st[i]);
+    return NEOX_OK;
+}
+
+int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, const void* cos,
+                    const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
+                    int32_t d_rot, const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                    int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
+                    int32_t backward, void* stream) {
+    static const char* what = "neox_rope_apply";
+    if (!out_q || !q || !cos || !sin) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if ((k == nullptr) != (out_k == nullptr))
+        return fail(NEOX_ERR_NULL_POINTER, "%s: k and out_k must both be given or both be null", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (cs_dtype != NEOX_F32 && cs_dtype != dtype)
+        return fail(NEOX_ERR_BAD_DTYPE, "%s: cos/sin must be fp32 or have the dtype of q (code %d)", what, cs_dtype);
+    const bool has_k = (k != nullptr);
+    if (s < 1 || b < 1 || h_q < 1 || (has_k && h_k < 1))
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: s=%d b=%d h_q=%d h_k=%d must be >= 1", what, s, b, h_q, h_k);
+    if (d_rot < 2 || (d_rot & 1))
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: d_rot=%d must be even and >= 2", what, d_rot);
+    if (b > 65535) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d exceeds 65535", what, b);
+    if (pos_offset < 0) return fail(NEOX_ERR_BAD_SHAPE, "%s: pos_offset=%d is negative", what, pos_offset);
+    if (cs_stride < d_rot) return fail(NEOX_ERR_BAD_STRIDE, "%s: cos/sin row stride %lld < d_rot=%d", what, (long long)cs_stride, d_rot);
+    if (int e = check_rope_strides(q_strides, what, "q")) return e;
+    if (int e = check_rope_strides(out_q_strides, what, "out_q")) return e;
+    if (has_k) {
+        if (int e = check_rope_strides(k_strides, what, "k")) return e;
+        if (int e = check_rope_strides(out_k_strides, what, "out_k")) return e;
+    }
+    const int cs_size = (cs_dtype == NEOX_F32) ? 4 : 2;
+    if (!aligned(q, 2) || !aligned(out_q, 2) || (has_k && (!aligned(k, 2) || !aligned(out_k, 2))) ||
+        !aligned(cos, cs_size) || !aligned(sin, cs_size))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    const int half = d_rot / 2;
+    // widest slot (elements) every access of the call can use
+    auto fits = [&](int w) {
+        if (half % w) return false;
+        const uintptr_t bytes = (uintptr_t)w * 2;
+        auto ok_t = [&](const void* p, const int64_t* st) {
+            return aligned(p, bytes) && st[0] % w == 0 && st[1] % w == 0 && st[2] % w == 0;
+        };
+        if (!ok_t(q, q_strides) || !ok_t(out_q, out_q_strides)) return false;
+        if (has_k && (!ok_t(k, k_strides) || !ok_t(out_k, out_k_strides))) return false;
+        // table accesses are at most 128 bits wide
+        const int tw = (cs_size == 4 && w > 4) ? 4 : w;
+        const uintptr_t tbytes = (uintptr_t)tw * cs_size;
+        return aligned(cos, tbytes) && aligned(sin, tbytes) && cs_stride % tw == 0;
+    };
+    int w = 1;
+    for (int cand : {8, 4, 2})
+        if (fits(cand)) {
+            w = cand;
+            break;
+        }
+    const int lpv = half / w;
+    if (lpv > 256) return fail(NEOX_ERR_BAD_SHAPE, "%s: d_rot=%d too large for slot width %d", what, d_rot, w);
+
+    // collapse (b, h) into one loop when every layout allows it
+    auto collapsible = [&](const int64_t* st, int h) { return b == 1 || st[1] == (int64_t)h * st[2]; };
+    bool collapse = collapsible(q_strides, h_q) && collapsible(out_q_strides, h_q);
+    if (has_k) collapse = collapse && collapsible(k_strides, h_k) && collapsible(out_k_strides, h_k);
+
+    RopeArgs a{};
+    auto fill = [&](RopeTensor& t, const void* in, void* out, const int64_t* is, const int64_t* os, int h) {
+        t.in = static_cast<const char*>(in);
+        t.out = static_cast<char*>(out);
+        for (int i = 0; i < 3; ++i) {
+            t.in_stride[i] = is[i];
+            t.out_stride[i] = os[i];
+        }
+        t.n_outer = collapse ? 1 : b;
+        t.n_inner = collapse ? b * h : h;
+    };
+    if ((int64_t)b * h_q > 0x7fffffffLL || (has_k && (int64_t)b * h_k > 0x7fffffffLL))
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: b*h exceeds 2^31", what);
+    fill(a.t[0], q, out_q, q_strides, out_q_strides, h_q);
+    if (has_k) fill(a.t[1], k, out_k, k_strides, out_k_strides, h_k);
+    a.cos = static_cast<const char*>(cos);
+    a.sin = static_cast<const char*>(sin);
+    a.cs_stride = cs_stride;
+    a.pos_offset = pos_offset;
+    a.half = half;
+    a.lpv = lpv;
+    a.nt = has_k ? 2 : 1;
+    return check_launch(launch_rope(a, s, collapse ? 1 : b, w, dtype, cs_dtype, backward != 0,
+                                    (hipStream_t)stream),
+                        what);
+}
+
+int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
+    static const char* what = "neox_copy_bytes";
+    if (!dst || !src) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
+    if (nbytes < 16 || nbytes % 16) return fail(NEOX_ERR_BAD_SHAPE, "%s: nbytes=%lld must be a positive multiple of 16", what, (long long)nbytes);
+    if (!aligned(dst, 16) || !aligned(src, 16)) return fail(NEOX_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", what);
+    const size_t n16 = (size_t)nbytes / 16;
+    const size_t blocks = (n16 + 1023) / 1024;
+    if (blocks > 0x7fffffffULL) return fail(NEOX_ERR_BAD_SHAPE, "%s: nbytes too large", what);
+    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), n16);
+    return check_launch(hipGetLastError(), what);
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

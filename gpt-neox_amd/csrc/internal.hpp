@@ -1,0 +1,28 @@
+// Host-side plumbing shared by the translation units of libneox_fused.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/neox_fused.h"
+#include "rope_kernels.hpp"
+#include "softmax_kernels.hpp"
+
+namespace neox {
+
+// Records a message for neox_fused_last_error() on this thread and returns `status`.
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Launchers: pick the kernel shape for the row length and launch on `stream`.
+// `vec_ok` says that 128-bit accesses are legal (sk % 8 == 0, pointers 16-byte aligned).
+hipError_t launch_softmax_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                              hipStream_t stream);
+hipError_t launch_softmax_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                              hipStream_t stream);
+hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
+                       bool backward, hipStream_t stream);
+
+// Longest row the register-resident kernels take (16 waves x 4 chunks x 512 columns).
+constexpr int kMaxRegisterRow = 16 * 4 * kChunk;
+
+}  // namespace neox

@@ -1,0 +1,57 @@
+// Rotary embedding kernels and their launcher.
+#include "internal.hpp"
+
+namespace neox {
+
+template <typename T, typename CS, int W, bool BWD>
+static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipStream_t st) {
+    const int lpv = a.lpv;
+    const int vpb = (256 / lpv) > 0 ? (256 / lpv) : 1;  // vectors per block iteration
+    int nmax = a.t[0].n_inner;
+    if (a.nt > 1 && a.t[1].n_inner > nmax) nmax = a.t[1].n_inner;
+    const int iters = (nmax + vpb - 1) / vpb;
+    // split the vector loop over blockIdx.z until the grid has a few thousand blocks
+    long long blocks = (long long)s * n_outer;
+    int zsplit = 1;
+    if (blocks < 4096) {
+        zsplit = (int)((4096 + blocks - 1) / blocks);
+        if (zsplit > iters) zsplit = iters;
+        if (zsplit > 65535) zsplit = 65535;
+        if (zsplit < 1) zsplit = 1;
+    }
+    const dim3 grid(s, n_outer, zsplit);
+    const dim3 block(lpv, vpb);
+    hipLaunchKernelGGL((rope_kernel<T, CS, W, BWD>), grid, block, 0, st, a);
+    return hipGetLastError();
+}
+
+template <typename T, typename CS, bool BWD>
+static hipError_t launch_rope_w(const RopeArgs& a, int s, int n_outer, int w, hipStream_t st) {
+    switch (w) {
+        case 8: return launch_rope_shape<T, CS, 8, BWD>(a, s, n_outer, st);
+        case 4: return launch_rope_shape<T, CS, 4, BWD>(a, s, n_outer, st);
+        case 2: return launch_rope_shape<T, CS, 2, BWD>(a, s, n_outer, st);
+        case 1: return launch_rope_shape<T, CS, 1, BWD>(a, s, n_outer, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename T, typename CS>
+static hipError_t launch_rope_dir(const RopeArgs& a, int s, int n_outer, int w, bool backward,
+                                  hipStream_t st) {
+    return backward ? launch_rope_w<T, CS, true>(a, s, n_outer, w, st)
+                    : launch_rope_w<T, CS, false>(a, s, n_outer, w, st);
+}
+
+hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
+                       bool backward, hipStream_t stream) {
+    const bool cs32 = (cs_dtype == NEOX_F32);
+    if (dtype == NEOX_F16) {
+        return cs32 ? launch_rope_dir<F16, float>(a, s, n_outer, w, backward, stream)
+                    : launch_rope_dir<F16, F16>(a, s, n_outer, w, backward, stream);
+    }
+    return cs32 ? launch_rope_dir<BF16, float>(a, s, n_outer, w, backward, stream)
+                : launch_rope_dir<BF16, BF16>(a, s, n_outer, w, backward, stream);
+}
+
+}  // namespace neox

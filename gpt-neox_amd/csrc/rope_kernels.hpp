@@ -1,0 +1,175 @@
+// Rotary positional embedding apply for gfx950: q and k in one launch, in place or
+// out of place, over the first d_rot dims of [s, b, h, d] tensors with arbitrary
+// s/b/h strides (the inputs are usually views into a fused QKV buffer).
+//
+// One block serves one sequence position: the position's cos/sin values are loaded
+// once into registers and reused for every head of q and k.  threadIdx.x selects
+// a slot of W consecutive dims in the first half of the rotated span; the thread
+// also owns the matching W dims of the second half, so the pair (j, j + d_rot/2)
+// never crosses lanes and in-place operation is race-free.  threadIdx.y walks the
+// (b, h) vectors.  W = 8 gives 128-bit accesses; W = 4, 2, 1 serve head sizes and
+// strides that do not allow them.
+//
+// Arithmetic is fp32 with the two products rounded separately (no fused
+// multiply-add), which is bit-identical to evaluating q*cos + rotate_half(q)*sin
+// in fp32; the result is rounded once to the storage type.
+#pragma once
+
+#include "wave.hpp"
+
+namespace neox {
+
+struct RopeTensor {
+    const char* in;
+    char* out;
+    int64_t in_stride[3];   // elements: position, batch, head
+    int64_t out_stride[3];
+    int32_t n_outer;        // loop extent addressed by stride[1] (1 when b and h are collapsed)
+    int32_t n_inner;        // vectors addressed by stride[2]
+};
+
+struct RopeArgs {
+    RopeTensor t[2];
+    const char* cos;
+    const char* sin;
+    int64_t cs_stride;   // elements between consecutive positions of cos/sin
+    int32_t pos_offset;
+    int32_t half;        // d_rot / 2
+    int32_t lpv;         // slots per vector = half / W
+    int32_t nt;          // 1: q only, 2: q and k
+};
+
+template <int W>
+struct Pack;  // W 16-bit elements
+template <>
+struct Pack<8> { typedef u32x4 type; };
+template <>
+struct Pack<4> { typedef u32x2 type; };
+template <>
+struct Pack<2> { typedef uint32_t type; };
+
+template <typename T, int W>
+__device__ __forceinline__ void load_elems(const char* p, float (&f)[W]) {
+    if constexpr (W == 1) {
+        f[0] = Elem<T>::load1(p);
+    } else {
+        typedef typename Pack<W>::type P;
+        const P w = *reinterpret_cast<const P*>(p);
+        const uint32_t* u = reinterpret_cast<const uint32_t*>(&w);
+#pragma unroll
+        for (int k = 0; k < W / 2; ++k) Elem<T>::unpack(u[k], f[2 * k], f[2 * k + 1]);
+    }
+}
+
+template <typename T, int W>
+__device__ __forceinline__ void store_elems(char* p, const float (&f)[W]) {
+    if constexpr (W == 1) {
+        Elem<T>::store1(p, f[0]);
+    } else {
+        typedef typename Pack<W>::type P;
+        P w;
+        uint32_t* u = reinterpret_cast<uint32_t*>(&w);
+#pragma unroll
+        for (int k = 0; k < W / 2; ++k) u[k] = Elem<T>::pack(f[2 * k], f[2 * k + 1]);
+        *reinterpret_cast<P*>(p) = w;
+    }
+}
+
+// cos/sin table element access: CS = float reads fp32, otherwise 16-bit type CS
+template <typename CS, int W>
+__device__ __forceinline__ void load_table(const char* base, int64_t idx, float (&f)[W]) {
+    if constexpr (sizeof(CS) == 4) {
+        const float* p = reinterpret_cast<const float*>(base) + idx;
+        if constexpr (W >= 4) {
+#pragma unroll
+            for (int k = 0; k < W / 4; ++k) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(p + 4 * k);
+                f[4 * k] = v.x;
+                f[4 * k + 1] = v.y;
+                f[4 * k + 2] = v.z;
+                f[4 * k + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < W; ++k) f[k] = p[k];
+        }
+    } else {
+        load_elems<CS, W>(base + idx * 2, f);
+    }
+}
+
+template <typename T, int W, bool BWD>
+__device__ __forceinline__ void rotate(const float (&xl)[W], const float (&xh)[W],
+                                       const float (&cl)[W], const float (&ch)[W],
+                                       const float (&sl)[W], const float (&sh)[W], float (&ol)[W],
+                                       float (&oh)[W]) {
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+        if constexpr (!BWD) {
+            ol[k] = xl[k] * cl[k] - xh[k] * sl[k];
+            oh[k] = xh[k] * ch[k] + xl[k] * sh[k];
+        } else {
+            ol[k] = xl[k] * cl[k] + xh[k] * sh[k];
+            oh[k] = xh[k] * ch[k] - xl[k] * sl[k];
+        }
+    }
+}
+
+template <typename T, typename CS, int W, bool BWD>
+__global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
+    const int slot = threadIdx.x;  // < lpv by construction of the block shape
+    const int pos = blockIdx.x;
+    const int outer = blockIdx.y;
+    const int j = slot * W;
+    const int half = a.half;
+
+    float cl[W], ch[W], sl[W], sh[W];
+    const int64_t crow = (int64_t)(pos + a.pos_offset) * a.cs_stride;
+    load_table<CS, W>(a.cos, crow + j, cl);
+    load_table<CS, W>(a.cos, crow + j + half, ch);
+    load_table<CS, W>(a.sin, crow + j, sl);
+    load_table<CS, W>(a.sin, crow + j + half, sh);
+
+    const int v_step = blockDim.y * gridDim.z;
+    const int n0 = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
+    const int n1 = (a.nt > 1 && outer < a.t[1].n_outer) ? a.t[1].n_inner : 0;
+    const int nmax = max(n0, n1);
+
+    const int64_t qi = (int64_t)pos * a.t[0].in_stride[0] + (int64_t)outer * a.t[0].in_stride[1] + j;
+    const int64_t qo = (int64_t)pos * a.t[0].out_stride[0] + (int64_t)outer * a.t[0].out_stride[1] + j;
+    const int64_t ki = (int64_t)pos * a.t[1].in_stride[0] + (int64_t)outer * a.t[1].in_stride[1] + j;
+    const int64_t ko = (int64_t)pos * a.t[1].out_stride[0] + (int64_t)outer * a.t[1].out_stride[1] + j;
+
+    for (int v = threadIdx.y + blockIdx.z * blockDim.y; v < nmax; v += v_step) {
+        float ql[W], qh[W], kl[W], kh[W];
+        const bool do_q = v < n0;
+        const bool do_k = v < n1;
+        const char* qp = a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2;
+        const char* kp = a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2;
+        if (do_q) {
+            load_elems<T, W>(qp, ql);
+            load_elems<T, W>(qp + (size_t)half * 2, qh);
+        }
+        if (do_k) {
+            load_elems<T, W>(kp, kl);
+            load_elems<T, W>(kp + (size_t)half * 2, kh);
+        }
+        if (do_q) {
+            float ol[W], oh[W];
+            rotate<T, W, BWD>(ql, qh, cl, ch, sl, sh, ol, oh);
+            char* op = a.t[0].out + (qo + (int64_t)v * a.t[0].out_stride[2]) * 2;
+            store_elems<T, W>(op, ol);
+            store_elems<T, W>(op + (size_t)half * 2, oh);
+        }
+        if (do_k) {
+            float ol[W], oh[W];
+            rotate<T, W, BWD>(kl, kh, cl, ch, sl, sh, ol, oh);
+            char* op = a.t[1].out + (ko + (int64_t)v * a.t[1].out_stride[2]) * 2;
+            store_elems<T, W>(op, ol);
+            store_elems<T, W>(op + (size_t)half * 2, oh);
+        }
+    }
+}
+
+}  // namespace neox

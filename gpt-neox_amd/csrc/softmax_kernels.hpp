@@ -1,0 +1,346 @@
+// Scaled masked softmax kernels for gfx950, forward and backward.
+//
+// Work decomposition: a row of the score matrix is owned by WPR wave64s (WPR = 1
+// for rows up to 2048-4096 columns, more for longer rows).  Each wave keeps its
+// share of the row in VGPRs as fp32 -- NCH "chunks" of 512 columns, lane l owning
+// columns 8l..8l+7 of a chunk, so every load/store is one 128-bit access per lane
+// and 1 KiB contiguous per wave.  With WPR > 1 the chunks of a row are dealt
+// round-robin to its waves (balanced under the causal mask) and the row maximum
+// and sum are combined through a few floats of LDS.
+//
+// Causal rows read only the columns j <= i: chunks entirely above the diagonal
+// are neither loaded nor computed (wave-uniform branch), lanes past the diagonal
+// inside the boundary chunk issue no load; the zeros of the upper triangle are
+// still stored because the consumer reads the matrix densely.
+//
+// Arithmetic: fp32, exp(x*scale - max) evaluated as exp2(x*(scale*log2e) - max'),
+// one reciprocal per row, one rounding to the storage type on store.
+#pragma once
+
+#include "wave.hpp"
+
+namespace neox {
+
+struct SoftmaxArgs {
+    void* out;            // y (forward) or dx (backward)
+    const void* in0;      // x (forward) or dy (backward)
+    const void* in1;      // unused (forward) or y (backward)
+    const uint8_t* mask;  // masked forward only
+    float scale;          // forward: scale*log2(e); backward: scale
+    uint32_t rows;        // total number of rows (batches*sq)
+    int32_t sq;
+    int32_t sk;
+    uint32_t rows_per_mask_batch;  // np*sq: rows sharing one mask sample
+    int32_t mask_bcast;            // mask batch dim is 1
+};
+
+enum class Mask { Causal, Bytes, None };
+
+// Combine a per-wave partial across the WPR waves of a row.
+template <typename Op, int WPR, int RPB>
+__device__ __forceinline__ float row_combine(float v, float* red, int wib, int rib, int lane) {
+    if constexpr (WPR == 1) {
+        return v;
+    } else {
+        if (lane == 0) red[wib] = v;
+        __syncthreads();
+        float r = red[rib * WPR];
+#pragma unroll
+        for (int w = 1; w < WPR; ++w) r = Op::f(r, red[rib * WPR + w]);
+        return r;
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------
+template <typename T, int NCH, int WPR, int RPB, Mask MASK>
+__global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArgs a) {
+    __shared__ float red_max[WPR * RPB];
+    __shared__ float red_sum[WPR * RPB];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = threadIdx.x >> 6;  // wave in block
+    const int rib = wib / WPR;         // row in block
+    const int wir = wib % WPR;         // wave in row
+
+    uint32_t row = blockIdx.x * RPB + rib;
+    const bool store = row < a.rows;  // surplus waves of the last block recompute the last row
+    if (!store) row = a.rows - 1;     // and store nothing, so every wave reaches the barriers
+
+    const int sk = a.sk;
+    const uint32_t i = row % (uint32_t)a.sq;
+    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;  // columns that take part
+
+    const char* x = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
+    char* y = static_cast<char*>(a.out) + (size_t)row * sk * 2;
+    const uint8_t* mrow = nullptr;
+    if constexpr (MASK == Mask::Bytes) {
+        const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
+        mrow = a.mask + ((size_t)mb * a.sq + i) * sk;
+    }
+
+    float v[NCH][8];
+    u32x4 raw[NCH];
+    u32x2 mk[NCH];
+
+    // ---- issue every load of the row before the first use
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int col = (wir + WPR * c) * kChunk + lane * kVec;
+        raw[c] = u32x4{0, 0, 0, 0};
+        mk[c] = u32x2{0, 0};
+        if (col < len) {
+            raw[c] = ld128(x + (size_t)col * 2);
+            if constexpr (MASK == Mask::Bytes) mk[c] = ld64_cached(mrow + col);
+        }
+    }
+
+    // ---- scale, mask, running maximum
+    const float ninf = -__builtin_inff();
+    float mx = ninf;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
+        if (c0 < len) {
+            unpack8<T>(raw[c], v[c]);
+            const int col = c0 + lane * kVec;
+            bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
+            if constexpr (MASK == Mask::Bytes) {
+                plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
+            }
+            if (plain) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    v[c][k] *= a.scale;
+                    mx = fmaxf(mx, v[c][k]);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    bool keep = (col + k) < len;
+                    if constexpr (MASK == Mask::Bytes) {
+                        const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
+                        keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
+                    }
+                    v[c][k] = keep ? v[c][k] * a.scale : ninf;
+                    mx = fmaxf(mx, v[c][k]);
+                }
+            }
+        }
+    }
+    mx = wave_reduce<OpMax>(mx);
+    mx = row_combine<OpMax, WPR, RPB>(mx, red_max, wib, rib, lane);
+
+    // A row whose every key is masked: the unfused path fills all scores with the same
+    // value, so the result is uniform over the sk columns.
+    const bool all_masked = (mx == ninf);
+
+    // ---- exponentials and their sum
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int c0 = (wir + WPR * c) * kChunk;
+        if (c0 < len) {
+            const int col = c0 + lane * kVec;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                float e = fast_exp2(v[c][k] - mx);
+                if (all_masked) e = ((col + k) < len) ? 1.f : 0.f;
+                v[c][k] = e;
+                sum += e;
+            }
+        }
+    }
+    sum = wave_reduce<OpSum>(sum);
+    sum = row_combine<OpSum, WPR, RPB>(sum, red_sum, wib, rib, lane);
+    const float inv = 1.0f / sum;
+
+    // ---- normalise and store; chunks above the diagonal store zeros
+    if (!store) return;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int c0 = (wir + WPR * c) * kChunk;
+        const int col = c0 + lane * kVec;
+        u32x4 o = u32x4{0, 0, 0, 0};
+        if (c0 < len) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[c][k] *= inv;
+            o = pack8<T>(v[c]);
+        }
+        if (col < sk) st128(y + (size_t)col * 2, o);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// backward:  dx = scale * y * (dy - sum_j dy_j*y_j)
+// ---------------------------------------------------------------------------------
+template <typename T, int NCH, int WPR, int RPB, Mask MASK>
+__global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArgs a) {
+    __shared__ float red_sum[WPR * RPB];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = threadIdx.x >> 6;
+    const int rib = wib / WPR;
+    const int wir = wib % WPR;
+
+    uint32_t row = blockIdx.x * RPB + rib;
+    const bool store = row < a.rows;
+    if (!store) row = a.rows - 1;
+
+    const int sk = a.sk;
+    const uint32_t i = row % (uint32_t)a.sq;
+    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+
+    const char* g = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
+    const char* p = static_cast<const char*>(a.in1) + (size_t)row * sk * 2;
+    char* dx = static_cast<char*>(a.out) + (size_t)row * sk * 2;
+
+    u32x4 rg[NCH], rp[NCH];
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int col = (wir + WPR * c) * kChunk + lane * kVec;
+        rg[c] = u32x4{0, 0, 0, 0};
+        rp[c] = u32x4{0, 0, 0, 0};
+        if (col < len) {
+            rg[c] = ld128(g + (size_t)col * 2);
+            rp[c] = ld128(p + (size_t)col * 2);
+        }
+    }
+
+    float gv[NCH][8], pv[NCH][8];
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int c0 = (wir + WPR * c) * kChunk;
+        if (c0 < len) {
+            unpack8<T>(rg[c], gv[c]);
+            unpack8<T>(rp[c], pv[c]);
+            const int col = c0 + lane * kVec;
+            if (c0 + kChunk > len) {
+                // the lane holding the diagonal may have loaded columns past it
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if ((col + k) >= len) pv[c][k] = 0.f;
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) dot = fmaf(gv[c][k], pv[c][k], dot);
+        }
+    }
+    dot = wave_reduce<OpSum>(dot);
+    dot = row_combine<OpSum, WPR, RPB>(dot, red_sum, wib, rib, lane);
+
+    if (!store) return;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+        const int c0 = (wir + WPR * c) * kChunk;
+        const int col = c0 + lane * kVec;
+        u32x4 o = u32x4{0, 0, 0, 0};
+        if (c0 < len) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) gv[c][k] = a.scale * (pv[c][k] * (gv[c][k] - dot));
+            o = pack8<T>(gv[c]);
+        }
+        if (col < sk) st128(dx + (size_t)col * 2, o);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Any-shape kernels: one 256-thread block per row, element-wise accesses, the row
+// is re-read for each pass (from L2).  Used when sk is not a multiple of 8, a
+// pointer is not 16-byte aligned, or the row exceeds the register-resident limit.
+// ---------------------------------------------------------------------------------
+constexpr int kGenericThreads = 256;
+
+template <typename Op>
+__device__ __forceinline__ float block_reduce(float v, float* red) {
+    v = wave_reduce<Op>(v);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = threadIdx.x >> 6;
+    __syncthreads();  // red may still be read from the previous reduction
+    if (lane == 0) red[wib] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < kGenericThreads / kWave; ++w) r = Op::f(r, red[w]);
+    return r;
+}
+
+template <typename T, Mask MASK>
+__global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(SoftmaxArgs a) {
+    __shared__ float red[kGenericThreads / kWave];
+    const uint32_t row = blockIdx.x;
+    const int sk = a.sk;
+    const uint32_t i = row % (uint32_t)a.sq;
+    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+    const char* x = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
+    char* y = static_cast<char*>(a.out) + (size_t)row * sk * 2;
+    const uint8_t* mrow = nullptr;
+    if constexpr (MASK == Mask::Bytes) {
+        const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
+        mrow = a.mask + ((size_t)mb * a.sq + i) * sk;
+    }
+    const float ninf = -__builtin_inff();
+
+    float mx = ninf;
+    for (int j = threadIdx.x; j < len; j += kGenericThreads) {
+        bool keep = true;
+        if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
+        if (keep) mx = fmaxf(mx, Elem<T>::load1(x + (size_t)j * 2) * a.scale);
+    }
+    mx = block_reduce<OpMax>(mx, red);
+    const bool all_masked = (mx == ninf);
+
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < len; j += kGenericThreads) {
+        bool keep = true;
+        if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
+        float e = keep ? fast_exp2(Elem<T>::load1(x + (size_t)j * 2) * a.scale - mx) : 0.f;
+        if (all_masked) e = 1.f;
+        sum += e;
+    }
+    sum = block_reduce<OpSum>(sum, red);
+    const float inv = 1.0f / sum;
+
+    // y may alias x: an element is read and written by the same thread only
+    for (int j = threadIdx.x; j < sk; j += kGenericThreads) {
+        float o = 0.f;
+        if (j < len) {
+            bool keep = true;
+            if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
+            float e = keep ? fast_exp2(Elem<T>::load1(x + (size_t)j * 2) * a.scale - mx) : 0.f;
+            if (all_masked) e = 1.f;
+            o = e * inv;
+        }
+        Elem<T>::store1(y + (size_t)j * 2, o);
+    }
+}
+
+template <typename T, Mask MASK>
+__global__ __launch_bounds__(kGenericThreads) void softmax_bwd_generic_kernel(SoftmaxArgs a) {
+    __shared__ float red[kGenericThreads / kWave];
+    const uint32_t row = blockIdx.x;
+    const int sk = a.sk;
+    const uint32_t i = row % (uint32_t)a.sq;
+    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+    const char* g = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
+    const char* p = static_cast<const char*>(a.in1) + (size_t)row * sk * 2;
+    char* dx = static_cast<char*>(a.out) + (size_t)row * sk * 2;
+
+    float dot = 0.f;
+    for (int j = threadIdx.x; j < len; j += kGenericThreads)
+        dot = fmaf(Elem<T>::load1(g + (size_t)j * 2), Elem<T>::load1(p + (size_t)j * 2), dot);
+    dot = block_reduce<OpSum>(dot, red);
+
+    for (int j = threadIdx.x; j < sk; j += kGenericThreads) {
+        float o = 0.f;
+        if (j < len) {
+            const float gj = Elem<T>::load1(g + (size_t)j * 2);
+            const float pj = Elem<T>::load1(p + (size_t)j * 2);
+            o = a.scale * (pj * (gj - dot));
+        }
+        Elem<T>::store1(dx + (size_t)j * 2, o);
+    }
+}
+
+}  // namespace neox

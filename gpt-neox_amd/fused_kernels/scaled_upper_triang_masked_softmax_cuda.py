@@ -1,0 +1,61 @@
+"""Extension-level API of the causal softmax, as the autograd Function calls it.
+
+Same functions and checks as the reference's pybind module
+``scaled_upper_triang_masked_softmax_cuda``
+(megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-70,
+megatron/fused_kernels/scaled_upper_triang_masked_softmax_cuda.cu:33-90),
+served by the gfx950 kernels behind ``neox_causal_softmax_fwd/_bwd``.
+Differences: no ``seq_len <= 2048`` limit; ``scale`` stays fp32 in the forward pass.
+"""
+import torch
+
+from .. import _lib
+
+_HALF = (torch.float16, torch.bfloat16)
+
+
+def forward(input, scale_factor):
+    if input.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    _lib.require_gpu(input)
+    input = input.contiguous()
+    attn_batches, sq, sk = input.shape
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_fwd(
+                softmax_results.data_ptr(), input.data_ptr(), float(scale_factor), attn_batches,
+                sq, sk, _lib.dtype_code(input.dtype), _lib.current_stream(input),
+            )
+        )
+    return softmax_results
+
+
+def backward(output_grads, softmax_results, scale_factor):
+    """Returns d(input); like the reference, the result is written into
+    ``output_grads`` itself when that tensor is contiguous."""
+    if output_grads.dim() != 3 or softmax_results.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if output_grads.dtype != softmax_results.dtype or output_grads.shape != softmax_results.shape:
+        raise RuntimeError("output_grads and softmax_results must have the same dtype and shape")
+    _lib.require_gpu(output_grads, softmax_results)
+    output_grads = output_grads.contiguous()
+    softmax_results = softmax_results.contiguous()
+    attn_batches, sq, sk = output_grads.shape
+    if output_grads.numel() == 0:
+        return output_grads
+    with torch.cuda.device(output_grads.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_bwd(
+                output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
+                float(scale_factor), attn_batches, sq, sk, _lib.dtype_code(output_grads.dtype),
+                _lib.current_stream(output_grads),
+            )
+        )
+    return output_grads

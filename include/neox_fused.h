@@ -1,0 +1,141 @@
+/*
+ * neox_fused.h — C-ABI of libneox_fused.so
+ *
+ * Hand-written gfx950 (MI355X) kernels for GPT-NeoX's fused attention-softmax
+ * and rotary-embedding path.  Every entry point
+ *   - takes plain device pointers, sizes and a hipStream_t passed as void*;
+ *   - is asynchronous with respect to the host (no allocation, no sync);
+ *   - returns NEOX_OK (0) or a negative neox_status; it never throws or exits;
+ *   - validates its arguments before the first HIP call, so argument errors
+ *     are reported on a machine without a GPU too.
+ * The caller owns all memory.  Element type codes are neox_dtype.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative
+ * to the GPT-NeoX source tree).
+ */
+#ifndef NEOX_FUSED_H
+#define NEOX_FUSED_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NEOX_FUSED_ABI_VERSION 1
+
+typedef enum neox_dtype {
+    NEOX_F16 = 0,  /* IEEE binary16 */
+    NEOX_BF16 = 1, /* bfloat16 */
+    NEOX_F32 = 2   /* only valid for the rotary cos/sin tables */
+} neox_dtype;
+
+typedef enum neox_status {
+    NEOX_OK = 0,
+    NEOX_ERR_NULL_POINTER = -1,  /* a required pointer is NULL */
+    NEOX_ERR_BAD_DTYPE = -2,     /* "Only fp16 and bf16 are supported" */
+    NEOX_ERR_BAD_SHAPE = -3,     /* a size is <= 0 or out of the supported range */
+    NEOX_ERR_BAD_STRIDE = -4,    /* negative stride or overlapping layout */
+    NEOX_ERR_MISALIGNED = -5,    /* pointer not aligned to the element size */
+    NEOX_ERR_LAUNCH = -6         /* hipLaunchKernel reported an error */
+} neox_status;
+
+/* ABI version of the loaded library (NEOX_FUSED_ABI_VERSION at build time). */
+int neox_fused_abi_version(void);
+
+/* Static description of a status code. Never NULL. */
+const char* neox_fused_strerror(int status);
+
+/* Message of the last failing call on the calling thread ("" if none). */
+const char* neox_fused_last_error(void);
+
+/*
+ * Scaled upper-triangular (causal) masked softmax, forward.
+ *   y[m,i,j] = softmax_j(scale * x[m,i,j]) over j <= i ;  y[m,i,j] = 0 for j > i
+ * x, y: [batches, sq, sk] contiguous, same dtype (fp16/bf16); y may alias x.
+ * fp32 arithmetic, one rounding on store.  Any sq, sk >= 1 (no 2048 cap).
+ * Replaces scaled_upper_triang_masked_softmax_cuda.forward
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:31-39
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax_cuda.cu:33-59
+ */
+int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int32_t sq,
+                            int32_t sk, int32_t dtype, void* stream);
+
+/*
+ * Causal softmax backward:  dx = scale * y * (dy - sum_j(dy*y)) over j <= i,
+ * dx = 0 for j > i.  dx may alias dy (the reference overwrites dy in place).
+ * Replaces scaled_upper_triang_masked_softmax_cuda.backward
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax.cpp:41-56
+ *   megatron/fused_kernels/scaled_upper_triang_masked_softmax_cuda.cu:61-90
+ */
+int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
+                            int32_t sq, int32_t sk, int32_t dtype, void* stream);
+
+/*
+ * Scaled masked softmax, forward.
+ *   y = softmax_j(mask ? excluded : scale * x);  masked positions are exactly 0;
+ *   a row with every key masked yields the uniform 1/sk (the unfused path's result).
+ * x, y: [b, np, sq, sk] contiguous.  mask: bytes [mask_b, 1, sq, sk] contiguous,
+ * non-zero = masked, mask_b in {1, b} (broadcast over heads, and over samples if 1).
+ * Replaces scaled_masked_softmax_cuda.forward
+ *   megatron/fused_kernels/scaled_masked_softmax.cpp:33-43
+ *   megatron/fused_kernels/scaled_masked_softmax_cuda.cu:38-84
+ */
+int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
+                            int32_t np, int32_t sq, int32_t sk, int32_t mask_b, int32_t dtype,
+                            void* stream);
+
+/*
+ * Masked softmax backward: dx = scale * y * (dy - sum_j(dy*y)) over each full row.
+ * rows = b*np*sq.  dx may alias dy.
+ * Replaces scaled_masked_softmax_cuda.backward
+ *   megatron/fused_kernels/scaled_masked_softmax.cpp:45-62
+ *   megatron/fused_kernels/scaled_masked_softmax_cuda.cu:86-108
+ */
+int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows,
+                            int32_t sk, int32_t dtype, void* stream);
+
+/*
+ * Rows-per-block figure the reference's dispatcher predicate consumes; kept for
+ * API compatibility (wave64 values).  Pure host arithmetic.
+ * Replaces scaled_masked_softmax_cuda.get_batch_per_block
+ *   megatron/fused_kernels/scaled_masked_softmax.h:338-352
+ */
+int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np);
+
+/*
+ * Rotary positional embedding over the first d_rot dims of q and (optionally) k
+ * in ONE launch.  Layout [s, b, h, d_rot(+pass-through)] addressed by element
+ * strides {stride_s, stride_b, stride_h}; the last dim has stride 1.
+ *   forward : out[j]      = x[j]*cos[j]           - x[j+d_rot/2]*sin[j]
+ *             out[j+d/2]  = x[j+d/2]*cos[j+d/2]   + x[j]*sin[j+d/2]
+ *   backward: out[j]      = g[j]*cos[j]           + g[j+d/2]*sin[j+d/2]
+ *             out[j+d/2]  = g[j+d/2]*cos[j+d/2]   - g[j]*sin[j]
+ * cos/sin: [>= pos_offset + s, d_rot] rows of stride cs_stride elements, dtype
+ * cs_dtype (NEOX_F32 or the same as dtype).  Arithmetic is fp32 with separately
+ * rounded products (bit-equal to torch's fp32 q*cos + rotate_half(q)*sin), one
+ * rounding to dtype on store.  out_* may alias the inputs (in place); dims
+ * >= d_rot are never read or written.  k / out_k may both be NULL.
+ * Replaces apply_rotary_pos_emb / apply_rotary_pos_emb_torch
+ *   megatron/model/positional_embeddings.py:103-126
+ * and fused_rotary_positional_embedding.forward_cached / backward_cached
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.cpp:83-127
+ */
+int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, const void* cos,
+                    const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
+                    int32_t d_rot, const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                    int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
+                    int32_t backward, void* stream);
+
+/*
+ * Plain device-to-device copy kernel (128-bit loads/stores, same launch shape as
+ * the softmax kernels).  Measurement aid: gives the HBM copy rate and the
+ * counter calibration the roofline figures are scaled against.  nbytes % 16 == 0.
+ */
+int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NEOX_FUSED_H */

@@ -1,0 +1,16 @@
+"""CPU restatement of the reference's unfused (torch) softmax and rotary path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under ``gpt-neox_amd/`` imports this package;
+it is used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` as the checker / the timed CPU baseline.
+
+* ``torch_ref``  -- the reference's torch expressions, restated op for op.
+* ``brute``      -- an independent float64 evaluation with Python/numpy loops, used
+                    to pin ``torch_ref`` on small inputs.
+
+Pins (tests/test_oracle_*.py): the reference ships no golden vectors, fixtures or
+asserting tests for this path, so every function here is pinned by closed forms,
+invariants, brute force on tiny inputs, fp64 gradcheck and -- for the rotary
+pairing convention -- the installed ``transformers`` GPT-NeoX implementation.
+No function of this package is "parity unpinned".
+"""

@@ -1,0 +1,152 @@
+"""The reference's unfused path, restated in plain torch (runs on any device).
+
+Each function names the reference lines it follows (paths relative to the
+GPT-NeoX source tree).  Test infrastructure: never imported by the product.
+"""
+import torch
+
+
+# --- masks -------------------------------------------------------------------------
+
+
+def get_attn_mask(seq_length, device="cpu", sliding_window_width=None):
+    """Boolean ``[1, 1, s, s]`` mask, True = hidden: everything above the diagonal,
+    and (optionally) everything more than ``sliding_window_width`` below it.
+    Follows megatron/utils.py:67-80."""
+    visible = torch.tril(torch.ones((1, seq_length, seq_length), device=device))
+    visible = visible.view(1, 1, seq_length, seq_length)
+    if sliding_window_width is not None:
+        visible = torch.triu(visible, diagonal=-sliding_window_width)
+    return visible < 0.5
+
+
+def gpt2_attention_mask_func(attention_scores, ltor_mask):
+    """Fill hidden positions with the most negative finite value of the score dtype,
+    in place.  Follows megatron/model/gpt2_model.py:49-57."""
+    lowest = torch.tensor(
+        torch.finfo(attention_scores.dtype).min,
+        dtype=attention_scores.dtype,
+        device=attention_scores.device,
+    )
+    attention_scores.masked_fill_(ltor_mask, lowest)
+    return attention_scores
+
+
+def padding_mask(lengths, sq, sk, device="cpu"):
+    """``[b, 1, sq, sk]`` bool mask hiding keys ``j >= lengths[b]``."""
+    lengths = torch.as_tensor(lengths, device=device)
+    hide = torch.arange(sk, device=device)[None, None, None, :] >= lengths[:, None, None, None]
+    return hide.expand(lengths.numel(), 1, sq, sk).contiguous()
+
+
+# --- softmax -----------------------------------------------------------------------
+
+
+def forward_torch_softmax(
+    input,
+    mask,
+    scale,
+    input_in_fp16=False,
+    input_in_bf16=False,
+    softmax_in_fp32=True,
+    mask_func=gpt2_attention_mask_func,
+):
+    """scale -> mask -> softmax over the last dim -> cast back.
+    Follows FusedScaleMaskSoftmax.forward_torch_softmax,
+    megatron/model/fused_softmax.py:184-199."""
+    half_in = input_in_fp16 or input_in_bf16
+    if half_in and softmax_in_fp32:
+        input = input.float()
+    if scale is not None:
+        input = input * scale
+    if mask is not None:
+        input = mask_func(input, mask)
+    probs = torch.nn.Softmax(dim=-1)(input)
+    if half_in and softmax_in_fp32:
+        probs = probs.half() if input_in_fp16 else probs.bfloat16()
+    return probs
+
+
+def softmax_fp32(x, mask, scale):
+    """The fp32 probabilities of the unfused path *before* the final cast: the value
+    the |err| <= 2e-3 (bf16) / 1e-3 (fp16) bars are measured against."""
+    t = x.float()
+    t = t * scale if scale is not None else t.clone()
+    if mask is not None:
+        t = gpt2_attention_mask_func(t, mask)
+    return torch.softmax(t, dim=-1)
+
+
+def softmax_backward_fp32(grad_out, probs, scale):
+    """d/dx of softmax(scale*x): ``scale * y * (g - sum_j g_j y_j)`` in fp32.
+    This is what the reference's fused backward evaluates
+    (megatron/fused_kernels/scaled_masked_softmax.h:240-335) and what autograd
+    gives for the unfused path wherever y > 0."""
+    g = grad_out.float()
+    y = probs.float()
+    dot = (g * y).sum(dim=-1, keepdim=True)
+    s = 1.0 if scale is None else scale
+    return s * (y * (g - dot))
+
+
+def softmax_autograd_fp32(x, mask, scale, grad_out):
+    """Forward + autograd backward of the unfused path in fp32; returns (probs, dx)."""
+    xf = x.detach().float().requires_grad_(True)
+    t = xf * scale if scale is not None else xf * 1.0
+    if mask is not None:
+        t = gpt2_attention_mask_func(t, mask)
+    y = torch.softmax(t, dim=-1)
+    y.backward(grad_out.float())
+    return y.detach(), xf.grad
+
+
+# --- rotary ------------------------------------------------------------------------
+
+
+def rotary_tables(dim, seq_len, base=10000, precision=torch.float):
+    """cos/sin ``[seq, 1, 1, dim]``: angle(t, j) = t * base^(-2 (j mod dim/2) / dim),
+    evaluated in fp32, then cast.  Follows RotaryEmbedding._prepare_cache,
+    megatron/model/positional_embeddings.py:60-80."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2).float() / dim))
+    t = torch.arange(seq_len).type_as(inv_freq)
+    freqs = torch.einsum("i,j->ij", t, inv_freq)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    cos = emb.cos()[:, None, None, :]
+    sin = emb.sin()[:, None, None, :]
+    return cos.to(precision), sin.to(precision)
+
+
+def rotate_half(x):
+    """Follows megatron/model/positional_embeddings.py:103-107."""
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2 :]
+    return torch.cat((-x2, x1), dim=x1.ndim - 1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, offset=0):
+    """Follows apply_rotary_pos_emb_torch, megatron/model/positional_embeddings.py:119-126."""
+    cos = cos[offset : q.shape[0] + offset, ...]
+    sin = sin[offset : q.shape[0] + offset, ...]
+    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+def rotary_fp32(q, k, cos, sin, offset=0):
+    """The unfused expression evaluated in fp32 from the stored q/k values."""
+    return apply_rotary_pos_emb(q.float(), k.float(), cos.float(), sin.float(), offset)
+
+
+def rotary_autograd_fp32(q, k, cos, sin, grad_q, grad_k, offset=0):
+    """Autograd gradients of the unfused expression in fp32; returns (dq, dk)."""
+    qf = q.detach().float().requires_grad_(True)
+    kf = k.detach().float().requires_grad_(True)
+    oq, ok = apply_rotary_pos_emb(qf, kf, cos.float(), sin.float(), offset)
+    torch.autograd.backward([oq, ok], [grad_q.float(), grad_k.float()])
+    return qf.grad, kf.grad
+
+
+def partial_rotary(q, k, cos, sin, rotary_ndims, offset=0):
+    """Slice the first ``rotary_ndims`` dims, rotate, concatenate the rest back.
+    Follows megatron/model/transformer.py:823-860."""
+    q_rot, q_pass = q[..., :rotary_ndims], q[..., rotary_ndims:]
+    k_rot, k_pass = k[..., :rotary_ndims], k[..., rotary_ndims:]
+    q_rot, k_rot = apply_rotary_pos_emb(q_rot, k_rot, cos, sin, offset)
+    return torch.cat((q_rot, q_pass), dim=-1), torch.cat((k_rot, k_pass), dim=-1)
