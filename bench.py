@@ -1,0 +1,348 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused softmax / rotary hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table]
+
+A step is one pass of the hot path over one batch of synthetic input with all
+tensors resident in HBM: the padding-masked scaled softmax forward + backward of
+BASELINE.json's configs[1] ([8, 16, 1024, 1024] fp16, bool mask [8, 1, 1024, 1024],
+scale 0.125, key lengths ~ U[256, 1024]).  K steps are timed after W warm-up
+steps between device synchronisations; the JSON line carries
+
+* value       -- algorithmic GB/s of the step (forward + backward bytes / step time);
+* roofline    -- the dominant kernel (the backward) alone: algorithmic bytes per
+                 launch / mean launch duration from HIP events recorded on the launch
+                 stream inside the timed region, against the 8 TB/s HBM peak;
+* cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
+                 this host's cores on a slice of the same batch;
+* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak.
+
+Buffers rotate over several distinct sets so that no launch finds its input in
+the 256 MB Infinity Cache left there by the previous one.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+METRIC = "softmax/rotary fwd+bwd achieved GB/s and % of MI355X HBM peak; µs per call"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
+    ap.add_argument("--only", type=str, default=None,
+                    help="run only the table rows whose name contains this text (profiling aid)")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is measured on ONE GPU; every row and every rotary vector is "
+              "independent, more GPUs only see a smaller batch (no collective). Use --gpus 1.",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from gpt_neox_amd import _lib
+    from oracle import torch_ref as R
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.lib()  # ImportError if the HIP library is not built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    F16, BF16, F32 = _lib.NEOX_F16, _lib.NEOX_BF16, _lib.NEOX_F32
+    code = {torch.float16: F16, torch.bfloat16: BF16}
+
+    def gen(seed):
+        return torch.Generator(device=dev).manual_seed(seed)
+
+    def ok(status):
+        if status != 0:
+            _lib.check(status)
+
+    # ------------------------------------------------------------------ workloads
+    def masked_sets(b, heads, sq, sk, dtype, seed, nsets):
+        sets = []
+        for i in range(nsets):
+            g0 = gen(seed + i)
+            x = (torch.randn(b, heads, sq, sk, device=dev, generator=g0) * 8).to(dtype)
+            lens = torch.randint(256, sk + 1, (b,), device=dev, generator=g0)
+            mask = R.padding_mask(lens, sq, sk, dev)
+            dy = torch.randn(b, heads, sq, sk, device=dev, generator=g0).to(dtype)
+            sets.append(dict(x=x, mask=mask, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x)))
+        return sets
+
+    def masked_fwd(s, b, heads, sq, sk, dtype, scale):
+        ok(lib.neox_masked_softmax_fwd(s["y"].data_ptr(), s["x"].data_ptr(), s["mask"].data_ptr(),
+                                       scale, b, heads, sq, sk, b, code[dtype], stream))
+
+    def masked_bwd(s, b, heads, sq, sk, dtype, scale):
+        ok(lib.neox_masked_softmax_bwd(s["dx"].data_ptr(), s["dy"].data_ptr(), s["y"].data_ptr(),
+                                       scale, b * heads * sq, sk, code[dtype], stream))
+
+    def causal_sets(batches, s, dtype, seed, nsets, need_bwd):
+        sets = []
+        for i in range(nsets):
+            g0 = gen(seed + i)
+            x = torch.empty(batches, s, s, device=dev, dtype=dtype)
+            for j in range(0, batches, 8):  # chunked: no full-size fp32 temporary
+                x[j : j + 8] = (torch.randn(x[j : j + 8].shape, device=dev, generator=g0) * 8).to(dtype)
+            d = dict(x=x, y=torch.empty_like(x))
+            if need_bwd:
+                dy = torch.empty_like(x)
+                for j in range(0, batches, 8):
+                    dy[j : j + 8] = torch.randn(dy[j : j + 8].shape, device=dev, generator=g0).to(dtype)
+                d.update(dy=dy, dx=torch.empty_like(x))
+            sets.append(d)
+        return sets
+
+    def causal_fwd(s, batches, n, dtype, scale):
+        ok(lib.neox_causal_softmax_fwd(s["y"].data_ptr(), s["x"].data_ptr(), scale, batches, n, n,
+                                       code[dtype], stream))
+
+    def causal_bwd(s, batches, n, dtype, scale):
+        ok(lib.neox_causal_softmax_bwd(s["dx"].data_ptr(), s["dy"].data_ptr(), s["y"].data_ptr(),
+                                       scale, batches, n, n, code[dtype], stream))
+
+    def rope_sets(s, b, h, hn, d_rot, dtype, seed, nsets):
+        cos, sin = R.rotary_tables(d_rot, s, 10000, torch.float)
+        cos, sin = cos.to(dev).reshape(s, d_rot), sin.to(dev).reshape(s, d_rot)
+        sets = []
+        for i in range(nsets):
+            g0 = gen(seed + i)
+            q = torch.randn(s, b, h, hn, device=dev, generator=g0).to(dtype)
+            k = torch.randn(s, b, h, hn, device=dev, generator=g0).to(dtype)
+            sets.append(dict(q=q, k=k, cos=cos, sin=sin, st=_lib.strides3(q)))
+        return sets
+
+    def rope_apply(t, s, b, h, d_rot, dtype, backward):
+        # in place over the first d_rot dims of whole heads, q and k in one launch
+        ok(lib.neox_rope_apply(t["q"].data_ptr(), t["k"].data_ptr(), t["q"].data_ptr(),
+                               t["k"].data_ptr(), t["cos"].data_ptr(), t["sin"].data_ptr(), s, b, h,
+                               h, d_rot, t["st"], t["st"], t["st"], t["st"], d_rot, 0, code[dtype],
+                               F32, backward, stream))
+
+    def time_launches(fn, sets, n_launch, repeats=5, warm=20):
+        """Mean duration (us) of back-to-back launches between two HIP events on the launch
+        stream; median over `repeats` such measurements."""
+        ns = len(sets)
+        for i in range(warm):
+            fn(sets[i % ns])
+        torch.cuda.synchronize()
+        means = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(n_launch):
+                fn(sets[i % ns])
+            e1.record()
+            torch.cuda.synchronize()
+            means.append(e0.elapsed_time(e1) * 1e3 / n_launch)
+        return statistics.median(means), min(means)
+
+    def row(name, nbytes, med_us, min_us):
+        gbps = nbytes / med_us / 1e3
+        return dict(op=name, bytes=nbytes, us_per_call=round(med_us, 2), best_us=round(min_us, 2),
+                    GBps=round(gbps, 1), pct_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 1))
+
+    # ------------------------------------------------------------------ main workload (configs[1])
+    b, heads, sq, sk, dtype, scale = 8, 16, 1024, 1024, torch.float16, 0.125
+    n_elem = b * heads * sq * sk
+    fwd_bytes = 2 * n_elem * 2 + b * sq * sk
+    bwd_bytes = 3 * n_elem * 2
+    sets = masked_sets(b, heads, sq, sk, dtype, 1234 + 1, nsets=3)
+
+    def step(s):
+        masked_fwd(s, b, heads, sq, sk, dtype, scale)
+        masked_bwd(s, b, heads, sq, sk, dtype, scale)
+
+    for i in range(args.warmup):
+        step(sets[i % len(sets)])
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        s = sets[i % len(sets)]
+        ev[i][0].record()
+        masked_fwd(s, b, heads, sq, sk, dtype, scale)
+        ev[i][1].record()
+        masked_bwd(s, b, heads, sq, sk, dtype, scale)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    fwd_us = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e3
+    bwd_us = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e3
+    value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+    bwd_gbps = bwd_bytes / bwd_us / 1e3
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: padding-masked scaled softmax fwd+bwd, scores [8,16,1024,1024] "
+                        "fp16 storage, bool mask [8,1,1024,1024], scale 0.125, lens~U[256,1024]",
+            "step": "1 forward launch + 1 backward launch",
+            "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes,
+            "buffer_sets": len(sets),
+        },
+        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1),
+        "us_per_call": {"fwd": round(fwd_us, 2), "bwd": round(bwd_us, 2)},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "softmax_bwd_kernel<F16, NCH=2, WPR=1, RPB=4, Mask::None>",
+            "achieved": round(bwd_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": bwd_bytes,
+            "avg_launch_us": round(bwd_us, 2),
+        },
+    }
+    del sets, ev
+    torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ CPU baseline
+    if not args.no_cpu:
+        cores = torch.get_num_threads()
+        sample_b = 2
+        g0 = torch.Generator().manual_seed(99)
+        xs = (torch.randn(sample_b, heads, sq, sk, generator=g0) * 8).half()
+        dys = torch.randn(sample_b, heads, sq, sk, generator=g0).half()
+        lens = torch.randint(256, sk + 1, (sample_b,), generator=g0)
+        ms = R.padding_mask(lens, sq, sk)
+
+        def cpu_step():
+            xin = xs.clone().requires_grad_(True)
+            y = R.forward_torch_softmax(xin, ms, scale, input_in_fp16=True, softmax_in_fp32=True)
+            y.backward(dys)
+            return xin.grad
+
+        cpu_step()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 50):
+            cpu_step()
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        sample_bytes = (fwd_bytes + bwd_bytes) * sample_b // b
+        result["cpu_baseline"] = {
+            "value": round(sample_bytes / cpu_s / 1e9, 3),
+            "unit": "GB/s",
+            "cores": cores,
+            "kind": "port",
+            "sample": f"{sample_b} of the {b} batch entries of configs[1] ([{sample_b},16,1024,1024] "
+                      f"fp16), forward + autograd backward of the oracle's torch path, {reps} "
+                      f"repetitions, {cpu_s * 1e3:.1f} ms each",
+            "ms_per_step_scaled_to_full_batch": round(cpu_s * 1e3 * b / sample_b, 1),
+        }
+        del xs, dys, ms
+
+    # ------------------------------------------------------------------ every BASELINE shape
+    if not args.no_table:
+        table = []
+
+        def want(name):
+            return args.only is None or args.only in name
+
+        def tri(n):
+            return n * (n + 1) // 2
+
+        # configs[0]: causal fwd, 125M shape
+        if want("cfg1"):
+            B, n, dt, sc = 48, 2048, torch.bfloat16, 0.125
+            s_ = causal_sets(B, n, dt, 1234, nsets=2, need_bwd=False)
+            table.append(row("cfg1 causal fwd [48,2048,2048] bf16", B * 2 * (tri(n) + n * n),
+                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100)))
+            del s_
+        # configs[1]
+        if want("cfg2"):
+            s_ = masked_sets(b, heads, sq, sk, dtype, 1235, nsets=3)
+            table.append(row("cfg2 padded fwd [8,16,1024,1024] fp16", fwd_bytes,
+                             *time_launches(lambda t: masked_fwd(t, b, heads, sq, sk, dtype, scale), s_, 100)))
+            table.append(row("cfg2 padded bwd [8,16,1024,1024] fp16", bwd_bytes,
+                             *time_launches(lambda t: masked_bwd(t, b, heads, sq, sk, dtype, scale), s_, 100)))
+            del s_
+        # configs[2]: partial rotary
+        if want("cfg3"):
+            S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1236, nsets=10)
+            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+            table.append(row("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
+                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200)))
+            table.append(row("cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
+                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200)))
+            del s_
+        # configs[3]: 20B shape
+        if want("cfg4"):
+            B, n, dt, sc = 64, 2048, torch.float16, 96 ** -0.5
+            s_ = causal_sets(B, n, dt, 1237, nsets=2, need_bwd=True)
+            table.append(row("cfg4 causal fwd [64,2048,2048] fp16", B * 2 * (tri(n) + n * n),
+                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100)))
+            table.append(row("cfg4 causal bwd [64,2048,2048] fp16", B * 2 * (2 * tri(n) + n * n),
+                             *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 100)))
+            del s_
+        # configs[4]: long context
+        if want("cfg5"):
+            torch.cuda.empty_cache()
+            B, n, dt, sc = 32, 8192, torch.bfloat16, 128 ** -0.5
+            s_ = causal_sets(B, n, dt, 1238, nsets=1, need_bwd=True)
+            table.append(row("cfg5 causal fwd [32,8192,8192] bf16", B * 2 * (tri(n) + n * n),
+                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 30, warm=5)))
+            table.append(row("cfg5 causal bwd [32,8192,8192] bf16", B * 2 * (2 * tri(n) + n * n),
+                             *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 30, warm=5)))
+            del s_
+            torch.cuda.empty_cache()
+            S, Bb, H, HN, DR = 8192, 1, 32, 128, 128
+            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1239, nsets=6)
+            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+            table.append(row("cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
+                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200)))
+            table.append(row("cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
+                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200)))
+            del s_
+        # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
+        if want("copy"):
+            nbytes = 1 << 30
+            src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+            dst = torch.empty_like(src)
+            table.append(row("copy 1 GiB (read + write)", 2 * nbytes,
+                             *time_launches(lambda t: ok(lib.neox_copy_bytes(dst.data_ptr(), src.data_ptr(),
+                                                                            nbytes, stream)), [None], 50)))
+        result["all_configs"] = table
+        pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
+        if pcts:
+            result["min_pct_hbm_peak_over_configs"] = min(pcts)
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

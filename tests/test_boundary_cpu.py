@@ -1,0 +1,259 @@
+"""The C-ABI boundary and the Python drop-in surface, checked without a GPU.
+
+Covers: the shared library loads and exports every symbol that
+include/neox_fused.h declares; argument errors come back as status codes before
+any HIP call; the dispatcher predicate; the error behaviour of the
+extension-level modules; the names and signatures the reference's callers import.
+"""
+import ctypes
+import inspect
+import os
+import re
+import sys
+
+import pytest
+import torch
+
+import gpt_neox_amd
+from gpt_neox_amd import _lib, fused_softmax, positional_embeddings
+from gpt_neox_amd.fused_kernels import (
+    fused_rotary_positional_embedding,
+    load_fused_kernels,
+    scaled_masked_softmax_cuda,
+    scaled_upper_triang_masked_softmax_cuda,
+)
+from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "neox_fused.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = re.findall(r"\b(?:int|const char\*)\s+(neox_\w+)\s*\(([^)]*)\)\s*;", text)
+    out = {}
+    for name, args in decls:
+        args = args.strip()
+        out[name] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def test_header_declares_the_expected_entry_points():
+    names = set(declared_functions())
+    assert {
+        "neox_causal_softmax_fwd", "neox_causal_softmax_bwd", "neox_masked_softmax_fwd",
+        "neox_masked_softmax_bwd", "neox_rope_apply", "neox_get_batch_per_block",
+        "neox_fused_abi_version", "neox_fused_strerror", "neox_fused_last_error",
+    } <= names
+
+
+def test_library_exports_every_declared_symbol_with_matching_arity():
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name, nargs in declared_functions().items():
+        assert hasattr(handle, name), f"{name} declared in the header but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+        assert len(_lib.SIGNATURES[name][1]) == nargs, name
+    assert set(_lib.SIGNATURES) == set(declared_functions())
+
+
+def test_abi_version_and_error_strings():
+    lib = _lib.lib()
+    assert lib.neox_fused_abi_version() == _lib.ABI_VERSION
+    for code in range(0, -7, -1):
+        assert lib.neox_fused_strerror(code)
+    assert lib.neox_fused_strerror(-99) == b"unknown status"
+
+
+def test_argument_errors_are_reported_without_touching_the_gpu():
+    lib = _lib.lib()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p = (p + 255) & ~255  # aligned fake "device" pointer: never dereferenced on these paths
+    F16, BF16, F32 = _lib.NEOX_F16, _lib.NEOX_BF16, _lib.NEOX_F32
+    assert lib.neox_causal_softmax_fwd(None, p, 1.0, 1, 8, 8, F16, None) == -1
+    assert b"null" in lib.neox_fused_last_error()
+    assert lib.neox_causal_softmax_fwd(p, p, 1.0, 1, 8, 8, F32, None) == -2
+    assert b"Only fp16 and bf16 are supported" in lib.neox_fused_last_error()
+    assert lib.neox_causal_softmax_fwd(p, p, 1.0, 0, 8, 8, F16, None) == -3
+    assert lib.neox_causal_softmax_fwd(p, p, 1.0, 1, 0, 8, F16, None) == -3
+    assert lib.neox_causal_softmax_fwd(p, p, 1.0, 1 << 40, 8, 8, F16, None) == -3
+    assert lib.neox_causal_softmax_fwd(p + 1, p, 1.0, 1, 8, 8, F16, None) == -5
+    assert lib.neox_causal_softmax_bwd(p, None, p, 1.0, 1, 8, 8, BF16, None) == -1
+    assert lib.neox_causal_softmax_bwd(p, p, p, 1.0, 1, 8, -1, BF16, None) == -3
+    assert lib.neox_masked_softmax_fwd(p, p, None, 1.0, 2, 2, 8, 8, 2, F16, None) == -1
+    assert lib.neox_masked_softmax_fwd(p, p, p, 1.0, 4, 2, 8, 8, 3, F16, None) == -3
+    assert b"mask batch dim" in lib.neox_fused_last_error()
+    assert lib.neox_masked_softmax_bwd(p, p, p, 1.0, 0, 8, F16, None) == -3
+    assert lib.neox_masked_softmax_bwd(p, p, p, 1.0, 8, 8, 7, None) == -2
+    st = (ctypes.c_int64 * 3)(64, 32, 8)
+    neg = (ctypes.c_int64 * 3)(64, -32, 8)
+    rope = lib.neox_rope_apply
+    assert rope(p, None, p, None, None, p, 4, 1, 2, 0, 8, st, None, st, None, 8, 0, F16, F32, 0, None) == -1
+    assert rope(p, p, p, None, p, p, 4, 1, 2, 2, 8, st, st, st, st, 8, 0, F16, F32, 0, None) == -1
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 7, st, None, st, None, 8, 0, F16, F32, 0, None) == -3
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, neg, None, st, None, 8, 0, F16, F32, 0, None) == -4
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 4, 0, F16, F32, 0, None) == -4
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 8, 0, F16, BF16, 0, None) == -2
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 8, -1, F16, F32, 0, None) == -3
+    assert lib.neox_copy_bytes(p, p, 24, None) == -3
+    assert lib.neox_copy_bytes(None, p, 32, None) == -1
+
+
+def test_get_batch_per_block_matches_the_reference_formula_on_wave64():
+    # megatron/fused_kernels/scaled_masked_softmax.h:338-352 with a 64-wide wavefront:
+    # wave = min(pow2(sk), 64); rows/wave = 2 if pow2(sk) <= 128 else 1; waves/block = 128/wave
+    table = {1: 256, 2: 128, 4: 64, 8: 32, 16: 16, 17: 8, 32: 8, 33: 4, 64: 4, 65: 4, 128: 4,
+             129: 2, 256: 2, 1000: 2, 1024: 2, 2048: 2, 8192: 2}
+    for sk, want in table.items():
+        assert FusedScaleMaskSoftmax.get_batch_per_block(1024, sk, 2, 4) == want, sk
+        assert scaled_masked_softmax_cuda.get_batch_per_block(8, sk, 1, 1) == want
+
+
+def test_missing_library_raises_import_error(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libneox_fused.so")
+    with pytest.raises(ImportError, match="not built"):
+        _lib.lib()
+    with pytest.raises(ImportError):
+        FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.general, None, True, None)
+    # no fusion requested: the library is not needed
+    FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None)
+
+
+def test_fused_calls_refuse_cpu_tensors_loudly():
+    x = torch.zeros(2, 8, 8, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused_softmax.ScaledUpperTriangMaskedSoftmax.apply(x, 1.0)
+    x4 = torch.zeros(1, 2, 8, 8, dtype=torch.bfloat16)
+    m = torch.zeros(1, 1, 8, 8, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused_softmax.ScaledMaskedSoftmax.apply(x4, m, 1.0)
+    mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, None, True, None)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mod(x4, m)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        fused_rotary_positional_embedding.forward_cached(
+            torch.zeros(4, 1, 2, 8, dtype=torch.float16), torch.zeros(4, 1, 1, 8), torch.zeros(4, 1, 1, 8)
+        )
+
+
+def test_extension_level_checks_mirror_the_reference_messages():
+    causal, masked = scaled_upper_triang_masked_softmax_cuda, scaled_masked_softmax_cuda
+    with pytest.raises(RuntimeError, match="expected 3D tensor"):
+        causal.forward(torch.zeros(1, 2, 8, 8, dtype=torch.float16), 1.0)
+    with pytest.raises(RuntimeError, match="Only fp16 and bf16 are supported"):
+        causal.forward(torch.zeros(2, 8, 8), 1.0)
+    with pytest.raises(RuntimeError, match="expected 3D tensor"):
+        causal.backward(torch.zeros(8, 8, dtype=torch.float16), torch.zeros(8, 8, dtype=torch.float16), 1.0)
+    with pytest.raises(RuntimeError, match="expected 4D tensor"):
+        masked.forward(torch.zeros(2, 8, 8, dtype=torch.float16), torch.zeros(1, 1, 8, 8, dtype=torch.bool), 1.0)
+    with pytest.raises(RuntimeError, match="Only fp16 and bf16 are supported"):
+        masked.forward(torch.zeros(1, 2, 8, 8), torch.zeros(1, 1, 8, 8, dtype=torch.bool), 1.0)
+    with pytest.raises(RuntimeError, match="expected 4D tensor"):
+        masked.forward(torch.zeros(1, 2, 8, 8, dtype=torch.float16), torch.zeros(8, 8, dtype=torch.bool), 1.0)
+    with pytest.raises(RuntimeError, match="mask"):
+        masked.forward(torch.zeros(4, 2, 8, 8, dtype=torch.float16), torch.zeros(3, 1, 8, 8, dtype=torch.bool), 1.0)
+    rope = fused_rotary_positional_embedding
+    t = torch.zeros(4, 1, 2, 8, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="same sequence length"):
+        rope.forward_cached(t, torch.zeros(5, 1, 1, 8), torch.zeros(5, 1, 1, 8))
+    with pytest.raises(RuntimeError, match="second and third dims"):
+        rope.forward_cached(t, torch.zeros(4, 2, 1, 8), torch.zeros(4, 2, 1, 8))
+    with pytest.raises(RuntimeError, match="greater than"):
+        rope.forward_cached(t, torch.zeros(4, 1, 1, 16), torch.zeros(4, 1, 1, 16))
+    with pytest.raises(RuntimeError, match="same dtype"):
+        rope.forward_cached(t, torch.zeros(4, 1, 1, 8), torch.zeros(4, 1, 1, 8, dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="must be float"):
+        rope.forward(t, torch.zeros(4, 1, 1, 8, dtype=torch.float16))
+
+
+def test_load_fused_kernels_registers_the_reference_module_names():
+    mods = load_fused_kernels()
+    for name in ("scaled_upper_triang_masked_softmax_cuda", "scaled_masked_softmax_cuda",
+                 "fused_rotary_positional_embedding"):
+        assert name in sys.modules
+    import scaled_masked_softmax_cuda as top  # the import statement the reference uses
+
+    assert top is mods[1] and callable(top.forward) and callable(top.backward)
+    assert callable(top.get_batch_per_block)
+
+
+# ---- dispatcher ---------------------------------------------------------------------
+
+
+def make(fusion, fp16=True, bf16=False, scale=None):
+    return FusedScaleMaskSoftmax(fp16, bf16, fusion, lambda s, m: s, True, scale)
+
+
+def test_is_kernel_available_table():
+    mask = torch.zeros(1, 1, 4, 4, dtype=torch.bool)
+    causal, general, none = (make(t) for t in (SoftmaxFusionTypes.upper_triang,
+                                                SoftmaxFusionTypes.general, SoftmaxFusionTypes.none))
+    # every BASELINE shape takes the fused branch, including the 8192 one
+    for b, np_, sq, sk in [(4, 12, 2048, 2048), (1, 64, 2048, 2048), (1, 32, 8192, 8192), (3, 5, 7, 7)]:
+        assert causal.is_kernel_available(mask, b, np_, sq, sk)
+    assert general.is_kernel_available(mask, 8, 16, 1024, 1024)
+    assert general.is_kernel_available(mask, 1, 3, 1, 77)  # decode step, odd sizes
+    assert not causal.is_kernel_available(mask, 1, 4, 1, 77)  # causal kernel needs sq == sk
+    assert not causal.is_kernel_available(None, 4, 12, 64, 64)  # no mask tensor
+    assert not general.is_kernel_available(None, 4, 12, 64, 64)
+    assert not none.is_kernel_available(mask, 4, 12, 64, 64)  # fusion not requested
+    fp32 = FusedScaleMaskSoftmax(False, False, SoftmaxFusionTypes.general, None, True, None)
+    assert not fp32.is_kernel_available(mask, 4, 12, 64, 64)  # fp32 input
+    assert not general.is_kernel_available(mask, 0, 12, 64, 64)  # empty
+
+
+def test_reference_predicate_restated():
+    # megatron/model/fused_softmax.py:148-168 with wave64 batch_per_block (= 2 for sk > 128)
+    ref = FusedScaleMaskSoftmax.reference_is_kernel_available
+    m = object()
+    assert ref(True, True, True, m, 4, 12, 2048, 2048)
+    assert not ref(True, True, True, m, 1, 32, 8192, 8192)  # the 2048 cap
+    assert not ref(True, True, True, m, 4, 12, 16, 16)  # sk must exceed 16
+    assert not ref(True, True, True, m, 4, 12, 2046, 2046)  # sq % 4
+    assert not ref(True, True, True, m, 1, 3, 64, 64)  # (b*np) % 4
+    assert not ref(True, True, True, None, 4, 12, 64, 64)
+    assert not ref(False, True, True, m, 4, 12, 64, 64)
+    assert not ref(True, True, False, m, 4, 12, 64, 64)
+    assert ref(True, False, True, m, 8, 16, 1024, 1024)
+    assert ref(True, False, True, m, 1, 4, 4, 32) is False  # sq=4, batch_per_block=8 at sk=32
+
+
+def test_constructor_contract():
+    with pytest.raises(AssertionError, match="Invalid fusion type"):
+        FusedScaleMaskSoftmax(True, False, "general", None, True, None)
+    with pytest.raises(AssertionError, match="softmax should be in fp32 when scaled"):
+        FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, False, 2.0)
+    m = make(SoftmaxFusionTypes.upper_triang, fp16=False, bf16=True, scale=3.0)
+    assert m.input_in_float16 and m.upper_triang_mask_fusion and not m.general_mask_fusion
+    assert m.fusion and m.scale == 3.0
+    with pytest.raises(AssertionError):
+        m(torch.zeros(2, 8, 8), None)  # input must be 4-D
+
+
+def test_public_names_and_signatures_match_the_reference_modules():
+    def params(fn):
+        return list(inspect.signature(fn).parameters)
+
+    assert params(FusedScaleMaskSoftmax.__init__) == [
+        "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale"]
+    assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask"]
+    assert params(FusedScaleMaskSoftmax.is_kernel_available) == ["self", "mask", "b", "np", "sq", "sk"]
+    assert params(FusedScaleMaskSoftmax.get_batch_per_block) == ["sq", "sk", "b", "np"]
+    assert params(fused_softmax.ScaledUpperTriangMaskedSoftmax.forward) == ["ctx", "inputs", "scale"]
+    assert params(fused_softmax.ScaledMaskedSoftmax.forward) == ["ctx", "inputs", "mask", "scale"]
+    assert [e.name for e in SoftmaxFusionTypes] == ["upper_triang", "general", "none"]
+    assert [e.value for e in SoftmaxFusionTypes] == [1, 2, 3]
+    pe = positional_embeddings
+    assert params(pe.RotaryEmbedding.__init__) == [
+        "self", "dim", "max_seq_len", "base", "precision", "save_inv_freqs"]
+    assert params(pe.RotaryEmbedding.forward) == ["self", "x", "seq_dim", "seq_len"]
+    assert params(pe.apply_rotary_pos_emb) == ["q", "k", "cos", "sin", "offset"]
+    assert params(pe.apply_rotary_pos_emb_torch) == ["q", "k", "cos", "sin", "offset"]
+    assert params(pe.rotate_half) == ["x"]
+    assert params(pe.SinusoidalPositionalEmbedding.__init__) == ["self", "dim", "base", "precision"]
+    assert params(pe.AliBi.__init__) == ["self", "num_heads", "mp_size", "mp_rank"]
+    for name in ("FusedScaleMaskSoftmax", "RotaryEmbedding", "apply_rotary_pos_emb_torch",
+                 "apply_rotary_pos_emb", "AliBi", "SoftmaxFusionTypes", "SinusoidalPositionalEmbedding"):
+        assert hasattr(gpt_neox_amd, name)

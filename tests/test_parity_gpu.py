@@ -1,0 +1,496 @@
+"""Parity of the gfx950 kernels (called through the C-ABI) with the oracle.
+
+Bars (BASELINE.json north_star): softmax |err| <= 2e-3 (bf16) / 1e-3 (fp16)
+against the fp32 computation of the reference's unfused path, masked positions
+exactly 0; rotary is bit-equal to the fp32 expression rounded once to the storage
+type.  The backward pass is compared with the fp32 closed form evaluated on the
+same saved (rounded) probabilities, which is what the reference's fused backward
+consumes, at the same bars.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpt_neox_amd import _lib
+from gpt_neox_amd.fused_kernels import (
+    fused_rotary_positional_embedding as rope_ext,
+    scaled_masked_softmax_cuda as masked_ext,
+    scaled_upper_triang_masked_softmax_cuda as causal_ext,
+)
+from gpt_neox_amd.fused_softmax import (
+    FusedScaleMaskSoftmax,
+    ScaledMaskedSoftmax,
+    ScaledUpperTriangMaskedSoftmax,
+    SoftmaxFusionTypes,
+)
+from gpt_neox_amd.positional_embeddings import (
+    RotaryEmbedding,
+    apply_rotary_pos_emb,
+    apply_rotary_pos_emb_,
+    apply_rotary_pos_emb_torch,
+)
+from oracle import torch_ref as R
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-3, torch.float16: 1e-3}
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+def gen(device, seed):
+    return torch.Generator(device=device).manual_seed(seed)
+
+
+def scores(shape, dtype, device, seed):
+    return (torch.randn(shape, device=device, generator=gen(device, seed)) * 8).to(dtype)
+
+
+def normal(shape, dtype, device, seed):
+    return torch.randn(shape, device=device, generator=gen(device, seed)).to(dtype)
+
+
+def max_err(a, b):
+    return (a.float() - b.float()).abs().max().item()
+
+
+# ---------------------------------------------------------------------------------
+# 16-bit conversions used by every kernel
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rounding_is_nearest_even(device, dtype):
+    # q = 1, sin = 0: the kernel stores round(cos).  cos walks through quarter-ulp steps of
+    # the storage type, so every fourth value is an exact tie (must go to the even neighbour).
+    p = 7 if dtype == torch.bfloat16 else 10  # explicit mantissa bits
+    steps = torch.arange(64, device=device, dtype=torch.float32)
+    cos = (1.0 + steps * 2.0 ** -(p + 2)).view(1, 1, 1, 64).expand(4, 1, 1, 64).contiguous()
+    sin = torch.zeros_like(cos)
+    q = torch.ones(4, 2, 3, 64, dtype=dtype, device=device)
+    oq, ok = apply_rotary_pos_emb(q, q, cos, sin)
+    want = cos.to(dtype).expand_as(q)
+    assert torch.equal(oq, want) and torch.equal(ok, want)
+    # identity table: every stored value survives unchanged
+    x = normal((8, 2, 4, 64), dtype, device, 1)
+    oq, _ = apply_rotary_pos_emb(x, x, torch.ones(8, 1, 1, 64, device=device), torch.zeros(8, 1, 1, 64, device=device))
+    assert torch.equal(oq, x)
+
+
+# ---------------------------------------------------------------------------------
+# golden vectors
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["causal_8", "causal_40"])
+def test_golden_causal(device, golden, name, dtype):
+    f = golden[name]
+    x = torch.tensor(f["x"], device=device).to(dtype)
+    assert torch.equal(x.float().cpu(), torch.tensor(f["x"]))  # inputs are exact in both types
+    y = causal_ext.forward(x, float(f["scale"]))
+    want = torch.tensor(f["y"], device=device)
+    assert max_err(y, want) <= TOL[dtype]
+    assert (y[want == 0] == 0).all()
+    g = torch.tensor(f["g"], device=device).to(dtype)
+    dx = causal_ext.backward(g.clone(), y, float(f["scale"]))
+    ref = R.softmax_backward_fp32(g, y, float(f["scale"]))
+    assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    # against the float64 fixture: adds the effect of the rounded probabilities
+    assert max_err(dx, torch.tensor(f["dx"], device=device)) <= 4 * TOL[dtype] * max(1.0, np.abs(f["dx"]).max())
+    assert (dx[want == 0] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["masked_4x16", "masked_3x37"])
+def test_golden_masked(device, golden, name, dtype):
+    f = golden[name]
+    x = torch.tensor(f["x"], device=device).to(dtype)
+    mask_u8 = torch.tensor(f["mask"], device=device)
+    want = torch.tensor(f["y"], device=device)
+    for mask in (mask_u8, mask_u8.bool(), mask_u8 * 7):  # any non-zero byte masks
+        y = masked_ext.forward(x, mask, float(f["scale"]))
+        assert max_err(y, want) <= TOL[dtype]
+        assert (y[want == 0] == 0).all()
+    g = torch.tensor(f["g"], device=device).to(dtype)
+    dx = masked_ext.backward(g.clone(), y, float(f["scale"]))
+    ref = R.softmax_backward_fp32(g, y, float(f["scale"]))
+    assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    assert (dx[want == 0] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["rotary_d8", "rotary_d32", "rotary_d24"])
+def test_golden_rotary(device, golden, name, dtype):
+    f = golden[name]
+    s, _, _, d = f["q"].shape
+    off = int(f["offset"])
+    cos, sin = (t.to(device) for t in R.rotary_tables(d, s + off, float(f["base"])))
+    q = torch.tensor(f["q"], device=device).to(dtype).requires_grad_(True)
+    k = torch.tensor(f["k"], device=device).to(dtype).requires_grad_(True)
+    oq, ok = apply_rotary_pos_emb(q, k, cos, sin, off)
+    ulp = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    for got, key in ((oq, "oq"), (ok, "ok")):
+        want = torch.tensor(f[key], device=device)
+        assert ((got.double() - want).abs() <= ulp * want.abs().clamp(min=1.0) + 1e-4).all(), key
+    torch.autograd.backward([oq, ok], [torch.tensor(f["gq"], device=device).to(dtype),
+                                       torch.tensor(f["gk"], device=device).to(dtype)])
+    for got, key in ((q.grad, "dq"), (k.grad, "dk")):
+        want = torch.tensor(f[key], device=device)
+        assert ((got.double() - want).abs() <= ulp * want.abs().clamp(min=1.0) + 1e-4).all(), key
+
+
+# ---------------------------------------------------------------------------------
+# causal softmax
+# ---------------------------------------------------------------------------------
+def check_causal(device, batches, s, dtype, scale, seed, chunk=4):
+    x = scores((batches, s, s), dtype, device, seed)
+    g = normal((batches, s, s), dtype, device, seed + 1000)
+    x_copy = x.clone()
+    y = causal_ext.forward(x, scale)
+    assert torch.equal(x, x_copy)  # the input is not modified
+    assert y.dtype == dtype and y.shape == x.shape and y.is_contiguous()
+    dx = causal_ext.backward(g.clone(), y, scale)
+    mask = R.get_attn_mask(s, device)
+    for i in range(0, batches, chunk):
+        ref = R.softmax_fp32(x[i : i + chunk].unsqueeze(0), mask, scale)[0]
+        assert max_err(y[i : i + chunk], ref) <= TOL[dtype], (batches, s, dtype)
+        hidden = mask[0].expand_as(y[i : i + chunk])
+        assert (y[i : i + chunk][hidden] == 0).all()
+        refb = R.softmax_backward_fp32(g[i : i + chunk], y[i : i + chunk], scale)
+        assert max_err(dx[i : i + chunk], refb) <= TOL[dtype] * max(1.0, refb.abs().max().item())
+        assert (dx[i : i + chunk][hidden] == 0).all()
+    return x, y, g, dx
+
+
+# row lengths chosen to hit: 1 column; lanes partly filled; not a multiple of 8 (element-wise
+# kernels); each chunk count 1..4 of the one-wave kernels; the 2-, 4-, 8- and 16-wave kernels
+# with 3 and 4 chunks per wave; a row longer than the register-resident limit.
+CAUSAL_SIZES = [1, 2, 7, 8, 16, 37, 64, 120, 512, 520, 1000, 1024, 1536, 2048, 2056, 3072, 4096,
+                5000, 6144, 8192]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("s", CAUSAL_SIZES)
+def test_causal_sizes(device, s, dtype):
+    batches = 3 if s <= 2056 else 1
+    check_causal(device, batches, s, dtype, 0.125, seed=s)
+
+
+@pytest.mark.parametrize("s", [12288, 16384, 33000])
+def test_causal_very_long_rows(device, s):
+    # 8 and 16 waves per row; 33000 exceeds the register-resident limit (element-wise kernels)
+    x = scores((1, s, s), torch.bfloat16, device, s)
+    y = causal_ext.forward(x, 0.05)
+    rows = torch.tensor([0, 1, 511, 512, 513, s // 2, s - 2, s - 1], device=device)
+    mask = R.get_attn_mask(s, device)[0, 0][rows]
+    ref = R.softmax_fp32(x[0][rows], mask, 0.05)
+    assert max_err(y[0][rows], ref) <= TOL[torch.bfloat16]
+    assert (y[0][rows][mask] == 0).all()
+    assert torch.allclose(y.float().sum(-1), torch.ones(1, s, device=device), atol=3e-2)
+    g = normal((1, s, s), torch.bfloat16, device, 5)
+    dx = causal_ext.backward(g.clone(), y, 0.05)
+    refb = R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)
+    assert max_err(dx[0][rows], refb) <= TOL[torch.bfloat16]
+    assert (dx[0][rows][mask] == 0).all()
+
+
+def test_causal_negative_and_large_scale(device):
+    for scale in (-0.25, 4.0, 1.0):
+        check_causal(device, 2, 96, torch.float16, scale, seed=3)
+
+
+def test_causal_forward_in_place_alias(device):
+    x = scores((2, 520, 520), torch.bfloat16, device, 9)
+    want = causal_ext.forward(x, 0.125)
+    ptr = x.data_ptr()
+    lib = _lib.lib()
+    _lib.check(lib.neox_causal_softmax_fwd(ptr, ptr, 0.125, 2, 520, 520, _lib.NEOX_BF16,
+                                           torch.cuda.current_stream().cuda_stream))
+    assert torch.equal(x, want)
+
+
+def test_causal_backward_overwrites_contiguous_grad_like_the_reference(device):
+    y = causal_ext.forward(scores((2, 64, 64), torch.float16, device, 1), 0.125)
+    g = normal((2, 64, 64), torch.float16, device, 2)
+    keep = g.clone()
+    dx = causal_ext.backward(g, y, 0.125)
+    assert dx.data_ptr() == g.data_ptr()
+    g_t = keep.transpose(1, 2)  # non-contiguous: a copy is made, the argument survives
+    dx2 = causal_ext.backward(g_t, y, 0.125)
+    assert dx2.data_ptr() != g_t.data_ptr() and torch.equal(g_t, keep.transpose(1, 2))
+    assert torch.equal(dx2, causal_ext.backward(g_t.contiguous(), y, 0.125))
+
+
+def test_causal_other_stream(device):
+    x = scores((4, 256, 256), torch.float16, device, 11)
+    want = causal_ext.forward(x, 0.5)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = causal_ext.forward(x, 0.5)
+    side.synchronize()
+    assert torch.equal(got, want)
+
+
+def test_causal_autograd_function_and_module(device):
+    for dtype, fp16, bf16 in ((torch.float16, True, False), (torch.bfloat16, False, True)):
+        b, heads, s = 2, 3, 72
+        x = scores((b, heads, s, s), dtype, device, 21)
+        mask = R.get_attn_mask(s, device)
+        fused = FusedScaleMaskSoftmax(fp16, bf16, SoftmaxFusionTypes.upper_triang,
+                                      R.gpt2_attention_mask_func, True, 0.3)
+        plain = FusedScaleMaskSoftmax(fp16, bf16, SoftmaxFusionTypes.none,
+                                      R.gpt2_attention_mask_func, True, 0.3)
+        xf = x.clone().requires_grad_(True)
+        xp = x.clone().requires_grad_(True)
+        yf, yp = fused(xf, mask), plain(xp, mask)
+        assert yf.shape == (b, heads, s, s) and yf.dtype == dtype
+        assert max_err(yf, yp) <= 2 * TOL[dtype]  # two roundings apart at most
+        g = normal(yf.shape, dtype, device, 22)
+        yf.backward(g.clone())
+        yp.backward(g.clone())
+        # the fused backward consumes the rounded probabilities, autograd the fp32 ones
+        assert max_err(xf.grad, xp.grad) <= 4 * TOL[dtype] * max(1.0, xp.grad.abs().max().item())
+        # scale None means 1.0
+        f1 = FusedScaleMaskSoftmax(fp16, bf16, SoftmaxFusionTypes.upper_triang, None, True, None)
+        assert torch.equal(f1(x, mask), ScaledUpperTriangMaskedSoftmax.apply(x.view(-1, s, s), 1.0).view_as(x))
+
+
+def test_causal_module_ignores_mask_contents_like_the_reference(device):
+    # megatron/model/fused_softmax.py:173-179: the causal branch never reads the mask
+    x = scores((1, 2, 40, 40), torch.float16, device, 4)
+    fused = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang, None, True, None)
+    a = fused(x, R.get_attn_mask(40, device))
+    b = fused(x, R.get_attn_mask(40, device, sliding_window_width=3))
+    assert torch.equal(a, b)
+
+
+def test_causal_decode_step_takes_the_torch_branch(device):
+    fused = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang,
+                                  R.gpt2_attention_mask_func, True, None)
+    x = scores((1, 2, 1, 33), torch.float16, device, 4)
+    mask = torch.zeros(1, 1, 1, 33, dtype=torch.bool, device=device)
+    assert torch.equal(fused(x, mask), R.forward_torch_softmax(x, mask, None, True, False, True))
+
+
+# ---------------------------------------------------------------------------------
+# mask-tensor softmax
+# ---------------------------------------------------------------------------------
+def check_masked(device, b, heads, sq, sk, dtype, scale, seed, mask=None, lo=1):
+    x = scores((b, heads, sq, sk), dtype, device, seed)
+    g = normal((b, heads, sq, sk), dtype, device, seed + 1)
+    if mask is None:
+        lens = torch.randint(lo, sk + 1, (b,), device=device, generator=gen(device, seed + 2))
+        mask = R.padding_mask(lens, sq, sk, device)
+    y = masked_ext.forward(x, mask, scale)
+    ref = R.softmax_fp32(x, mask.bool(), scale)
+    assert max_err(y, ref) <= TOL[dtype], (b, heads, sq, sk, dtype)
+    hidden = mask.bool().expand_as(y)
+    full_rows = hidden.all(-1, keepdim=True).expand_as(y)
+    assert (y[hidden & ~full_rows] == 0).all()
+    dx = masked_ext.backward(g.clone(), y, scale)
+    refb = R.softmax_backward_fp32(g, y, scale)
+    assert max_err(dx, refb) <= TOL[dtype] * max(1.0, refb.abs().max().item())
+    assert (dx[hidden & ~full_rows] == 0).all()
+    return x, mask, y, g, dx
+
+
+MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (2, 2, 16, 64), (3, 2, 9, 520),
+                 (2, 2, 33, 1000), (2, 2, 8, 1024), (1, 2, 6, 2048), (1, 1, 4, 3072), (1, 2, 3, 4096),
+                 (1, 1, 3, 8192), (1, 1, 2, 20000), (1, 1, 2, 40000), (1, 3, 1, 77)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", MASKED_SHAPES)
+def test_masked_shapes(device, shape, dtype):
+    check_masked(device, *shape, dtype, 0.125, seed=sum(shape))
+
+
+def test_masked_broadcast_over_batch_and_arbitrary_pattern(device):
+    b, heads, sq, sk = 3, 2, 24, 136
+    pattern = torch.rand(1, 1, sq, sk, device=device, generator=gen(device, 5)) < 0.5
+    pattern[0, 0, 3, :] = True  # fully masked row -> uniform 1/sk
+    pattern[0, 0, 4, :] = False
+    x, mask, y, g, dx = check_masked(device, b, heads, sq, sk, torch.float16, 0.2, 6, mask=pattern)
+    assert torch.allclose(y[:, :, 3, :].float(), torch.full((b, heads, sk), 1.0 / sk, device=device), atol=1e-5)
+    per_sample = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, 7)) < 0.3
+    check_masked(device, b, heads, sq, sk, torch.bfloat16, 0.2, 8, mask=per_sample)
+    check_masked(device, b, heads, sq, sk, torch.bfloat16, 0.2, 8, mask=per_sample.to(torch.uint8) * 255)
+
+
+def test_masked_autograd_function_and_module(device):
+    b, heads, sq, sk = 2, 4, 48, 200
+    dtype = torch.bfloat16
+    x = scores((b, heads, sq, sk), dtype, device, 31)
+    lens = torch.tensor([200, 77], device=device)
+    mask = R.padding_mask(lens, sq, sk, device)
+    fused = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.125)
+    plain = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.125)
+    xf, xp = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    yf, yp = fused(xf, mask), plain(xp, mask)
+    assert max_err(yf, yp) <= 2 * TOL[dtype]
+    g = normal(yf.shape, dtype, device, 32)
+    yf.backward(g.clone())
+    yp.backward(g.clone())
+    assert max_err(xf.grad, xp.grad) <= 4 * TOL[dtype] * max(1.0, xp.grad.abs().max().item())
+    assert torch.equal(ScaledMaskedSoftmax.apply(x, mask, 0.125), yf.detach())
+
+
+def test_masked_non_contiguous_input_is_accepted(device):
+    x = scores((2, 2, 64, 32), torch.float16, device, 1).transpose(2, 3)  # [2,2,32,64] strided
+    mask = torch.zeros(2, 1, 32, 64, dtype=torch.bool, device=device)
+    y = masked_ext.forward(x, mask, 1.0)
+    assert max_err(y, R.softmax_fp32(x, mask, 1.0)) <= TOL[torch.float16]
+
+
+def test_empty_tensors(device):
+    assert causal_ext.forward(torch.empty(0, 8, 8, dtype=torch.float16, device=device), 1.0).shape == (0, 8, 8)
+    m = torch.zeros(1, 1, 4, 8, dtype=torch.bool, device=device)
+    assert masked_ext.forward(torch.empty(0, 2, 4, 8, dtype=torch.float16, device=device), m[:0], 1.0).numel() == 0
+
+
+# ---------------------------------------------------------------------------------
+# rotary
+# ---------------------------------------------------------------------------------
+def check_rotary(device, s, b, hq, hk, hn, d_rot, dtype, seed, offset=0, table_dtype=torch.float,
+                 qkv_view=False):
+    if qkv_view:  # q, k as slices of a fused [s, b, h, 3*hn] projection (hq == hk)
+        qkv = normal((s, b, hq, 3 * hn), dtype, device, seed)
+        q_full, k_full = qkv[..., :hn], qkv[..., hn : 2 * hn]
+    else:
+        q_full = normal((s, b, hq, hn), dtype, device, seed)
+        k_full = normal((s, b, hk, hn), dtype, device, seed + 1)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + offset + 3, 10000, table_dtype))
+    q, k = q_full[..., :d_rot], k_full[..., :d_rot]
+    # leaves that keep the strides of the slices: the kernels see the strided views
+    qr, kr = q.detach().requires_grad_(True), k.detach().requires_grad_(True)
+    oq, ok = apply_rotary_pos_emb(qr, kr, cos, sin, offset)
+    assert oq.dtype == dtype and oq.shape == q.shape and ok.shape == k.shape
+    rq, rk = R.rotary_fp32(q, k, cos, sin, offset)
+    assert torch.equal(oq, rq.to(dtype)) and torch.equal(ok, rk.to(dtype)), "forward not bit-equal"
+    gq = normal(oq.shape, dtype, device, seed + 2)
+    gk = normal(ok.shape, dtype, device, seed + 3)
+    torch.autograd.backward([oq, ok], [gq, gk])
+    dq, dk = R.rotary_autograd_fp32(q, k, cos, sin, gq, gk, offset)
+    assert torch.equal(qr.grad, dq.to(dtype)) and torch.equal(kr.grad, dk.to(dtype)), "backward not bit-equal"
+    # in place over whole heads: rotated span as above, remaining dims untouched
+    q2, k2 = q_full.clone(), k_full.clone()
+    r1, r2 = apply_rotary_pos_emb_(q2, k2, cos, sin, offset, d_rot)
+    assert r1.data_ptr() == q2.data_ptr() and r2.data_ptr() == k2.data_ptr()
+    assert torch.equal(q2[..., :d_rot], oq) and torch.equal(k2[..., :d_rot], ok)
+    assert torch.equal(q2[..., d_rot:], q_full[..., d_rot:]) and torch.equal(k2[..., d_rot:], k_full[..., d_rot:])
+
+
+ROTARY_CASES = [
+    # s, b, hq, hk, hn, d_rot
+    (16, 2, 4, 4, 64, 64), (16, 2, 4, 4, 128, 32), (9, 3, 5, 5, 96, 24), (7, 2, 3, 3, 80, 80),
+    (5, 1, 2, 2, 16, 6), (33, 2, 8, 2, 128, 128), (12, 2, 6, 6, 96, 96), (4, 5, 3, 3, 256, 256),
+    (1, 7, 9, 9, 64, 16), (300, 1, 1, 1, 8, 2), (64, 4, 32, 32, 128, 32), (6, 2, 4, 4, 64, 48),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", ROTARY_CASES)
+def test_rotary_cases(device, case, dtype):
+    check_rotary(device, *case, dtype, seed=sum(case))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rotary_offset_and_qkv_views(device, dtype):
+    check_rotary(device, 20, 2, 4, 4, 64, 16, dtype, seed=1, offset=5)
+    check_rotary(device, 20, 2, 4, 4, 64, 64, dtype, seed=2, offset=0, qkv_view=True)
+    check_rotary(device, 11, 3, 4, 4, 128, 32, dtype, seed=3, offset=2, qkv_view=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rotary_half_precision_tables(device, dtype):
+    # tables in the dtype of q (the model's usual setting): fp32 arithmetic on the table
+    # values as stored, one rounding
+    s, b, h, d = 24, 2, 4, 32
+    q, k = normal((s, b, h, d), dtype, device, 1), normal((s, b, h, d), dtype, device, 2)
+    emb = RotaryEmbedding(d, 64, precision=dtype)
+    cos, sin = emb(q, seq_len=s)
+    assert cos.device == q.device and cos.dtype == dtype
+    oq, ok = apply_rotary_pos_emb_torch(q, k, cos, sin)
+    rq, rk = R.rotary_fp32(q, k, cos, sin)
+    assert torch.equal(oq, rq.to(dtype)) and torch.equal(ok, rk.to(dtype))
+    # and within the bf16/fp16 noise of the all-half-precision torch expression
+    tq, _ = R.apply_rotary_pos_emb(q, k, cos, sin)
+    assert max_err(oq, tq) <= (0.05 if dtype == torch.bfloat16 else 0.01)
+    assert emb(q, seq_len=s)[0].data_ptr() == cos.data_ptr()  # device copy is kept, not re-made
+
+
+def test_rotary_non_collapsible_layout(device):
+    # [s, b, h, d] view of a [b, s, h, d] buffer: stride_b != h * stride_h
+    s, b, h, d = 10, 3, 4, 32
+    base_q = normal((b, s, h, d), torch.bfloat16, device, 1)
+    base_k = normal((b, s, h, d), torch.bfloat16, device, 2)
+    q, k = base_q.transpose(0, 1), base_k.transpose(0, 1)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d, s))
+    oq, ok = apply_rotary_pos_emb(q, k, cos, sin)
+    rq, rk = R.rotary_fp32(q, k, cos, sin)
+    assert torch.equal(oq, rq.bfloat16()) and torch.equal(ok, rk.bfloat16())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("transpose", [False, True])
+def test_fused_rope_extension_api(device, dtype, transpose):
+    s, b, h, d, d2 = 12, 2, 3, 64, 16
+    t = normal((s, b, h, d), dtype, device, 5)
+    cos, sin = (x.to(device) for x in R.rotary_tables(d2, s))
+    out = rope_ext.forward_cached(t, cos, sin, transpose)
+    want, _ = R.partial_rotary(t.float(), t.float(), cos, sin, d2)
+    assert out.shape == (s, b, h, d) and torch.equal(out, want.to(dtype))
+    assert out.transpose(0, 1).is_contiguous() == transpose
+    g = normal((s, b, h, d), dtype, device, 6)
+    gin = rope_ext.backward_cached(g, cos, sin, transpose)
+    dq, _ = R.rotary_autograd_fp32(t[..., :d2], t[..., :d2], cos, sin, g[..., :d2], g[..., :d2])
+    assert torch.equal(gin[..., :d2], dq.to(dtype)) and torch.equal(gin[..., d2:], g[..., d2:])
+    # angles given instead of tables
+    freqs = torch.outer(torch.arange(s, device=device).float(),
+                        1.0 / (10000 ** (torch.arange(0, d2, 2, device=device).float() / d2)))
+    freqs = torch.cat((freqs, freqs), -1)[:, None, None, :]
+    out2 = rope_ext.forward(t, freqs, transpose)
+    w2, _ = R.partial_rotary(t.float(), t.float(), freqs.cos(), freqs.sin(), d2)
+    assert torch.equal(out2, w2.to(dtype))
+
+
+def test_rotary_round_trip_property(device):
+    # backward is the inverse rotation: bwd(fwd(x)) == x up to two roundings
+    s, b, h, d = 128, 2, 8, 64
+    q, k = normal((s, b, h, d), torch.float16, device, 1), normal((s, b, h, d), torch.float16, device, 2)
+    cos, sin = (t.to(device).reshape(s, d) for t in R.rotary_tables(d, s))
+    oq, ok = torch.empty_like(q), torch.empty_like(k)
+    rope_ext.rope_launch(oq, ok, q, k, cos, sin, d, 0, backward=False)
+    bq, bk = torch.empty_like(q), torch.empty_like(k)
+    rope_ext.rope_launch(bq, bk, oq, ok, cos, sin, d, 0, backward=True)
+    assert max_err(bq, q) <= 8e-3 and max_err(bk, k) <= 8e-3
+
+
+# ---------------------------------------------------------------------------------
+# BASELINE.json shapes at full size
+# ---------------------------------------------------------------------------------
+def test_config1_causal_fwd_125m(device):
+    x, y, g, dx = check_causal(device, 48, 2048, torch.bfloat16, 0.125, seed=1234)
+    sums = y.float().sum(-1)
+    assert (sums - 1).abs().max().item() < 2e-2  # bf16-rounded rows still sum to ~1
+
+
+def test_config2_padding_fwd_bwd(device):
+    x, mask, y, g, dx = check_masked(device, 8, 16, 1024, 1024, torch.float16, 0.125, seed=1235, lo=256)
+    assert (y.float().sum(-1) - 1).abs().max().item() < 5e-3
+    assert dx.float().sum(-1).abs().max().item() < 5e-2  # rows of dx sum to 0
+
+
+def test_config3_partial_rotary(device):
+    check_rotary(device, 2048, 4, 32, 32, 128, 32, torch.bfloat16, seed=1236)
+
+
+def test_config4_causal_20b(device):
+    x, y, g, dx = check_causal(device, 64, 2048, torch.float16, 96**-0.5, seed=1237)
+    assert dx.float().sum(-1).abs().max().item() < 5e-2
+
+
+def test_config5_long_context(device):
+    x, y, g, dx = check_causal(device, 32, 8192, torch.bfloat16, 128**-0.5, seed=1238, chunk=2)
+    del x, g, dx
+    assert (y.float().sum(-1) - 1).abs().max().item() < 3e-2
+    del y
+    torch.cuda.empty_cache()
+    check_rotary(device, 8192, 1, 32, 32, 128, 128, torch.bfloat16, seed=1239)
