@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused softmax / rotary hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table] [--quick] [--only TEXT]
 
 A step is one pass of the hot path over one batch of synthetic input with all
 tensors resident in HBM: the padding-masked scaled softmax forward + backward of
@@ -42,6 +42,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
+    ap.add_argument("--quick", action="store_true",
+                    help="few launches per table row (for counter-collection runs)")
     ap.add_argument("--only", type=str, default=None,
                     help="run only the table rows whose name contains this text (profiling aid)")
     return ap.parse_args()
@@ -143,6 +145,8 @@ def main():
         """Mean duration (us) of back-to-back launches between two HIP events on the launch
         stream; median over `repeats` such measurements."""
         ns = len(sets)
+        if args.quick:
+            n_launch, repeats, warm = min(n_launch, 10), 1, 2
         for i in range(warm):
             fn(sets[i % ns])
         torch.cuda.synchronize()
