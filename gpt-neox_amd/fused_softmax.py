@@ -1,13 +1,19 @@
 """Drop-in for ``megatron/model/fused_softmax.py`` on MI355X.
 
-Same public names, constructor arguments, call signatures and tensor layouts as
-the reference module (megatron/model/fused_softmax.py:24-205):
-``ScaledUpperTriangMaskedSoftmax``, ``ScaledMaskedSoftmax``, ``SoftmaxFusionTypes``,
-``FusedScaleMaskSoftmax``.  The fused branches run hand-written gfx950 kernels
-through the C-ABI library; the unfused branch is the same sequence of torch ops
-as the reference's ``forward_torch_softmax``.
+Public names, constructor arguments, call signatures and tensor layouts are those
+of the reference module (megatron/model/fused_softmax.py:24-205):
 
-What differs from the reference, on purpose:
+* ``ScaledUpperTriangMaskedSoftmax.apply(inputs[B, sq, sk], scale)``
+* ``ScaledMaskedSoftmax.apply(inputs[b, np, sq, sk], mask[1|b, 1, sq, sk], scale)``
+* ``SoftmaxFusionTypes``
+* ``FusedScaleMaskSoftmax(input_in_fp16, input_in_bf16, fusion_type, mask_func,
+  softmax_in_fp32, scale)`` with ``forward(input, mask)``, ``is_kernel_available``,
+  ``forward_fused_softmax``, ``forward_torch_softmax``, ``get_batch_per_block``.
+
+The fused branches run hand-written gfx950 kernels through the C-ABI library; the
+unfused branch evaluates the same torch expression as the reference.
+
+Deliberate differences from the reference:
 
 * the fused kernels take any ``sk`` (the reference stops at 2048 and silently
   runs the torch path beyond it) and need none of the ``sq % 4``,
@@ -22,65 +28,66 @@ What differs from the reference, on purpose:
 import enum
 
 import torch
-import torch.nn as nn
 
 from .fused_kernels import load_fused_kernels
-from .fused_kernels import scaled_masked_softmax_cuda
-from .fused_kernels import scaled_upper_triang_masked_softmax_cuda
+from .fused_kernels import scaled_masked_softmax_cuda as _masked_ext
+from .fused_kernels import scaled_upper_triang_masked_softmax_cuda as _causal_ext
+
+
+def _remember(ctx, probs, scale_t):
+    ctx.save_for_backward(probs, scale_t)
+    return probs
+
+
+def _scale_tensor(scale):
+    # the reference keeps the scale as a one-element fp32 CPU tensor next to the saved
+    # probabilities (fused_softmax.py:36-41); same here, so the kernels see the
+    # fp32-rounded value in both passes
+    return torch.tensor([scale])
+
+
+def _recall(ctx):
+    probs, scale_t = ctx.saved_tensors
+    return probs, scale_t[0].item()
 
 
 class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
-    """
-    Fused operation which performs following three operations in sequence
-    1. Scale the tensor.
-    2. Apply upper triangular mask (typically used in gpt models).
-    3. Perform softmax.
+    """scale -> causal (upper-triangular) mask -> softmax, in one kernel.
 
-    ``inputs`` is ``[attn_batches, sq, sk]`` fp16/bf16; reference:
-    megatron/model/fused_softmax.py:24-53.
+    ``inputs``: ``[attn_batches, sq, sk]`` fp16/bf16 on the GPU; returns probabilities
+    of the same shape and dtype with exact zeros above the diagonal.  The gradient
+    kernel writes into the incoming gradient buffer when it is contiguous, as the
+    reference does.  Reference: megatron/model/fused_softmax.py:24-53.
     """
 
     @staticmethod
     def forward(ctx, inputs, scale):
-        scale_t = torch.tensor([scale])  # 1-element fp32 CPU tensor, as in the reference
-        softmax_results = scaled_upper_triang_masked_softmax_cuda.forward(inputs, scale_t[0].item())
-        ctx.save_for_backward(softmax_results, scale_t)
-        return softmax_results
+        scale_t = _scale_tensor(scale)
+        return _remember(ctx, _causal_ext.forward(inputs, scale_t[0].item()), scale_t)
 
     @staticmethod
     def backward(ctx, output_grads):
-        softmax_results, scale_t = ctx.saved_tensors
-        input_grads = scaled_upper_triang_masked_softmax_cuda.backward(
-            output_grads, softmax_results, scale_t[0].item()
-        )
-        return input_grads, None
+        probs, scale = _recall(ctx)
+        return _causal_ext.backward(output_grads, probs, scale), None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
-    """
-    Fused operation which performs following three operations in sequence
-    1. Scale the tensor.
-    2. Apply the mask.
-    3. Perform softmax.
+    """scale -> mask tensor -> softmax, in one kernel.
 
-    ``inputs`` is ``[b, np, sq, sk]`` fp16/bf16, ``mask`` is ``[1 or b, 1, sq, sk]``
-    bool/uint8 with True = masked; reference: megatron/model/fused_softmax.py:56-83.
+    ``inputs``: ``[b, np, sq, sk]`` fp16/bf16; ``mask``: ``[1 or b, 1, sq, sk]`` bool or
+    uint8, non-zero = masked, shared by all heads.  Reference:
+    megatron/model/fused_softmax.py:56-83.
     """
 
     @staticmethod
     def forward(ctx, inputs, mask, scale):
-        scale_t = torch.tensor([scale])
-        softmax_results = scaled_masked_softmax_cuda.forward(inputs, mask, scale_t[0].item())
-        ctx.save_for_backward(softmax_results, scale_t)
-        return softmax_results
+        scale_t = _scale_tensor(scale)
+        return _remember(ctx, _masked_ext.forward(inputs, mask, scale_t[0].item()), scale_t)
 
     @staticmethod
     def backward(ctx, output_grads):
-        softmax_results, scale_t = ctx.saved_tensors
-        input_grads = scaled_masked_softmax_cuda.backward(
-            output_grads, softmax_results, scale_t[0].item()
-        )
-        return input_grads, None, None
+        probs, scale = _recall(ctx)
+        return _masked_ext.backward(output_grads, probs, scale), None, None
 
 
 class SoftmaxFusionTypes(enum.Enum):
@@ -89,62 +96,39 @@ class SoftmaxFusionTypes(enum.Enum):
     none = 3  # no fusion
 
 
-class FusedScaleMaskSoftmax(nn.Module):
-    """
-    fused operation: scaling + mask + softmax
-    Arguments:
-        input_in_fp16: flag to indicate if input in fp16 data format.
-        input_in_bf16: flag to indicate if input in bf16 data format.
-        fusion_type: type of fusion to perform, should be either upper_triang, general or none. None will perform a regular torch softmax.
-        mask_func: mask function to be applied.
-        softmax_in_fp32: if true, softmax in performed at fp32 precision.
-        scale: scaling factor used in input tensor scaling.
+class FusedScaleMaskSoftmax(torch.nn.Module):
+    """Scaling + masking + softmax of attention scores ``[b, np, sq, sk]``.
+
+    input_in_fp16 / input_in_bf16: storage type of the scores.
+    fusion_type: a ``SoftmaxFusionTypes``; ``none`` always takes the torch branch.
+    mask_func: ``mask_func(scores, mask) -> scores`` used by the torch branch.
+    softmax_in_fp32: torch branch computes in fp32 (the kernels always do).
+    scale: multiplier applied before the softmax, or None.
 
     Reference: megatron/model/fused_softmax.py:92-205.
     """
 
-    def __init__(
-        self,
-        input_in_fp16,
-        input_in_bf16,
-        fusion_type,
-        mask_func,
-        softmax_in_fp32,
-        scale,
-    ):
+    def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale):
         super().__init__()
+        assert fusion_type in list(SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
+        assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
+
         self.input_in_fp16 = input_in_fp16
         self.input_in_bf16 = input_in_bf16
-        self.input_in_float16 = self.input_in_fp16 or self.input_in_bf16
-
-        assert fusion_type in [
-            SoftmaxFusionTypes.upper_triang,
-            SoftmaxFusionTypes.general,
-            SoftmaxFusionTypes.none,
-        ], f"Invalid fusion type {fusion_type}"
-
-        if fusion_type != SoftmaxFusionTypes.none:
-            load_fused_kernels()  # check fused kernels are installed
-
-        self.upper_triang_mask_fusion = fusion_type == SoftmaxFusionTypes.upper_triang
-        self.general_mask_fusion = fusion_type == SoftmaxFusionTypes.general
-        self.fusion = fusion_type != SoftmaxFusionTypes.none
-
+        self.input_in_float16 = input_in_fp16 or input_in_bf16
+        self.fusion = fusion_type is not SoftmaxFusionTypes.none
+        self.upper_triang_mask_fusion = fusion_type is SoftmaxFusionTypes.upper_triang
+        self.general_mask_fusion = fusion_type is SoftmaxFusionTypes.general
         self.mask_func = mask_func
         self.softmax_in_fp32 = softmax_in_fp32
         self.scale = scale
-
-        assert (
-            self.scale is None or softmax_in_fp32
-        ), "softmax should be in fp32 when scaled"
+        if self.fusion:
+            load_fused_kernels()  # ImportError here, not at the first forward
 
     def forward(self, input, mask):
-        # [b, np, sq, sk]
-        assert input.dim() == 4
-        if self.is_kernel_available(mask, *input.size()):
-            return self.forward_fused_softmax(input, mask)
-        else:
-            return self.forward_torch_softmax(input, mask)
+        assert input.dim() == 4  # [b, np, sq, sk]
+        fused = self.is_kernel_available(mask, *input.size())
+        return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """Whether the fused branch serves this call.
@@ -160,60 +144,41 @@ class FusedScaleMaskSoftmax(nn.Module):
             return False
         if b * np * sq * sk == 0:
             return False
-        if self.upper_triang_mask_fusion:
-            return sq == sk
-        return True
+        return sq == sk if self.upper_triang_mask_fusion else True
 
     @staticmethod
     def reference_is_kernel_available(fusion, upper_triang, input_in_float16, mask, b, np, sq, sk):
         """The reference's own predicate (megatron/model/fused_softmax.py:148-168),
         evaluated with wave64 ``get_batch_per_block`` values; for comparison only."""
-        attn_batches = b * np
-        if (
-            fusion
-            and input_in_float16
-            and mask is not None
-            and 16 < sk <= 2048
-            and sq % 4 == 0
-            and attn_batches % 4 == 0
-        ):
-            batch_per_block = FusedScaleMaskSoftmax.get_batch_per_block(sq, sk, b, np)
-            if upper_triang:
-                return attn_batches % batch_per_block == 0
-            return sq % batch_per_block == 0
-        return False
+        shape_ok = 16 < sk <= 2048 and sq % 4 == 0 and (b * np) % 4 == 0
+        if not (fusion and input_in_float16 and mask is not None and shape_ok):
+            return False
+        per_block = FusedScaleMaskSoftmax.get_batch_per_block(sq, sk, b, np)
+        return ((b * np) if upper_triang else sq) % per_block == 0
 
     def forward_fused_softmax(self, input, mask):
         b, np, sq, sk = input.size()
-        scale = self.scale if self.scale is not None else 1.0
-        if self.upper_triang_mask_fusion:
-            assert sq == sk, "causal mask is only for self attention"
-
-            # input is 3D tensor (attn_batches, sq, sk)
-            input = input.view(-1, sq, sk)
-            probs = ScaledUpperTriangMaskedSoftmax.apply(input, scale)
-            return probs.view(b, np, sq, sk)
-        else:
-            # input is 4D tensor (b, np, sq, sk)
+        scale = 1.0 if self.scale is None else self.scale
+        if not self.upper_triang_mask_fusion:
             return ScaledMaskedSoftmax.apply(input, mask, scale)
+        # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
+        assert sq == sk, "causal mask is only for self attention"
+        probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
+        return probs.view(b, np, sq, sk)
 
     def forward_torch_softmax(self, input, mask):
-        if self.input_in_float16 and self.softmax_in_fp32:
-            input = input.float()
-
+        """The unfused path: optional upcast, scale, ``mask_func``, softmax, cast back."""
+        upcast = self.input_in_float16 and self.softmax_in_fp32
+        scores = input.float() if upcast else input
         if self.scale is not None:
-            input = input * self.scale
-        mask_output = self.mask_func(input, mask) if mask is not None else input
-        probs = torch.nn.Softmax(dim=-1)(mask_output)
-
-        if self.input_in_float16 and self.softmax_in_fp32:
-            if self.input_in_fp16:
-                probs = probs.half()
-            else:
-                probs = probs.bfloat16()
-
+            scores = scores * self.scale
+        if mask is not None:
+            scores = self.mask_func(scores, mask)
+        probs = torch.softmax(scores, dim=-1)
+        if upcast:
+            probs = probs.half() if self.input_in_fp16 else probs.bfloat16()
         return probs
 
     @staticmethod
     def get_batch_per_block(sq, sk, b, np):
-        return scaled_masked_softmax_cuda.get_batch_per_block(sq, sk, b, np)
+        return _masked_ext.get_batch_per_block(sq, sk, b, np)
