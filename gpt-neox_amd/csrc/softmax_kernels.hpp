@@ -8,10 +8,10 @@
 // round-robin to its waves (balanced under the causal mask) and the row maximum
 // and sum are combined through a few floats of LDS.
 //
-// Causal rows read only the columns j <= i: chunks entirely above the diagonal
-// are neither loaded nor computed (wave-uniform branch), lanes past the diagonal
-// inside the boundary chunk issue no load; the zeros of the upper triangle are
-// still stored because the consumer reads the matrix densely.
+// Causal rows read only the columns j <= i: the row is described to the hardware as a
+// buffer of i+1 elements, so lanes past the diagonal fetch nothing, and chunks entirely
+// above the diagonal are not computed (wave-uniform branch); the zeros of the upper
+// triangle are still stored because the consumer reads the matrix densely.
 //
 // Arithmetic: fp32, exp(x*scale - max) evaluated as exp2(x*(scale*log2e) - max'),
 // one reciprocal per row, one rounding to the storage type on store.
@@ -36,6 +36,32 @@ struct SoftmaxArgs {
 
 enum class Mask { Causal, Bytes, None };
 
+// Compile-time tuning switches of the row kernels.
+constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
+constexpr int kNtStore = 2;  // non-temporal hint on the streaming stores
+constexpr int kDefaultFlags = kNtLoad | kNtStore;
+
+// Where a wave works: the row, its position i inside its [sq, sk] matrix, the number of
+// columns that take part, and whether the result is stored (surplus waves of the last
+// block recompute the last row and store nothing, so that every wave of a block reaches
+// the barriers).  All fields are wave-uniform.
+struct RowPos {
+    uint32_t row;
+    uint32_t i;
+    int len;
+    bool store;
+};
+
+template <Mask MASK>
+__device__ __forceinline__ RowPos locate(uint32_t row, const SoftmaxArgs& a) {
+    RowPos p;
+    p.store = row < a.rows;
+    p.row = p.store ? row : a.rows - 1;
+    p.i = p.row % (uint32_t)a.sq;
+    p.len = (MASK == Mask::Causal) ? min((int)p.i + 1, a.sk) : a.sk;
+    return p;
+}
+
 // Combine a per-wave partial across the WPR waves of a row.
 template <typename Op, int WPR, int RPB>
 __device__ __forceinline__ float row_combine(float v, float* red, int wib, int rib, int lane) {
@@ -53,195 +79,200 @@ __device__ __forceinline__ float row_combine(float v, float* red, int wib, int r
 
 // ---------------------------------------------------------------------------------
 // forward
+//
+// One launch covers all rows: block b owns rows b*RPB .. b*RPB+RPB-1 and retires when they
+// are done; the hardware dispatcher keeps every CU supplied with fresh blocks, which
+// measured faster on MI355X than a persistent grid that prefetches its next row.
+// Loads and stores are range-checked buffer accesses against the row's valid length:
+// lanes past the causal diagonal (or the row end) fetch nothing, and no branch surrounds
+// a memory instruction, so the waits are exact.
 // ---------------------------------------------------------------------------------
-template <typename T, int NCH, int WPR, int RPB, Mask MASK>
+template <typename T, int NCH, int WPR, int RPB, Mask MASK, int FLAGS = kDefaultFlags>
 __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArgs a) {
     __shared__ float red_max[WPR * RPB];
     __shared__ float red_sum[WPR * RPB];
+    constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wib = threadIdx.x >> 6;  // wave in block
-    const int rib = wib / WPR;         // row in block
-    const int wir = wib % WPR;         // wave in row
-
-    uint32_t row = blockIdx.x * RPB + rib;
-    const bool store = row < a.rows;  // surplus waves of the last block recompute the last row
-    if (!store) row = a.rows - 1;     // and store nothing, so every wave reaches the barriers
-
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave in block
+    const int rib = wib / WPR;                                         // row in block
+    const int wir = wib % WPR;                                         // wave in row
     const int sk = a.sk;
-    const uint32_t i = row % (uint32_t)a.sq;
-    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;  // columns that take part
+    const float ninf = -__builtin_inff();
+    // byte offset of the lane inside the row, first chunk of its wave.  Everything goes into
+    // the per-lane offset: the hardware's range check does not see the scalar offset operand.
+    const int voff = lane * 16 + wir * kChunk * 2;
 
-    const char* x = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
-    char* y = static_cast<char*>(a.out) + (size_t)row * sk * 2;
-    const uint8_t* mrow = nullptr;
-    if constexpr (MASK == Mask::Bytes) {
-        const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
-        mrow = a.mask + ((size_t)mb * a.sq + i) * sk;
-    }
-
-    float v[NCH][8];
+    const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
     u32x4 raw[NCH];
     u32x2 mk[NCH];
-
-    // ---- issue every load of the row before the first use
+    {
+        // ---- issue every load of the row before the first use
+        const char* x = static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2;
+        const rsrc_t rx = make_rsrc(x, (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u);
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int col = (wir + WPR * c) * kChunk + lane * kVec;
-        raw[c] = u32x4{0, 0, 0, 0};
-        mk[c] = u32x2{0, 0};
-        if (col < len) {
-            raw[c] = ld128(x + (size_t)col * 2);
-            if constexpr (MASK == Mask::Bytes) mk[c] = ld64_cached(mrow + col);
+        for (int c = 0; c < NCH; ++c) raw[c] = buf_ld128<kLdNt>(rx, voff + c * WPR * kChunk * 2, 0);
+        if constexpr (MASK == Mask::Bytes) {
+            const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
+            const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)pos.len);
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) mk[c] = buf_ld64(rm, lane * 8 + (wir + c * WPR) * kChunk, 0);
         }
     }
+    {
+        const int len = pos.len;
+        float v[NCH][8];
 
-    // ---- scale, mask, running maximum
-    const float ninf = -__builtin_inff();
-    float mx = ninf;
+        // ---- scale, mask, running maximum
+        float mx = ninf;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
-        if (c0 < len) {
-            unpack8<T>(raw[c], v[c]);
-            const int col = c0 + lane * kVec;
-            bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
-            if constexpr (MASK == Mask::Bytes) {
-                plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
-            }
-            if (plain) {
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    v[c][k] *= a.scale;
-                    mx = fmaxf(mx, v[c][k]);
+        for (int c = 0; c < NCH; ++c) {
+            const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
+            if (c0 < len) {
+                unpack8<T>(raw[c], v[c]);
+                const int col = c0 + lane * kVec;
+                bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
+                if constexpr (MASK == Mask::Bytes) {
+                    plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
                 }
-            } else {
+                if (plain) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    bool keep = (col + k) < len;
-                    if constexpr (MASK == Mask::Bytes) {
-                        const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
-                        keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
+                    for (int k = 0; k < 8; ++k) {
+                        v[c][k] *= a.scale;
+                        mx = fmaxf(mx, v[c][k]);
                     }
-                    v[c][k] = keep ? v[c][k] * a.scale : ninf;
-                    mx = fmaxf(mx, v[c][k]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        bool keep = (col + k) < len;
+                        if constexpr (MASK == Mask::Bytes) {
+                            const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
+                            keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
+                        }
+                        v[c][k] = keep ? v[c][k] * a.scale : ninf;
+                        mx = fmaxf(mx, v[c][k]);
+                    }
                 }
             }
         }
-    }
-    mx = wave_reduce<OpMax>(mx);
-    mx = row_combine<OpMax, WPR, RPB>(mx, red_max, wib, rib, lane);
+        mx = wave_reduce<OpMax>(mx);
+        mx = row_combine<OpMax, WPR, RPB>(mx, red_max, wib, rib, lane);
 
-    // A row whose every key is masked: the unfused path fills all scores with the same
-    // value, so the result is uniform over the sk columns.
-    const bool all_masked = (mx == ninf);
+        // A row whose every key is masked: the unfused path fills all scores with the same
+        // value, so the result is uniform over the sk columns.
+        const bool all_masked = (mx == ninf);
 
-    // ---- exponentials and their sum
-    float sum = 0.f;
+        // ---- exponentials and their sum
+        float sum = 0.f;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int c0 = (wir + WPR * c) * kChunk;
-        if (c0 < len) {
-            const int col = c0 + lane * kVec;
+        for (int c = 0; c < NCH; ++c) {
+            const int c0 = (wir + WPR * c) * kChunk;
+            if (c0 < len) {
+                const int col = c0 + lane * kVec;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                float e = fast_exp2(v[c][k] - mx);
-                if (all_masked) e = ((col + k) < len) ? 1.f : 0.f;
-                v[c][k] = e;
-                sum += e;
+                for (int k = 0; k < 8; ++k) {
+                    float e = fast_exp2(v[c][k] - mx);
+                    if (all_masked) e = ((col + k) < len) ? 1.f : 0.f;
+                    v[c][k] = e;
+                    sum += e;
+                }
             }
         }
-    }
-    sum = wave_reduce<OpSum>(sum);
-    sum = row_combine<OpSum, WPR, RPB>(sum, red_sum, wib, rib, lane);
-    const float inv = 1.0f / sum;
+        sum = wave_reduce<OpSum>(sum);
+        sum = row_combine<OpSum, WPR, RPB>(sum, red_sum, wib, rib, lane);
+        const float inv = 1.0f / sum;
 
-    // ---- normalise and store; chunks above the diagonal store zeros
-    if (!store) return;
+        // ---- normalise and store; chunks above the diagonal store zeros
+        char* y = static_cast<char*>(a.out) + (size_t)pos.row * sk * 2;
+        const rsrc_t ry = make_rsrc(y, pos.store ? (uint32_t)sk * 2u : 0u);
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int c0 = (wir + WPR * c) * kChunk;
-        const int col = c0 + lane * kVec;
-        u32x4 o = u32x4{0, 0, 0, 0};
-        if (c0 < len) {
+        for (int c = 0; c < NCH; ++c) {
+            const int c0 = (wir + WPR * c) * kChunk;
+            u32x4 o = u32x4{0, 0, 0, 0};
+            if (c0 < len) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[c][k] *= inv;
-            o = pack8<T>(v[c]);
+                for (int k = 0; k < 8; ++k) v[c][k] *= inv;
+                o = pack8<T>(v[c]);
+            }
+            buf_st128<kStNt>(ry, o, voff + c * WPR * kChunk * 2, 0);
         }
-        if (col < sk) st128(y + (size_t)col * 2, o);
     }
 }
 
 // ---------------------------------------------------------------------------------
 // backward:  dx = scale * y * (dy - sum_j dy_j*y_j)
 // ---------------------------------------------------------------------------------
-template <typename T, int NCH, int WPR, int RPB, Mask MASK>
+template <typename T, int NCH, int WPR, int RPB, Mask MASK, int FLAGS = kDefaultFlags>
 __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArgs a) {
     __shared__ float red_sum[WPR * RPB];
+    constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
 
     const int lane = threadIdx.x & (kWave - 1);
-    const int wib = threadIdx.x >> 6;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rib = wib / WPR;
     const int wir = wib % WPR;
-
-    uint32_t row = blockIdx.x * RPB + rib;
-    const bool store = row < a.rows;
-    if (!store) row = a.rows - 1;
-
     const int sk = a.sk;
-    const uint32_t i = row % (uint32_t)a.sq;
-    const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+    const int voff = lane * 16 + wir * kChunk * 2;  // the range check ignores a scalar offset
 
-    const char* g = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
-    const char* p = static_cast<const char*>(a.in1) + (size_t)row * sk * 2;
-    char* dx = static_cast<char*>(a.out) + (size_t)row * sk * 2;
-
+    const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
     u32x4 rg[NCH], rp[NCH];
+    {
+        const uint32_t bytes = (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
+        const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2, bytes);
+        const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int col = (wir + WPR * c) * kChunk + lane * kVec;
-        rg[c] = u32x4{0, 0, 0, 0};
-        rp[c] = u32x4{0, 0, 0, 0};
-        if (col < len) {
-            rg[c] = ld128(g + (size_t)col * 2);
-            rp[c] = ld128(p + (size_t)col * 2);
+        for (int c = 0; c < NCH; ++c) {
+            rg[c] = buf_ld128<kLdNt>(bg, voff + c * WPR * kChunk * 2, 0);
+            rp[c] = buf_ld128<kLdNt>(by, voff + c * WPR * kChunk * 2, 0);
         }
     }
+    {
+        // dx may alias dy: a row is read and written by the same waves only, reads first
+        const int len = pos.len;
 
-    float gv[NCH][8], pv[NCH][8];
-    float dot = 0.f;
+        // the row stays packed; it is unpacked once for the dot product and once for dx
+        float dot = 0.f;
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int c0 = (wir + WPR * c) * kChunk;
-        if (c0 < len) {
-            unpack8<T>(rg[c], gv[c]);
-            unpack8<T>(rp[c], pv[c]);
-            const int col = c0 + lane * kVec;
-            if (c0 + kChunk > len) {
-                // the lane holding the diagonal may have loaded columns past it
+        for (int c = 0; c < NCH; ++c) {
+            const int c0 = (wir + WPR * c) * kChunk;
+            if (c0 < len) {
+                float gv[8], pv[8];
+                unpack8<T>(rg[c], gv);
+                unpack8<T>(rp[c], pv);
+                const int col = c0 + lane * kVec;
+                if (c0 + kChunk > len) {
+                    // the lane holding the diagonal may have loaded columns past it
 #pragma unroll
-                for (int k = 0; k < 8; ++k)
-                    if ((col + k) >= len) pv[c][k] = 0.f;
+                    for (int k = 0; k < 8; ++k)
+                        if ((col + k) >= len) pv[k] = 0.f;
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) dot = fmaf(gv[k], pv[k], dot);
             }
-#pragma unroll
-            for (int k = 0; k < 8; ++k) dot = fmaf(gv[c][k], pv[c][k], dot);
         }
-    }
-    dot = wave_reduce<OpSum>(dot);
-    dot = row_combine<OpSum, WPR, RPB>(dot, red_sum, wib, rib, lane);
+        dot = wave_reduce<OpSum>(dot);
+        dot = row_combine<OpSum, WPR, RPB>(dot, red_sum, wib, rib, lane);
 
-    if (!store) return;
+        char* dx = static_cast<char*>(a.out) + (size_t)pos.row * sk * 2;
+        const rsrc_t rdx = make_rsrc(dx, pos.store ? (uint32_t)sk * 2u : 0u);
 #pragma unroll
-    for (int c = 0; c < NCH; ++c) {
-        const int c0 = (wir + WPR * c) * kChunk;
-        const int col = c0 + lane * kVec;
-        u32x4 o = u32x4{0, 0, 0, 0};
-        if (c0 < len) {
+        for (int c = 0; c < NCH; ++c) {
+            const int c0 = (wir + WPR * c) * kChunk;
+            u32x4 o = u32x4{0, 0, 0, 0};
+            if (c0 < len) {
+                float gv[8], pv[8];
+                unpack8<T>(rg[c], gv);
+                unpack8<T>(rp[c], pv);
+                const int col = c0 + lane * kVec;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) gv[c][k] = a.scale * (pv[c][k] * (gv[c][k] - dot));
-            o = pack8<T>(gv[c]);
+                for (int k = 0; k < 8; ++k) {
+                    gv[k] = a.scale * (pv[k] * (gv[k] - dot));
+                    if ((c0 + kChunk > len) && (col + k) >= len) gv[k] = 0.f;
+                }
+                o = pack8<T>(gv);
+            }
+            buf_st128<kStNt>(rdx, o, voff + c * WPR * kChunk * 2, 0);
         }
-        if (col < sk) st128(dx + (size_t)col * 2, o);
     }
 }
 

@@ -103,6 +103,33 @@ __device__ __forceinline__ u32x2 ld64_cached(const void* p) {
     return *reinterpret_cast<const u32x2*>(p);
 }
 
+// ---- buffer (range-checked) access --------------------------------------------------
+// A buffer resource describes one row: base address and its length in bytes.  Lanes whose
+// byte offset falls outside [0, bytes) load zeros / store nothing and cause no memory
+// traffic, so partially filled rows need no branch around their loads and stores -- and
+// with a fixed number of memory instructions per row the compiler can wait on exactly the
+// loads it needs while later stores are still in flight.  The range check covers the
+// per-lane offset plus the instruction's immediate; a scalar offset operand is NOT
+// checked, so callers keep `soffset` at 0.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+constexpr int kAuxNt = 2;               // non-temporal hint
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kRsrcFlags);
+}
+template <bool NT>
+__device__ __forceinline__ u32x4 buf_ld128(rsrc_t r, int voffset, int soffset) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, voffset, soffset, NT ? kAuxNt : 0);
+}
+template <bool NT>
+__device__ __forceinline__ void buf_st128(rsrc_t r, const u32x4& v, int voffset, int soffset) {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, voffset, soffset, NT ? kAuxNt : 0);
+}
+__device__ __forceinline__ u32x2 buf_ld64(rsrc_t r, int voffset, int soffset) {
+    return __builtin_amdgcn_raw_buffer_load_b64(r, voffset, soffset, 0);
+}
+
 // ---- wave64 reductions --------------------------------------------------------
 // DPP controls (GCN3+/CDNA encoding)
 constexpr int kDppQuadSwap1 = 0xB1;    // quad_perm:[1,0,3,2]

@@ -190,6 +190,35 @@ def test_causal_very_long_rows(device, s):
     assert (dx[0][rows][mask] == 0).all()
 
 
+@pytest.mark.parametrize("s", [520, 1032, 2056, 4104, 8200])
+def test_nothing_is_written_past_the_end_of_the_output(device, s):
+    # rows that do not fill the last chunk of their waves: lanes past the row end must
+    # store nothing, neither into the next row nor behind the tensor
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 2 * s * s
+    x = scores((2, s, s), torch.float16, device, s)
+    g = normal((2, s, s), torch.float16, device, s + 1)
+    guard = 4096
+    for kind in ("causal", "masked"):
+        out = torch.full((n + guard,), 7.0, dtype=torch.float16, device=device)
+        dxo = torch.full((n + guard,), 7.0, dtype=torch.float16, device=device)
+        if kind == "causal":
+            _lib.check(lib.neox_causal_softmax_fwd(out.data_ptr(), x.data_ptr(), 0.125, 2, s, s, _lib.NEOX_F16, stream))
+            _lib.check(lib.neox_causal_softmax_bwd(dxo.data_ptr(), g.data_ptr(), out.data_ptr(), 0.125, 2, s, s,
+                                                   _lib.NEOX_F16, stream))
+            want = causal_ext.forward(x, 0.125)
+        else:
+            mask = torch.zeros(1, 1, s, s, dtype=torch.bool, device=device)
+            _lib.check(lib.neox_masked_softmax_fwd(out.data_ptr(), x.data_ptr(), mask.data_ptr(), 0.125, 1, 2, s, s,
+                                                   1, _lib.NEOX_F16, stream))
+            _lib.check(lib.neox_masked_softmax_bwd(dxo.data_ptr(), g.data_ptr(), out.data_ptr(), 0.125, 2 * s, s,
+                                                   _lib.NEOX_F16, stream))
+            want = masked_ext.forward(x.view(1, 2, s, s), mask, 0.125)
+        assert torch.equal(out[:n].view(2, s, s), want.view(2, s, s))
+        assert (out[n:] == 7.0).all() and (dxo[n:] == 7.0).all(), kind
+
+
 def test_causal_negative_and_large_scale(device):
     for scale in (-0.25, 4.0, 1.0):
         check_causal(device, 2, 96, torch.float16, scale, seed=3)
