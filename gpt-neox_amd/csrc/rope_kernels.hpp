@@ -3,12 +3,21 @@
 // s/b/h strides (the inputs are usually views into a fused QKV buffer).
 //
 // One block serves one sequence position: the position's cos/sin values are loaded
-// once into registers and reused for every head of q and k.  threadIdx.x selects
-// a slot of W consecutive dims in the first half of the rotated span; the thread
-// also owns the matching W dims of the second half, so the pair (j, j + d_rot/2)
-// never crosses lanes and in-place operation is race-free.  threadIdx.y walks the
-// (b, h) vectors.  W = 8 gives 128-bit accesses; W = 4, 2, 1 serve head sizes and
-// strides that do not allow them.
+// once into registers and reused for every head of q and k.  Two kernels:
+//
+// * rope_span_kernel -- d_rot/8 a power of two (d_rot = 16 ... 512) and 16-byte aligned
+//   layouts.  Each lane owns ONE 16-byte slot (8 dims) of a head's rotated span and
+//   consecutive lanes own consecutive slots, so a wave access covers whole contiguous
+//   spans (64 B for d_rot = 32, 256 B for d_rot = 128).  The partner dims (j +- d_rot/2)
+//   live d_rot/16 lanes away and are fetched with a wave shuffle.  q and k of one
+//   block iteration are loaded together before any arithmetic.
+// * rope_kernel -- every other head size / alignment.  threadIdx.x selects a slot of W
+//   consecutive dims in the first half of the rotated span; the thread also owns the
+//   matching W dims of the second half, so no data crosses lanes (W = 8, 4, 2, 1).
+//
+// In both, a lane reads everything it needs before it writes, and a pair
+// (j, j + d_rot/2) is written by the lane(s) that read it, so in-place operation is
+// race-free.  q/k accesses carry the non-temporal hint (each byte is touched once).
 //
 // Arithmetic is fp32 with the two products rounded separately (no fused
 // multiply-add), which is bit-identical to evaluating q*cos + rotate_half(q)*sin
@@ -48,20 +57,21 @@ struct Pack<4> { typedef u32x2 type; };
 template <>
 struct Pack<2> { typedef uint32_t type; };
 
-template <typename T, int W>
+template <typename T, int W, bool NT = false>
 __device__ __forceinline__ void load_elems(const char* p, float (&f)[W]) {
     if constexpr (W == 1) {
         f[0] = Elem<T>::load1(p);
     } else {
         typedef typename Pack<W>::type P;
-        const P w = *reinterpret_cast<const P*>(p);
+        const P w = NT ? __builtin_nontemporal_load(reinterpret_cast<const P*>(p))
+                       : *reinterpret_cast<const P*>(p);
         const uint32_t* u = reinterpret_cast<const uint32_t*>(&w);
 #pragma unroll
         for (int k = 0; k < W / 2; ++k) Elem<T>::unpack(u[k], f[2 * k], f[2 * k + 1]);
     }
 }
 
-template <typename T, int W>
+template <typename T, int W, bool NT = false>
 __device__ __forceinline__ void store_elems(char* p, const float (&f)[W]) {
     if constexpr (W == 1) {
         Elem<T>::store1(p, f[0]);
@@ -71,7 +81,8 @@ __device__ __forceinline__ void store_elems(char* p, const float (&f)[W]) {
         uint32_t* u = reinterpret_cast<uint32_t*>(&w);
 #pragma unroll
         for (int k = 0; k < W / 2; ++k) u[k] = Elem<T>::pack(f[2 * k], f[2 * k + 1]);
-        *reinterpret_cast<P*>(p) = w;
+        if constexpr (NT) __builtin_nontemporal_store(w, reinterpret_cast<P*>(p));
+        else *reinterpret_cast<P*>(p) = w;
     }
 }
 
@@ -148,26 +159,103 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
         const char* qp = a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2;
         const char* kp = a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2;
         if (do_q) {
-            load_elems<T, W>(qp, ql);
-            load_elems<T, W>(qp + (size_t)half * 2, qh);
+            load_elems<T, W, true>(qp, ql);
+            load_elems<T, W, true>(qp + (size_t)half * 2, qh);
         }
         if (do_k) {
-            load_elems<T, W>(kp, kl);
-            load_elems<T, W>(kp + (size_t)half * 2, kh);
+            load_elems<T, W, true>(kp, kl);
+            load_elems<T, W, true>(kp + (size_t)half * 2, kh);
         }
         if (do_q) {
             float ol[W], oh[W];
             rotate<T, W, BWD>(ql, qh, cl, ch, sl, sh, ol, oh);
             char* op = a.t[0].out + (qo + (int64_t)v * a.t[0].out_stride[2]) * 2;
-            store_elems<T, W>(op, ol);
-            store_elems<T, W>(op + (size_t)half * 2, oh);
+            store_elems<T, W, true>(op, ol);
+            store_elems<T, W, true>(op + (size_t)half * 2, oh);
         }
         if (do_k) {
             float ol[W], oh[W];
             rotate<T, W, BWD>(kl, kh, cl, ch, sl, sh, ol, oh);
             char* op = a.t[1].out + (ko + (int64_t)v * a.t[1].out_stride[2]) * 2;
-            store_elems<T, W>(op, ol);
-            store_elems<T, W>(op + (size_t)half * 2, oh);
+            store_elems<T, W, true>(op, ol);
+            store_elems<T, W, true>(op + (size_t)half * 2, oh);
+        }
+    }
+}
+
+// ---- contiguous-span kernel -----------------------------------------------------------
+constexpr int kSpanIters = 2;  // head vectors per thread and tensor whose loads are in flight together
+
+template <typename T, typename CS, bool BWD>
+__global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
+    const int lps = a.lpv * 2;  // 16-byte slots per rotated span: a power of two <= 64
+    const int hl = a.lpv;       // lane distance to the partner slot
+    const int tid = threadIdx.x;
+    const int slot = tid & (lps - 1);
+    const int vib = tid / lps;   // vector handled in a block iteration
+    const int vpb = 256 / lps;   // vectors per block iteration
+    const int pos = blockIdx.x;
+    const int outer = blockIdx.y;
+    const bool second = slot >= hl;
+    const int j = slot * 8;            // first dim this lane owns
+    const int jp = (slot ^ hl) * 8;    // first dim of the partner lane
+
+    // out = x*cos[own] + sign * partner * sin[.]: the forward pass takes sin at the lane's own
+    // dims with sign -,+ for the first/second half; the backward pass takes sin at the
+    // partner's dims with sign +,-.  Folding the sign into sin is exact.
+    float c[8], sn[8];
+    const int64_t crow = (int64_t)(pos + a.pos_offset) * a.cs_stride;
+    load_table<CS, 8>(a.cos, crow + j, c);
+    load_table<CS, 8>(a.sin, crow + (BWD ? jp : j), sn);
+    if (second == BWD) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sn[k] = -sn[k];
+    }
+
+    const int nq = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
+    const int nk = (a.nt > 1 && outer < a.t[1].n_outer) ? a.t[1].n_inner : 0;
+    const int nmax = max(nq, nk);
+    const int64_t qi = (int64_t)pos * a.t[0].in_stride[0] + (int64_t)outer * a.t[0].in_stride[1] + j;
+    const int64_t qo = (int64_t)pos * a.t[0].out_stride[0] + (int64_t)outer * a.t[0].out_stride[1] + j;
+    const int64_t ki = (int64_t)pos * a.t[1].in_stride[0] + (int64_t)outer * a.t[1].in_stride[1] + j;
+    const int64_t ko = (int64_t)pos * a.t[1].out_stride[0] + (int64_t)outer * a.t[1].out_stride[1] + j;
+
+    const int step = vpb * kSpanIters;
+    // every lane of a wave runs the same number of iterations (the shuffles need all lanes)
+    for (int v0 = blockIdx.z * step; v0 < nmax; v0 += step * gridDim.z) {
+        u32x4 xq[kSpanIters], xk[kSpanIters];
+#pragma unroll
+        for (int u = 0; u < kSpanIters; ++u) {
+            const int v = v0 + u * vpb + vib;
+            xq[u] = u32x4{0, 0, 0, 0};
+            xk[u] = u32x4{0, 0, 0, 0};
+            if (v < nq) xq[u] = ld128(a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2);
+            if (v < nk) xk[u] = ld128(a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2);
+        }
+#pragma unroll
+        for (int u = 0; u < kSpanIters; ++u) {
+            const int v = v0 + u * vpb + vib;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const u32x4 x = t ? xk[u] : xq[u];
+                u32x4 p;
+                p.x = __shfl_xor((int)x.x, hl);
+                p.y = __shfl_xor((int)x.y, hl);
+                p.z = __shfl_xor((int)x.z, hl);
+                p.w = __shfl_xor((int)x.w, hl);
+                float xf[8], pf[8], o[8];
+                unpack8<T>(x, xf);
+                unpack8<T>(p, pf);
+                {
+#pragma clang fp contract(off)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) o[k] = xf[k] * c[k] + pf[k] * sn[k];
+                }
+                if (v < (t ? nk : nq)) {
+                    char* op = a.t[t].out + ((t ? ko : qo) + (int64_t)v * a.t[t].out_stride[2]) * 2;
+                    st128(op, pack8<T>(o));
+                }
+            }
         }
     }
 }
