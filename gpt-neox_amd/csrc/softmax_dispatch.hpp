@@ -1,12 +1,15 @@
 // Kernel-shape selection for the softmax kernels.
 //
-// chunks = ceil(sk / 512) decides how a row is laid over waves:
-//   chunks <= 4            one wave per row, 4 rows per 256-thread block
-//   chunks <= 8            2 waves per row
-//   chunks <= 16           4 waves per row          (sk <= 8192)
-//   chunks <= 32 / <= 64   8 / 16 waves per row     (sk <= 32768)
-// so that no wave holds more than 4 chunks (32 fp32 values per lane) and the
-// occupancy stays at 8 waves per SIMD for every row length.
+// chunks = ceil(sk / 512) decides how a row is laid over waves.  Measured on MI355X, a
+// wave that holds 2 chunks (1024 columns) is the sweet spot at every row length -- 4 chunks
+// per wave cost 3-5 % of bandwidth, 1 chunk per wave 10-20 % -- so a row gets
+// ceil(chunks / 2) waves:
+//   chunks <= 2    1 wave per row, 4 rows per 256-thread block      (sk <= 1024)
+//   chunks <= 4    2 waves per row, 2 rows per block                 (sk <= 2048)
+//   chunks <= 8    4 waves per row                                   (sk <= 4096)
+//   chunks <= 16   8 waves per row, 512-thread block                 (sk <= 8192)
+//   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
+//   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 #pragma once
 
 #include "internal.hpp"
@@ -37,28 +40,18 @@ static hipError_t launch_generic(const SoftmaxArgs& a, hipStream_t st) {
     return hipGetLastError();
 }
 
-template <typename T, Mask M, bool BWD, int WPR, int RPB>
-static hipError_t launch_split(const SoftmaxArgs& a, int chunks, hipStream_t st) {
-    // chunks in (2*WPR, 4*WPR]
-    if (chunks <= 3 * WPR) return launch_shape<T, M, BWD, 3, WPR, RPB>(a, st);
-    return launch_shape<T, M, BWD, 4, WPR, RPB>(a, st);
-}
-
 template <typename T, Mask M, bool BWD>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     const int chunks = (a.sk + kChunk - 1) / kChunk;
     if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD>(a, st);
-    switch (chunks) {
-        case 1: return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
-        case 2: return launch_shape<T, M, BWD, 2, 1, 4>(a, st);
-        case 3: return launch_shape<T, M, BWD, 3, 1, 4>(a, st);
-        case 4: return launch_shape<T, M, BWD, 4, 1, 4>(a, st);
-        default: break;
-    }
-    if (chunks <= 8) return launch_split<T, M, BWD, 2, 2>(a, chunks, st);
-    if (chunks <= 16) return launch_split<T, M, BWD, 4, 1>(a, chunks, st);
-    if (chunks <= 32) return launch_split<T, M, BWD, 8, 1>(a, chunks, st);
-    return launch_split<T, M, BWD, 16, 1>(a, chunks, st);
+    if (chunks == 1) return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
+    if (chunks == 2) return launch_shape<T, M, BWD, 2, 1, 4>(a, st);
+    if (chunks <= 4) return launch_shape<T, M, BWD, 2, 2, 2>(a, st);
+    if (chunks <= 8) return launch_shape<T, M, BWD, 2, 4, 1>(a, st);
+    if (chunks <= 16) return launch_shape<T, M, BWD, 2, 8, 1>(a, st);
+    if (chunks <= 32) return launch_shape<T, M, BWD, 2, 16, 1>(a, st);
+    if (chunks <= 48) return launch_shape<T, M, BWD, 3, 16, 1>(a, st);
+    return launch_shape<T, M, BWD, 4, 16, 1>(a, st);
 }
 
 template <bool BWD>

@@ -1,12 +1,12 @@
 // Scaled masked softmax kernels for gfx950, forward and backward.
 //
-// Work decomposition: a row of the score matrix is owned by WPR wave64s (WPR = 1
-// for rows up to 2048-4096 columns, more for longer rows).  Each wave keeps its
-// share of the row in VGPRs as fp32 -- NCH "chunks" of 512 columns, lane l owning
-// columns 8l..8l+7 of a chunk, so every load/store is one 128-bit access per lane
-// and 1 KiB contiguous per wave.  With WPR > 1 the chunks of a row are dealt
-// round-robin to its waves (balanced under the causal mask) and the row maximum
-// and sum are combined through a few floats of LDS.
+// Work decomposition: a row of the score matrix is owned by WPR wave64s (1 for rows up
+// to 1024 columns, 2 up to 2048, ... 16 beyond 8192).  Each wave keeps its share of the
+// row in VGPRs as fp32 -- NCH "chunks" of 512 columns, lane l owning columns 8l..8l+7 of
+// a chunk, so every load/store is one 128-bit access per lane and 1 KiB contiguous per
+// wave.  With WPR > 1 the chunks of a row are dealt round-robin to its waves (balanced
+// under the causal mask) and the row maximum and sum are combined through a few floats
+// of LDS.
 //
 // Causal rows read only the columns j <= i: the row is described to the hardware as a
 // buffer of i+1 elements, so lanes past the diagonal fetch nothing, and chunks entirely

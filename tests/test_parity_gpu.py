@@ -159,8 +159,8 @@ def check_causal(device, batches, s, dtype, scale, seed, chunk=4):
 
 
 # row lengths chosen to hit: 1 column; lanes partly filled; not a multiple of 8 (element-wise
-# kernels); each chunk count 1..4 of the one-wave kernels; the 2-, 4-, 8- and 16-wave kernels
-# with 3 and 4 chunks per wave; a row longer than the register-resident limit.
+# kernels); 1 and 2 chunks of 512 columns on one wave; the 2-, 4- and 8-wave kernels with rows
+# that fill their last chunk exactly, partly, or leave whole chunks of a wave empty.
 CAUSAL_SIZES = [1, 2, 7, 8, 16, 37, 64, 120, 512, 520, 1000, 1024, 1536, 2048, 2056, 3072, 4096,
                 5000, 6144, 8192]
 
@@ -172,9 +172,10 @@ def test_causal_sizes(device, s, dtype):
     check_causal(device, batches, s, dtype, 0.125, seed=s)
 
 
-@pytest.mark.parametrize("s", [12288, 16384, 33000])
+@pytest.mark.parametrize("s", [12288, 16384, 20000, 28672, 33000])
 def test_causal_very_long_rows(device, s):
-    # 8 and 16 waves per row; 33000 exceeds the register-resident limit (element-wise kernels)
+    # 16 waves per row with 2, 3 and 4 chunks per wave; 33000 exceeds the register-resident
+    # limit (element-wise kernels)
     x = scores((1, s, s), torch.bfloat16, device, s)
     y = causal_ext.forward(x, 0.05)
     rows = torch.tensor([0, 1, 511, 512, 513, s // 2, s - 2, s - 1], device=device)
@@ -322,7 +323,7 @@ def check_masked(device, b, heads, sq, sk, dtype, scale, seed, mask=None, lo=1):
 
 MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (2, 2, 16, 64), (3, 2, 9, 520),
                  (2, 2, 33, 1000), (2, 2, 8, 1024), (1, 2, 6, 2048), (1, 1, 4, 3072), (1, 2, 3, 4096),
-                 (1, 1, 3, 8192), (1, 1, 2, 20000), (1, 1, 2, 40000), (1, 3, 1, 77)]
+                 (1, 1, 3, 8192), (1, 1, 2, 12000), (1, 1, 2, 20000), (1, 1, 2, 30000), (1, 1, 2, 40000), (1, 3, 1, 77)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
