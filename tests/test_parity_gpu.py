@@ -481,6 +481,77 @@ def test_fused_rope_extension_api(device, dtype, transpose):
     assert torch.equal(out2, w2.to(dtype))
 
 
+def test_rotary_in_place_on_views_of_a_fused_qkv_buffer(device):
+    # megatron/model/transformer.py:798-809 produces [sq, b, np, 3*hn] and splits it into q, k, v
+    # views; rotating q and k in place must leave v and the pass-through dims untouched
+    s, b, h, hn, d_rot = 48, 2, 6, 64, 16
+    qkv = normal((s, b, h, 3 * hn), torch.float16, device, 77)
+    before = qkv.clone()
+    q, k, v = qkv[..., :hn], qkv[..., hn : 2 * hn], qkv[..., 2 * hn :]
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s))
+    apply_rotary_pos_emb_(q, k, cos, sin, 0, d_rot)
+    rq, rk = R.rotary_fp32(before[..., :d_rot], before[..., hn : hn + d_rot], cos, sin)
+    assert torch.equal(qkv[..., :d_rot], rq.half()) and torch.equal(qkv[..., hn : hn + d_rot], rk.half())
+    assert torch.equal(qkv[..., d_rot:hn], before[..., d_rot:hn])
+    assert torch.equal(qkv[..., hn + d_rot : 2 * hn], before[..., hn + d_rot : 2 * hn])
+    assert torch.equal(v, before[..., 2 * hn :])
+
+
+def test_rotary_in_place_autograd(device):
+    s, b, h, hn, d_rot = 16, 2, 3, 32, 16
+    q0 = normal((s, b, h, hn), torch.bfloat16, device, 1)
+    k0 = normal((s, b, h, hn), torch.bfloat16, device, 2)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s))
+    qa, ka = q0.clone().requires_grad_(True), k0.clone().requires_grad_(True)
+    oq, ok = apply_rotary_pos_emb_(qa * 1, ka * 1, cos, sin, 0, d_rot)  # in place on non-leaf copies
+    gq, gk = normal(oq.shape, torch.bfloat16, device, 3), normal(ok.shape, torch.bfloat16, device, 4)
+    torch.autograd.backward([oq, ok], [gq, gk])
+    dq, dk = R.rotary_autograd_fp32(q0[..., :d_rot], k0[..., :d_rot], cos, sin, gq[..., :d_rot], gk[..., :d_rot])
+    assert torch.equal(qa.grad[..., :d_rot], dq.bfloat16()) and torch.equal(ka.grad[..., :d_rot], dk.bfloat16())
+    assert torch.equal(qa.grad[..., d_rot:], gq[..., d_rot:]) and torch.equal(ka.grad[..., d_rot:], gk[..., d_rot:])
+
+
+def test_entry_points_can_be_captured_in_a_hip_graph(device):
+    # no allocation, no synchronisation inside the library: a captured sequence replays to the
+    # same result as the eager one, also with other work between the replays
+    lib = _lib.lib()
+    B, n = 4, 520
+    x = scores((B, n, n), torch.float16, device, 5)
+    g = normal((B, n, n), torch.float16, device, 6)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    q = normal((64, 2, 4, 64), torch.float16, device, 7)
+    k = normal((64, 2, 4, 64), torch.float16, device, 8)
+    oq, ok = torch.empty_like(q), torch.empty_like(k)
+    cos, sin = (t.to(device).reshape(64, 64).contiguous() for t in R.rotary_tables(64, 64))
+
+    def run():
+        st = torch.cuda.current_stream().cuda_stream
+        _lib.check(lib.neox_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), 0.125, B, n, n, _lib.NEOX_F16, st))
+        _lib.check(lib.neox_causal_softmax_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), 0.125, B, n, n,
+                                               _lib.NEOX_F16, st))
+        rope_ext.rope_launch(oq, ok, q, k, cos, sin, 64, 0, backward=False)
+
+    run()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in (y, dx, oq, ok)]
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()  # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            run()
+    for rep in range(3):
+        for t in (y, dx, oq, ok):
+            t.fill_(float(rep))  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip((y, dx, oq, ok), want):
+            assert torch.equal(got, ref), rep
+
+
 def test_rotary_round_trip_property(device):
     # backward is the inverse rotation: bwd(fwd(x)) == x up to two roundings
     s, b, h, d = 128, 2, 8, 64
