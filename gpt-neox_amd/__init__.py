@@ -23,6 +23,7 @@ from .positional_embeddings import (  # noqa: F401
     SinusoidalPositionalEmbedding,
     apply_rotary_pos_emb,
     apply_rotary_pos_emb_,
+    apply_rotary_pos_emb_qkv_,
     apply_rotary_pos_emb_torch,
     rotate_half,
 )
@@ -37,6 +38,7 @@ __all__ = [
     "SinusoidalPositionalEmbedding",
     "apply_rotary_pos_emb",
     "apply_rotary_pos_emb_",
+    "apply_rotary_pos_emb_qkv_",
     "apply_rotary_pos_emb_torch",
     "rotate_half",
 ]

@@ -22,7 +22,8 @@ What differs from the reference, on purpose:
 
 Other dtypes and CPU tensors evaluate the reference's torch expression.
 ``apply_rotary_pos_emb_`` is an in-place variant over whole heads (partial
-rotary without the slice/concatenate round trip).
+rotary without the slice/concatenate round trip) and ``apply_rotary_pos_emb_qkv_``
+does the same directly on the fused QKV projection of the attention layer.
 """
 import math
 
@@ -247,6 +248,62 @@ def apply_rotary_pos_emb_(q, k, cos, sin, offset: int = 0, rotary_ndims=None):
     if d_rot > q.shape[-1] or d_rot % 2:
         raise RuntimeError(f"rotary_ndims={d_rot} must be even and <= head size {q.shape[-1]}")
     return _FusedRotaryInplace.apply(q, k, cos.to(q.device), sin.to(q.device), offset, d_rot)
+
+
+class _FusedQKVRotary(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, mixed, cos, sin, offset, d_rot):
+        hn = mixed.shape[-1] // 3
+        cos2 = _as_table(cos, d_rot, offset + mixed.shape[0])
+        sin2 = _as_table(sin, d_rot, offset + mixed.shape[0])
+        if mixed.numel():
+            q, k = mixed[..., :hn], mixed[..., hn : 2 * hn]
+            _rope_ext.rope_launch(q, k, q, k, cos2, sin2, d_rot, offset, backward=False)
+        ctx.mark_dirty(mixed)
+        ctx.save_for_backward(cos2, sin2)
+        ctx.offset, ctx.d_rot, ctx.hn = offset, d_rot, hn
+        return mixed
+
+    @staticmethod
+    def backward(ctx, grad_mixed):
+        cos2, sin2 = ctx.saved_tensors
+        dm = grad_mixed.clone(memory_format=torch.contiguous_format)  # v and pass-through dims: identity
+        if dm.numel():
+            dq, dk = dm[..., : ctx.hn], dm[..., ctx.hn : 2 * ctx.hn]
+            _rope_ext.rope_launch(dq, dk, dq, dk, cos2, sin2, ctx.d_rot, ctx.offset, backward=True)
+        return dm, None, None, None, None
+
+
+def apply_rotary_pos_emb_qkv_(mixed_x_layer, cos, sin, offset: int = 0, rotary_ndims=None):
+    """Rotary at the call site of the attention layer, without its slice / concatenate copies.
+
+    ``mixed_x_layer`` is the fused projection ``[sq, b, np, 3*hn]``
+    (megatron/model/transformer.py:798-809).  The q and k thirds are rotated in place over
+    their first ``rotary_ndims`` dims (all ``hn`` when None) in one launch; v and the
+    pass-through dims are not touched.  Returns the views ``(query, key, value)``, each
+    ``[sq, b, np, hn]`` -- what megatron/model/transformer.py:807-860 produces with two
+    ``torch.cat`` and four slices.  Differentiable with respect to ``mixed_x_layer``.
+    """
+    if mixed_x_layer.dim() != 4 or mixed_x_layer.shape[-1] % 3:
+        raise RuntimeError("mixed_x_layer must be [sq, b, np, 3*hn]")
+    hn = mixed_x_layer.shape[-1] // 3
+    d_rot = hn if rotary_ndims is None else int(rotary_ndims)
+    if d_rot > hn or d_rot % 2:
+        raise RuntimeError(f"rotary_ndims={d_rot} must be even and <= head size {hn}")
+    if (
+        not mixed_x_layer.is_cuda
+        or mixed_x_layer.dtype not in _HALF
+        or mixed_x_layer.stride(-1) != 1
+        or cos.dtype != sin.dtype
+        or cos.dtype not in (torch.float32, mixed_x_layer.dtype)
+    ):
+        raise RuntimeError(
+            "apply_rotary_pos_emb_qkv_ needs an fp16/bf16 GPU tensor with a dense last dim and "
+            "cos/sin in fp32 or its dtype"
+        )
+    dev = mixed_x_layer.device
+    mixed = _FusedQKVRotary.apply(mixed_x_layer, cos.to(dev), sin.to(dev), offset, d_rot)
+    return mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]
 
 
 class AliBi(torch.nn.Module):

@@ -27,6 +27,7 @@ from gpt_neox_amd.positional_embeddings import (
     RotaryEmbedding,
     apply_rotary_pos_emb,
     apply_rotary_pos_emb_,
+    apply_rotary_pos_emb_qkv_,
     apply_rotary_pos_emb_torch,
 )
 from oracle import torch_ref as R
@@ -495,6 +496,37 @@ def test_rotary_in_place_on_views_of_a_fused_qkv_buffer(device):
     assert torch.equal(qkv[..., d_rot:hn], before[..., d_rot:hn])
     assert torch.equal(qkv[..., hn + d_rot : 2 * hn], before[..., hn + d_rot : 2 * hn])
     assert torch.equal(v, before[..., 2 * hn :])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rotary_ndims,offset", [(None, 0), (16, 0), (32, 3)])
+def test_rotary_call_site_fusion_matches_slice_rotate_concatenate(device, dtype, rotary_ndims, offset):
+    # the sequence of megatron/model/transformer.py:807-860 on a fused projection, against
+    # one in-place launch; forward values and the gradient of the projection output
+    s, b, h, hn = 24, 2, 4, 64
+    d_rot = hn if rotary_ndims is None else rotary_ndims
+    w = normal((s, b, h, 3 * hn), dtype, device, 11)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + offset))
+
+    def reference(mixed):  # fp32 arithmetic, rounded once where the kernels round
+        q, k, v = mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]
+        oq, ok = R.partial_rotary(q, k, cos, sin, d_rot, offset)
+        return oq, ok, v
+
+    wr = w.detach().float().requires_grad_(True)
+    rq, rk, rv = reference(wr * 1.0)
+    wf = w.detach().clone().requires_grad_(True)
+    fq, fk, fv = apply_rotary_pos_emb_qkv_(wf * 1, cos, sin, offset, rotary_ndims)
+    assert fq.shape == (s, b, h, hn) and fq.data_ptr() + 2 * hn == fk.data_ptr()  # views of one buffer
+    assert torch.equal(fq, rq.to(dtype)) and torch.equal(fk, rk.to(dtype)) and torch.equal(fv, rv.to(dtype))
+    gq, gk, gv = (normal((s, b, h, hn), dtype, device, 20 + i) for i in range(3))
+    torch.autograd.backward([rq, rk, rv], [gq.float(), gk.float(), gv.float()])
+    torch.autograd.backward([fq, fk, fv], [gq, gk, gv])
+    assert torch.equal(wf.grad, wr.grad.to(dtype))
+    with torch.no_grad():  # inference: same values, really in place
+        buf = w.clone()
+        q2, k2, v2 = apply_rotary_pos_emb_qkv_(buf, cos, sin, offset, rotary_ndims)
+        assert q2.data_ptr() == buf.data_ptr() and torch.equal(q2, fq) and torch.equal(k2, fk)
 
 
 def test_rotary_in_place_autograd(device):
