@@ -19,6 +19,12 @@ Deliberate differences from the reference:
   runs the torch path beyond it) and need none of the ``sq % 4``,
   ``attn_batches % 4`` or ``% batch_per_block`` divisibility rules, which were
   artefacts of the CUDA launch shape -- see :meth:`is_kernel_available`;
+* the causal branch checks once per mask tensor that the mask really is the plain
+  upper-triangular one and otherwise (sliding-window masks, packed-sequence masks)
+  runs the mask-tensor kernel with the mask it was given -- the reference's causal
+  kernel ignores the mask's contents, so above its 2048 limit (torch path) and below
+  it (fused kernel) the reference computes two different things for such masks; here
+  both agree with the torch path;
 * masked scores are excluded, so their probability is exactly 0 as in the torch
   path (the reference's padded kernel fills -10000), and a fully masked row is
   uniform ``1/sk`` as in the torch path;
@@ -26,6 +32,7 @@ Deliberate differences from the reference:
 * a missing kernel library raises ``ImportError`` instead of calling ``exit()``.
 """
 import enum
+import weakref
 
 import torch
 
@@ -49,6 +56,42 @@ def _scale_tensor(scale):
 def _recall(ctx):
     probs, scale_t = ctx.saved_tensors
     return probs, scale_t[0].item()
+
+
+class _CausalMaskMemo:
+    """Remembers, per live mask tensor, whether it equals ``triu(ones, 1)``.
+
+    The verdict costs one pass over the mask and one host synchronisation; the attention
+    mask of a training step is one tensor shared by all layers, so it is paid once per
+    step.  Entries are keyed by the tensor object (weak reference) and its version
+    counter, never by address, so a recycled allocation cannot inherit a verdict."""
+
+    def __init__(self, limit=16):
+        self._entries = {}
+        self._limit = limit
+
+    def is_plain_causal(self, mask):
+        key = id(mask)
+        hit = self._entries.get(key)
+        if hit is not None:
+            ref, version, verdict = hit
+            if ref() is mask and version == mask._version:
+                return verdict
+        sq, sk = mask.shape[-2], mask.shape[-1]
+        cols = torch.arange(sk, device=mask.device)
+        rows = torch.arange(sq, device=mask.device)
+        expected = cols[None, :] > rows[:, None]
+        verdict = bool(torch.equal(mask.bool().expand(mask.shape[0], 1, sq, sk),
+                                   expected.expand(mask.shape[0], 1, sq, sk)))
+        if len(self._entries) >= self._limit:
+            self._entries = {k: v for k, v in self._entries.items() if v[0]() is not None}
+            if len(self._entries) >= self._limit:
+                self._entries.clear()
+        self._entries[key] = (weakref.ref(mask), mask._version, verdict)
+        return verdict
+
+
+_causal_memo = _CausalMaskMemo()
 
 
 class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
@@ -161,10 +204,24 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         scale = 1.0 if self.scale is None else self.scale
         if not self.upper_triang_mask_fusion:
             return ScaledMaskedSoftmax.apply(input, mask, scale)
-        # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
         assert sq == sk, "causal mask is only for self attention"
+        if not self.mask_is_plain_causal(mask):
+            # e.g. a sliding-window mask: what the torch path computes, from the mask itself
+            return ScaledMaskedSoftmax.apply(input, mask, scale)
+        # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
         probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
         return probs.view(b, np, sq, sk)
+
+    @staticmethod
+    def mask_is_plain_causal(mask):
+        """True if ``mask`` hides exactly the keys ``j > i``.  Decided once per mask tensor
+        (see ``_CausalMaskMemo``); while a HIP graph is being captured the check cannot
+        synchronise, so the answer is False and the mask-tensor kernel is used."""
+        if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
+            return False
+        if mask.is_cuda and torch.cuda.is_current_stream_capturing():
+            return False
+        return _causal_memo.is_plain_causal(mask)
 
     def forward_torch_softmax(self, input, mask):
         """The unfused path: optional upcast, scale, ``mask_func``, softmax, cast back."""

@@ -204,6 +204,24 @@ def test_is_kernel_available_table():
     assert not general.is_kernel_available(mask, 0, 12, 64, 64)  # empty
 
 
+def test_plain_causal_mask_detection_and_memo():
+    from oracle import torch_ref as R
+
+    f = FusedScaleMaskSoftmax.mask_is_plain_causal
+    plain = R.get_attn_mask(9)
+    assert f(plain) and f(plain)
+    assert f(plain.expand(3, 1, 9, 9).contiguous()) and f(plain.to(torch.uint8))
+    assert not f(R.get_attn_mask(9, sliding_window_width=2))
+    assert not f(torch.zeros(1, 1, 9, 9, dtype=torch.bool))
+    assert not f(plain[0])  # not 4-D
+    per_sample = plain.expand(2, 1, 9, 9).clone()
+    assert f(per_sample)
+    per_sample[1, 0, 8, 0] = True  # version bump: the remembered verdict is dropped
+    assert not f(per_sample)
+    for _ in range(40):  # the memo stays bounded and correct under churn
+        assert f(R.get_attn_mask(5))
+
+
 def test_reference_predicate_restated():
     # megatron/model/fused_softmax.py:148-168 with wave64 batch_per_block (= 2 for sk > 128)
     ref = FusedScaleMaskSoftmax.reference_is_kernel_available

@@ -283,13 +283,26 @@ def test_causal_autograd_function_and_module(device):
         assert torch.equal(f1(x, mask), ScaledUpperTriangMaskedSoftmax.apply(x.view(-1, s, s), 1.0).view_as(x))
 
 
-def test_causal_module_ignores_mask_contents_like_the_reference(device):
-    # megatron/model/fused_softmax.py:173-179: the causal branch never reads the mask
-    x = scores((1, 2, 40, 40), torch.float16, device, 4)
-    fused = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang, None, True, None)
-    a = fused(x, R.get_attn_mask(40, device))
-    b = fused(x, R.get_attn_mask(40, device, sliding_window_width=3))
-    assert torch.equal(a, b)
+def test_causal_module_honours_masks_that_are_not_plain_causal(device):
+    # a sliding-window mask (megatron/utils.py:75-77) given to the causal-fusion module: the
+    # result is what the torch path computes from that mask, at any length -- the reference's
+    # causal kernel would ignore the window below 2048 and apply it (torch path) above
+    for s, dtype, fp16, bf16 in ((40, torch.float16, True, False), (2560, torch.bfloat16, False, True)):
+        x = scores((1, 2, s, s), dtype, device, 4)
+        fused = FusedScaleMaskSoftmax(fp16, bf16, SoftmaxFusionTypes.upper_triang,
+                                      R.gpt2_attention_mask_func, True, 0.25)
+        plain = R.get_attn_mask(s, device)
+        window = R.get_attn_mask(s, device, sliding_window_width=3)
+        assert fused.mask_is_plain_causal(plain) and not fused.mask_is_plain_causal(window)
+        assert fused.mask_is_plain_causal(plain)  # remembered verdict
+        a, b = fused(x, plain), fused(x, window)
+        assert max_err(a, R.softmax_fp32(x, plain, 0.25)) <= TOL[dtype]
+        assert max_err(b, R.softmax_fp32(x, window, 0.25)) <= TOL[dtype]
+        assert (b[window.expand_as(b)] == 0).all() and not torch.equal(a, b)
+        # an in-place edit of a remembered mask is noticed
+        plain[0, 0, s - 1, 0] = True
+        assert not fused.mask_is_plain_causal(plain)
+        assert max_err(fused(x, plain), R.softmax_fp32(x, plain, 0.25)) <= TOL[dtype]
 
 
 def test_causal_decode_step_takes_the_torch_branch(device):
