@@ -142,6 +142,8 @@ int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float s
     a.sk = sk;
     a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
     a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
+    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
     const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(mask, 8);
     return check_launch(launch_softmax_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
 }

@@ -4,7 +4,8 @@
 // wave that holds 2 chunks (1024 columns) is the sweet spot at every row length -- 4 chunks
 // per wave cost 3-5 % of bandwidth, 1 chunk per wave 10-20 % -- so a row gets
 // ceil(chunks / 2) waves:
-//   chunks <= 2    1 wave per row, 4 rows per 256-thread block      (sk <= 1024)
+//   chunks == 1    several rows per wave (packed kernels)            (sk <= 512)
+//   chunks == 2    1 wave per row, 4 rows per 256-thread block      (sk <= 1024)
 //   chunks <= 4    2 waves per row, 2 rows per block                 (sk <= 2048)
 //   chunks <= 8    4 waves per row                                   (sk <= 4096)
 //   chunks <= 16   8 waves per row, 512-thread block                 (sk <= 8192)
@@ -40,11 +41,44 @@ static hipError_t launch_generic(const SoftmaxArgs& a, hipStream_t st) {
     return hipGetLastError();
 }
 
+template <typename T, Mask M, bool BWD, int G>
+static hipError_t launch_packed(const SoftmaxArgs& a, hipStream_t st) {
+    // passes per wave: 4 everywhere except the causal forward of the longer packed rows,
+    // which measured 15 % faster with 2
+    constexpr int R = (!BWD && M == Mask::Causal && G >= 32) ? 2 : kPackedPasses;
+    const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
+    const dim3 grid((a.rows + per_block - 1) / per_block);
+    if constexpr (BWD) {
+        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, kDefaultFlags, R>), grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags, R>), grid, dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
+}
+
+// sk <= 512: lane groups of G = pow2 >= sk/8 lanes per row
+template <typename T, Mask M, bool BWD>
+static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
+    const int lanes = (a.sk + kVec - 1) / kVec;
+    if (lanes <= 1) return launch_packed<T, M, BWD, 1>(a, st);
+    if (lanes <= 2) return launch_packed<T, M, BWD, 2>(a, st);
+    if (lanes <= 4) return launch_packed<T, M, BWD, 4>(a, st);
+    if (lanes <= 8) return launch_packed<T, M, BWD, 8>(a, st);
+    if (lanes <= 16) return launch_packed<T, M, BWD, 16>(a, st);
+    if (lanes <= 32) return launch_packed<T, M, BWD, 32>(a, st);
+    return launch_packed<T, M, BWD, 64>(a, st);
+}
+
 template <typename T, Mask M, bool BWD>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     const int chunks = (a.sk + kChunk - 1) / kChunk;
     if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD>(a, st);
-    if (chunks == 1) return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
+    if (chunks == 1) {
+        // the forward mask kernel addresses the mask through one 32-bit-sized buffer
+        const bool mask_ok = BWD || M != Mask::Bytes || a.mask_bytes != 0;
+        if (mask_ok) return dispatch_packed<T, M, BWD>(a, st);
+        return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
+    }
     if (chunks == 2) return launch_shape<T, M, BWD, 2, 1, 4>(a, st);
     if (chunks <= 4) return launch_shape<T, M, BWD, 2, 2, 2>(a, st);
     if (chunks <= 8) return launch_shape<T, M, BWD, 2, 4, 1>(a, st);

@@ -32,6 +32,7 @@ struct SoftmaxArgs {
     int32_t sk;
     uint32_t rows_per_mask_batch;  // np*sq: rows sharing one mask sample
     int32_t mask_bcast;            // mask batch dim is 1
+    uint32_t mask_bytes;           // size of the mask tensor, 0 if it does not fit 32 bits
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -70,10 +71,10 @@ __device__ __forceinline__ float row_combine(float v, float* red, int wib, int r
     } else {
         if (lane == 0) red[wib] = v;
         __syncthreads();
-        float r = red[rib * WPR];
+        typename Op::type r = Op::enc(red[rib * WPR]);
 #pragma unroll
-        for (int w = 1; w < WPR; ++w) r = Op::f(r, red[rib * WPR + w]);
-        return r;
+        for (int w = 1; w < WPR; ++w) r = Op::f(r, Op::enc(red[rib * WPR + w]));
+        return Op::dec(r);
     }
 }
 
@@ -158,23 +159,32 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         mx = wave_reduce<OpMax>(mx);
         mx = row_combine<OpMax, WPR, RPB>(mx, red_max, wib, rib, lane);
 
-        // A row whose every key is masked: the unfused path fills all scores with the same
-        // value, so the result is uniform over the sk columns.
-        const bool all_masked = (mx == ninf);
-
         // ---- exponentials and their sum
         float sum = 0.f;
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             if (c0 < len) {
-                const int col = c0 + lane * kVec;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    float e = fast_exp2(v[c][k] - mx);
-                    if (all_masked) e = ((col + k) < len) ? 1.f : 0.f;
-                    v[c][k] = e;
-                    sum += e;
+                    v[c][k] = fast_exp2(v[c][k] - mx);
+                    sum += v[c][k];
+                }
+            }
+        }
+        if constexpr (MASK == Mask::Bytes) {
+            // A row whose every key is masked (row-uniform, rare): the unfused path fills all
+            // scores with the same value, so the result is uniform over the sk columns.
+            if (mx == ninf) {
+                sum = 0.f;
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    const int col = (wir + WPR * c) * kChunk + lane * kVec;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        v[c][k] = ((col + k) < len) ? 1.f : 0.f;
+                        sum += v[c][k];
+                    }
                 }
             }
         }
@@ -277,6 +287,169 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
 }
 
 // ---------------------------------------------------------------------------------
+// Short rows (sk <= 512): several rows per wave.
+//
+// A row is owned by an aligned group of G consecutive lanes (G = 64 for sk in (256, 512],
+// 32 for (128, 256], ... 1 for sk = 8), each lane holding 8 columns; a wave covers
+// 64/G rows per pass and makes R passes, so it always has a few KiB in flight however
+// short the rows are (one row per wave caps out at ~3.6 G rows/s).  Rows of a wave are
+// consecutive in memory; its loads and stores go through one buffer resource spanning
+// just those rows, with out-of-range offsets for the lanes that have nothing to fetch.
+// No LDS, no barriers: reductions stay inside the lane group.
+// ---------------------------------------------------------------------------------
+constexpr int kPackedPasses = 4;  // default number of passes R
+constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;
+
+// (i0 + lr) mod sq for lr below the rows of a wave: one conditional subtraction when a
+// matrix has at least that many rows, a division only for tiny matrices.
+__device__ __forceinline__ uint32_t wrap_row(uint32_t i, uint32_t sq) {
+    if (sq >= 256u) return i >= sq ? i - sq : i;  // wave-uniform branch; rows per wave <= 256
+    return i % sq;
+}
+
+template <int G, int R = kPackedPasses>
+struct Packed {
+    static constexpr int kRowsPerPass = kWave / G;
+    static constexpr int kRowsPerWave = kRowsPerPass * R;
+    static constexpr int kRowsPerBlock = kRowsPerWave * 4;  // 256-thread blocks
+};
+
+template <typename T, int G, Mask MASK, int FLAGS = kDefaultFlags, int R = kPackedPasses>
+__global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) {
+    constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
+    constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t row0 = wave * RPW;  // first row of this wave
+    if (row0 >= a.rows) return;
+    const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
+    const int sk = a.sk;
+    const int grp = lane / G;
+    const int col = (lane % G) * kVec;
+    const float ninf = -__builtin_inff();
+
+    const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+    const rsrc_t ry = make_rsrc(static_cast<char*>(a.out) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+    const rsrc_t rm = make_rsrc(a.mask, a.mask_bytes);
+
+    u32x4 raw[R];
+    u32x2 mk[R];
+    int len[R];
+    uint32_t off[R];
+    const uint32_t i0 = row0 % (uint32_t)a.sq;  // wave-uniform
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const uint32_t lr = p * RPP + grp;  // row of this lane group inside the wave
+        const uint32_t row = row0 + lr;
+        const uint32_t i = wrap_row(i0 + lr, (uint32_t)a.sq);
+        len[p] = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+        if (lr >= rows_here) len[p] = 0;
+        off[p] = (lr * sk + col) * 2u;
+        raw[p] = buf_ld128<kLdNt>(rx, col < len[p] ? off[p] : kOutOfRange, 0);
+        if constexpr (MASK == Mask::Bytes) {
+            const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
+            const uint32_t moff = (mb * (uint32_t)a.sq + i) * sk + col;
+            mk[p] = buf_ld64(rm, col < len[p] ? moff : kOutOfRange, 0);
+        }
+    }
+
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        float v[8];
+        unpack8<T>(raw[p], v);
+        float mx = ninf;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            bool keep = (col + k) < len[p];
+            if constexpr (MASK == Mask::Bytes) {
+                const uint32_t w = (k < 4) ? mk[p].x : mk[p].y;
+                keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
+            }
+            v[k] = keep ? v[k] * a.scale : ninf;
+            mx = fmaxf(mx, v[k]);
+        }
+        mx = group_reduce<OpMax, G>(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            v[k] = fast_exp2(v[k] - mx);
+            sum += v[k];
+        }
+        if constexpr (MASK == Mask::Bytes) {
+            // rows with every key hidden (rare): uniform over the sk columns
+            const bool all_masked = (mx == ninf) && len[p] > 0;
+            if (__builtin_amdgcn_ballot_w64(all_masked) != 0) {
+                if (all_masked) {
+                    sum = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        v[k] = ((col + k) < len[p]) ? 1.f : 0.f;
+                        sum += v[k];
+                    }
+                }
+            }
+        }
+        sum = group_reduce<OpSum, G>(sum);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] *= inv;  // lanes of absent rows hold NaN and store nothing
+        const bool st = (p * RPP + grp) < (int)rows_here && col < sk;
+        buf_st128<kStNt>(ry, pack8<T>(v), st ? off[p] : kOutOfRange, 0);
+    }
+}
+
+template <typename T, int G, Mask MASK, int FLAGS = kDefaultFlags, int R = kPackedPasses>
+__global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) {
+    constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
+    constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t row0 = wave * RPW;
+    if (row0 >= a.rows) return;
+    const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
+    const int sk = a.sk;
+    const int grp = lane / G;
+    const int col = (lane % G) * kVec;
+
+    const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+    const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+    const rsrc_t bo = make_rsrc(static_cast<char*>(a.out) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+
+    u32x4 rg[R], rp[R];
+    int len[R];
+    uint32_t off[R];
+    const uint32_t i0 = row0 % (uint32_t)a.sq;  // wave-uniform
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const uint32_t lr = p * RPP + grp;
+        const uint32_t i = wrap_row(i0 + lr, (uint32_t)a.sq);
+        len[p] = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
+        if (lr >= rows_here) len[p] = 0;
+        off[p] = (lr * sk + col) * 2u;
+        const uint32_t o = col < len[p] ? off[p] : kOutOfRange;
+        rg[p] = buf_ld128<kLdNt>(bg, o, 0);
+        rp[p] = buf_ld128<kLdNt>(by, o, 0);
+    }
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        float gv[8], pv[8];
+        unpack8<T>(rg[p], gv);
+        unpack8<T>(rp[p], pv);
+        float dot = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            if ((col + k) >= len[p]) pv[k] = 0.f;  // past the diagonal / row end
+            dot = fmaf(gv[k], pv[k], dot);
+        }
+        dot = group_reduce<OpSum, G>(dot);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) gv[k] = a.scale * (pv[k] * (gv[k] - dot));
+        const bool st = (p * RPP + grp) < (int)rows_here && col < sk;
+        buf_st128<kStNt>(bo, pack8<T>(gv), st ? off[p] : kOutOfRange, 0);
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // Any-shape kernels: one 256-thread block per row, element-wise accesses, the row
 // is re-read for each pass (from L2).  Used when sk is not a multiple of 8, a
 // pointer is not 16-byte aligned, or the row exceeds the register-resident limit.
@@ -291,10 +464,10 @@ __device__ __forceinline__ float block_reduce(float v, float* red) {
     __syncthreads();  // red may still be read from the previous reduction
     if (lane == 0) red[wib] = v;
     __syncthreads();
-    float r = red[0];
+    typename Op::type r = Op::enc(red[0]);
 #pragma unroll
-    for (int w = 1; w < kGenericThreads / kWave; ++w) r = Op::f(r, red[w]);
-    return r;
+    for (int w = 1; w < kGenericThreads / kWave; ++w) r = Op::f(r, Op::enc(red[w]));
+    return Op::dec(r);
 }
 
 template <typename T, Mask MASK>

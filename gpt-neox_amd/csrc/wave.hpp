@@ -136,41 +136,68 @@ constexpr int kDppQuadSwap1 = 0xB1;    // quad_perm:[1,0,3,2]
 constexpr int kDppQuadSwap2 = 0x4E;    // quad_perm:[2,3,0,1]
 constexpr int kDppRowHalfMirror = 0x141;
 constexpr int kDppRowMirror = 0x140;
+constexpr int kSwizzleXor16 = 0x401F;  // ds_swizzle bit mode: and 0x1f, or 0, xor 0x10
 
-template <int Ctrl>
-__device__ __forceinline__ float dpp(float v) {
-    int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, false);
-    return __builtin_bit_cast(float, r);
-}
-
-__device__ __forceinline__ float lane_read(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-
-struct OpMax {
-    static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
-};
 struct OpSum {
+    typedef float type;
     static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+    static __device__ __forceinline__ float enc(float v) { return v; }
+    static __device__ __forceinline__ float dec(float v) { return v; }
+};
+// Maximum of floats taken on order-preserving integer keys (sign-magnitude -> two's
+// complement): v_max_i32 needs no NaN canonicalisation of the shuffled operand, so each
+// step is a single DPP instruction.  -inf and finite values order as floats do.
+struct OpMax {
+    typedef int type;
+    static __device__ __forceinline__ int f(int a, int b) { return a > b ? a : b; }
+    static __device__ __forceinline__ int enc(float v) {
+        const int b = __builtin_bit_cast(int, v);
+        return b ^ ((b >> 31) & 0x7fffffff);
+    }
+    static __device__ __forceinline__ float dec(int k) {
+        return __builtin_bit_cast(float, k ^ ((k >> 31) & 0x7fffffff));
+    }
 };
 
-// Reduce across each DPP row (16 consecutive lanes); every lane of the row gets the result.
-template <typename Op>
-__device__ __forceinline__ float row16_reduce(float v) {
-    v = Op::f(v, dpp<kDppQuadSwap1>(v));
-    v = Op::f(v, dpp<kDppQuadSwap2>(v));
-    v = Op::f(v, dpp<kDppRowHalfMirror>(v));
-    v = Op::f(v, dpp<kDppRowMirror>(v));
-    return v;
+template <int Ctrl, typename V>
+__device__ __forceinline__ V dpp(V v) {
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Ctrl, 0xF, 0xF, false);
+    return __builtin_bit_cast(V, r);
+}
+template <typename V>
+__device__ __forceinline__ V lane_read(V v, int lane) {
+    return __builtin_bit_cast(V, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Reduce across aligned groups of G consecutive lanes (G a power of two); every lane of a
+// group gets the group's result.  Steps of 1..8 lanes are DPP operations, 16 is a
+// ds_swizzle (no LDS memory is touched), the last step of a full wave reads four lanes.
+// Must be called with all 64 lanes active.
+template <typename Op, int G>
+__device__ __forceinline__ float group_reduce(float x) {
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "group size");
+    typedef typename Op::type V;
+    V v = Op::enc(x);
+    if constexpr (G >= 2) v = Op::f(v, dpp<kDppQuadSwap1>(v));
+    if constexpr (G >= 4) v = Op::f(v, dpp<kDppQuadSwap2>(v));
+    if constexpr (G >= 8) v = Op::f(v, dpp<kDppRowHalfMirror>(v));
+    if constexpr (G >= 16) v = Op::f(v, dpp<kDppRowMirror>(v));
+    if constexpr (G == 32) {
+        const int o = __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), kSwizzleXor16);
+        v = Op::f(v, __builtin_bit_cast(V, o));
+    }
+    if constexpr (G == 64) {
+        const V a = Op::f(lane_read(v, 0), lane_read(v, 16));
+        const V b = Op::f(lane_read(v, 32), lane_read(v, 48));
+        v = Op::f(a, b);
+    }
+    return Op::dec(v);
 }
 
 // Reduce across the whole wave; the result is wave-uniform.
 template <typename Op>
 __device__ __forceinline__ float wave_reduce(float v) {
-    v = row16_reduce<Op>(v);
-    float a = Op::f(lane_read(v, 0), lane_read(v, 16));
-    float b = Op::f(lane_read(v, 32), lane_read(v, 48));
-    return Op::f(a, b);
+    return group_reduce<Op, kWave>(v);
 }
 
 constexpr float kLog2e = 1.4426950408889634f;

@@ -162,7 +162,7 @@ def check_causal(device, batches, s, dtype, scale, seed, chunk=4):
 # row lengths chosen to hit: 1 column; lanes partly filled; not a multiple of 8 (element-wise
 # kernels); 1 and 2 chunks of 512 columns on one wave; the 2-, 4- and 8-wave kernels with rows
 # that fill their last chunk exactly, partly, or leave whole chunks of a wave empty.
-CAUSAL_SIZES = [1, 2, 7, 8, 16, 37, 64, 120, 512, 520, 1000, 1024, 1536, 2048, 2056, 3072, 4096,
+CAUSAL_SIZES = [1, 2, 7, 8, 16, 24, 37, 40, 64, 72, 120, 128, 200, 256, 264, 384, 504, 512, 520, 1000, 1024, 1536, 2048, 2056, 3072, 4096,
                 5000, 6144, 8192]
 
 
@@ -219,6 +219,26 @@ def test_nothing_is_written_past_the_end_of_the_output(device, s):
             want = masked_ext.forward(x.view(1, 2, s, s), mask, 0.125)
         assert torch.equal(out[:n].view(2, s, s), want.view(2, s, s))
         assert (out[n:] == 7.0).all() and (dxo[n:] == 7.0).all(), kind
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_short_rows_packed_several_per_wave(device, dtype):
+    # sk <= 512 packs 64/G rows into a wave (G lanes per row): row counts that do not fill the
+    # last wave / block, fully masked rows inside a packed wave, per-sample masks, in-place
+    for batches, s in ((1, 8), (5, 8), (7, 16), (3, 24), (9, 40), (2, 136), (3, 264), (1, 512)):
+        check_causal(device, batches, s, dtype, 0.3, seed=batches * 1000 + s)
+    b, heads, sq, sk = 3, 2, 21, 48
+    pattern = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, 3)) < 0.4
+    pattern[1, 0, 5, :] = True
+    pattern[2, 0, 20, :] = True
+    x, mask, y, g, dx = check_masked(device, b, heads, sq, sk, dtype, 0.2, 9, mask=pattern)
+    assert torch.allclose(y[1, :, 5, :].float(), torch.full((heads, sk), 1.0 / sk, device=device), atol=2e-4)
+    check_masked(device, b, heads, sq, sk, dtype, 0.2, 10, mask=pattern[:1].contiguous())
+    x2 = x.clone()
+    _lib.check(_lib.lib().neox_masked_softmax_fwd(x2.data_ptr(), x2.data_ptr(), mask.data_ptr(), 0.2, b, heads,
+                                                  sq, sk, b, _lib.dtype_code(dtype),
+                                                  torch.cuda.current_stream().cuda_stream))
+    assert torch.equal(x2, y)
 
 
 def test_causal_negative_and_large_scale(device):
@@ -335,7 +355,8 @@ def check_masked(device, b, heads, sq, sk, dtype, scale, seed, mask=None, lo=1):
     return x, mask, y, g, dx
 
 
-MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (2, 2, 16, 64), (3, 2, 9, 520),
+MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (3, 5, 7, 8), (2, 3, 5, 16), (2, 2, 33, 24), (2, 2, 16, 64),
+                 (3, 3, 50, 72), (2, 2, 31, 128), (2, 3, 17, 200), (2, 2, 65, 256), (1, 3, 129, 384), (2, 2, 9, 512), (3, 2, 9, 520),
                  (2, 2, 33, 1000), (2, 2, 8, 1024), (1, 2, 6, 2048), (1, 1, 4, 3072), (1, 2, 3, 4096),
                  (1, 1, 3, 8192), (1, 1, 2, 12000), (1, 1, 2, 20000), (1, 1, 2, 30000), (1, 1, 2, 40000), (1, 3, 1, 77)]
 
