@@ -100,6 +100,29 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     assert lib.neox_copy_bytes(None, p, 32, None) == -1
 
 
+def test_last_error_is_kept_per_thread():
+    import threading
+
+    lib = _lib.lib()
+    seen = {}
+
+    def worker(name, bad_sk):
+        buf = ctypes.create_string_buffer(64)
+        p = (ctypes.addressof(buf) + 15) & ~15
+        for _ in range(200):
+            assert lib.neox_masked_softmax_bwd(p, p, p, 1.0, 4, bad_sk, _lib.NEOX_F16, None) == -3
+            msg = lib.neox_fused_last_error().decode()
+            assert f"sk={bad_sk}" in msg, msg
+        seen[name] = True
+
+    threads = [threading.Thread(target=worker, args=(i, -1 - i)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert len(seen) == 4
+
+
 def test_get_batch_per_block_matches_the_reference_formula_on_wave64():
     # megatron/fused_kernels/scaled_masked_softmax.h:338-352 with a 64-wide wavefront:
     # wave = min(pow2(sk), 64); rows/wave = 2 if pow2(sk) <= 128 else 1; waves/block = 128/wave

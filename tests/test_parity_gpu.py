@@ -241,6 +241,31 @@ def test_short_rows_packed_several_per_wave(device, dtype):
     assert torch.equal(x2, y)
 
 
+def test_seeded_random_shapes_around_every_dispatch_boundary(device):
+    # row lengths next to each kernel-shape boundary (8 lanes-per-row steps, 512, 1024, 2048,
+    # 4096, 8192) and odd row counts, both storage types, both mask kinds, forward + backward
+    import random
+
+    rnd = random.Random(20240611)
+    edges = [8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192]
+    for case in range(40):
+        edge = rnd.choice(edges)
+        sk = max(8, edge + 8 * rnd.choice([-2, -1, 0, 0, 1, 2]))
+        dtype = rnd.choice(DTYPES)
+        scale = rnd.choice([0.125, 0.5, 1.0, 2.0])
+        if rnd.random() < 0.5:
+            batches = rnd.randint(1, 3) if sk <= 2064 else 1
+            check_causal(device, batches, sk, dtype, scale, seed=case, chunk=1)
+        else:
+            b, heads = rnd.randint(1, 3), rnd.randint(1, 3)
+            sq = rnd.randint(1, 70) if sk <= 1040 else rnd.randint(1, 9)
+            mask = None
+            if rnd.random() < 0.5:
+                mb = rnd.choice([1, b])
+                mask = torch.rand(mb, 1, sq, sk, device=device, generator=gen(device, case)) < rnd.random()
+            check_masked(device, b, heads, sq, sk, dtype, scale, seed=case, mask=mask)
+
+
 def test_causal_negative_and_large_scale(device):
     for scale in (-0.25, 4.0, 1.0):
         check_causal(device, 2, 96, torch.float16, scale, seed=3)
