@@ -5,6 +5,7 @@
 // per wave cost 3-5 % of bandwidth, 1 chunk per wave 10-20 % -- so a row gets
 // ceil(chunks / 2) waves:
 //   chunks == 1    several rows per wave (packed kernels)            (sk <= 512)
+//   chunks <= 4    full-row backward only: packed kernel, one wave per row, R x C = 4
 //   chunks == 2    1 wave per row, 4 rows per 256-thread block      (sk <= 1024)
 //   chunks <= 4    2 waves per row, 2 rows per block                 (sk <= 2048)
 //   chunks <= 8    4 waves per row                                   (sk <= 4096)
@@ -41,19 +42,24 @@ static hipError_t launch_generic(const SoftmaxArgs& a, hipStream_t st) {
     return hipGetLastError();
 }
 
+template <typename T, Mask M, bool BWD, int G, int R, int C>
+static hipError_t launch_packed_shape(const SoftmaxArgs& a, hipStream_t st) {
+    const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
+    const dim3 grid((a.rows + per_block - 1) / per_block);
+    if constexpr (BWD) {
+        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
+}
+
 template <typename T, Mask M, bool BWD, int G>
 static hipError_t launch_packed(const SoftmaxArgs& a, hipStream_t st) {
     // passes per wave: 4 everywhere except the causal forward of the longer packed rows,
     // which measured 15 % faster with 2
     constexpr int R = (!BWD && M == Mask::Causal && G >= 32) ? 2 : kPackedPasses;
-    const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
-    const dim3 grid((a.rows + per_block - 1) / per_block);
-    if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, kDefaultFlags, R>), grid, dim3(256), 0, st, a);
-    } else {
-        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags, R>), grid, dim3(256), 0, st, a);
-    }
-    return hipGetLastError();
+    return launch_packed_shape<T, M, BWD, G, R, 1>(a, st);
 }
 
 // sk <= 512: lane groups of G = pow2 >= sk/8 lanes per row
@@ -78,6 +84,12 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         const bool mask_ok = BWD || M != Mask::Bytes || a.mask_bytes != 0;
         if (mask_ok) return dispatch_packed<T, M, BWD>(a, st);
         return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
+    }
+    if constexpr (BWD && M == Mask::None) {
+        // full rows up to 2048 columns: straight-line packed kernel, R x C = 4 accesses per tensor
+        if (chunks == 2) return launch_packed_shape<T, M, BWD, kWave, 2, 2>(a, st);
+        if (chunks == 3) return launch_packed_shape<T, M, BWD, kWave, 1, 3>(a, st);
+        if (chunks == 4) return launch_packed_shape<T, M, BWD, kWave, 1, 4>(a, st);
     }
     if (chunks == 2) return launch_shape<T, M, BWD, 2, 1, 4>(a, st);
     if (chunks <= 4) return launch_shape<T, M, BWD, 2, 2, 2>(a, st);
