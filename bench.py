@@ -15,7 +15,10 @@ steps between device synchronisations; the JSON line carries
                  stream inside the timed region, against the 8 TB/s HBM peak;
 * cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
                  this host's cores on a slice of the same batch;
-* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak.
+* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak, the error
+                 of the kernel's output on a slice against the oracle (max |err|, non-zero
+                 masked outputs; bit-equality for rotary) and the oracle's CPU time on a
+                 slice scaled to the full shape.
 
 Buffers rotate over several distinct sets so that no launch finds its input in
 the 256 MB Infinity Cache left there by the previous one.
@@ -274,6 +277,73 @@ def main():
         del xs, dys, ms
 
     # ------------------------------------------------------------------ every BASELINE shape
+    def cpu_time_us(fn, budget_s=1.5):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2 or (time.perf_counter() - t0 < budget_s and reps < 20):
+            fn()
+            reps += 1
+        return (time.perf_counter() - t0) / reps * 1e6
+
+    def softmax_extras(r, x, y, mask, sc, dt, total, dy=None, dx=None):
+        """Parity of the kernels' own output on a slice (against the oracle evaluated on the
+        GPU in fp32) and the oracle's CPU time on the same slice scaled to the full batch.
+        x, y (, dy, dx): [k, sq, sk] or [k, np, sq, sk] slices; mask broadcastable to them."""
+        k = x.shape[0]
+        x4 = x if x.dim() == 4 else x.unsqueeze(1)
+        y4 = y if y.dim() == 4 else y.unsqueeze(1)
+        if dx is None:
+            ref = R.softmax_fp32(x4, mask, sc)
+            r["max_abs_err"] = float((y4.float() - ref).abs().max())
+            r["masked_nonzero"] = int((y4[mask.expand_as(y4)] != 0).sum())
+        else:
+            dy4 = dy if dy.dim() == 4 else dy.unsqueeze(1)
+            dx4 = dx if dx.dim() == 4 else dx.unsqueeze(1)
+            r["max_abs_err"] = float((dx4.float() - R.softmax_backward_fp32(dy4, y4, sc)).abs().max())
+            r["masked_nonzero"] = int((dx4[mask.expand_as(dx4)] != 0).sum())
+        if not args.no_cpu:
+            xc, mc = x4.cpu(), mask.cpu()
+            f16 = dt == torch.float16
+            if dx is None:
+                us = cpu_time_us(lambda: R.forward_torch_softmax(xc, mc, sc, f16, not f16, True))
+            else:
+                gc = dy4.cpu()
+                xin = xc.clone().requires_grad_(True)
+                yc = R.forward_torch_softmax(xin, mc, sc, f16, not f16, True)
+                us = cpu_time_us(lambda: torch.autograd.grad(yc, xin, gc, retain_graph=True))
+            r["cpu_us_per_call"] = round(us * total / k, 1)
+            r["cpu_sample"] = f"{k} of {total} along dim 0, {torch.get_num_threads()} threads, scaled"
+        return r
+
+    def rope_extras(r, S, Bb, H, HN, DR, backward):
+        """Fresh tensors of the full shape: bit-equality with the fp32 expression rounded once
+        (all positions), CPU time of the torch expression on 256 positions scaled."""
+        g0 = gen(4321)
+        q = torch.randn(S, Bb, H, HN, device=dev, generator=g0).bfloat16()
+        k = torch.randn(S, Bb, H, HN, device=dev, generator=g0).bfloat16()
+        t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1, nsets=1)[0]
+        t["q"], t["k"] = q.clone(), k.clone()
+        rope_apply(t, S, Bb, H, DR, torch.bfloat16, backward)
+        cos4, sin4 = t["cos"].view(S, 1, 1, DR), t["sin"].view(S, 1, 1, DR)
+        if backward:
+            rq, rk = R.rotary_autograd_fp32(q[..., :DR], k[..., :DR], cos4, sin4, q[..., :DR], k[..., :DR])
+        else:
+            rq, rk = R.rotary_fp32(q[..., :DR], k[..., :DR], cos4, sin4)
+        r["bit_equal_to_fp32_rounded_once"] = bool(
+            torch.equal(t["q"][..., :DR], rq.bfloat16()) and torch.equal(t["k"][..., :DR], rk.bfloat16())
+            and torch.equal(t["q"][..., DR:], q[..., DR:]))
+        if not args.no_cpu:
+            n = 256
+            qc, kc = q[:n, ..., :DR].cpu(), k[:n, ..., :DR].cpu()
+            cc, sc_ = cos4[:n].cpu(), sin4[:n].cpu()
+            if backward:
+                us = cpu_time_us(lambda: R.rotary_autograd_fp32(qc, kc, cc, sc_, qc, kc))
+            else:
+                us = cpu_time_us(lambda: R.apply_rotary_pos_emb(qc, kc, cc, sc_))
+            r["cpu_us_per_call"] = round(us * S / n, 1)
+            r["cpu_sample"] = f"{n} of {S} positions, {torch.get_num_threads()} threads, scaled"
+        return r
+
     if not args.no_table:
         table = []
 
@@ -287,54 +357,71 @@ def main():
         if want("cfg1"):
             B, n, dt, sc = 48, 2048, torch.bfloat16, 0.125
             s_ = causal_sets(B, n, dt, 1234, nsets=2, need_bwd=False)
-            table.append(row("cfg1 causal fwd [48,2048,2048] bf16", B * 2 * (tri(n) + n * n),
-                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100)))
+            r = row("cfg1 causal fwd [48,2048,2048] bf16", B * 2 * (tri(n) + n * n),
+                    *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100))
+            table.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], R.get_attn_mask(n, dev), sc, dt, B))
             del s_
         # configs[1]
         if want("cfg2"):
             s_ = masked_sets(b, heads, sq, sk, dtype, 1235, nsets=3)
-            table.append(row("cfg2 padded fwd [8,16,1024,1024] fp16", fwd_bytes,
-                             *time_launches(lambda t: masked_fwd(t, b, heads, sq, sk, dtype, scale), s_, 100)))
-            table.append(row("cfg2 padded bwd [8,16,1024,1024] fp16", bwd_bytes,
-                             *time_launches(lambda t: masked_bwd(t, b, heads, sq, sk, dtype, scale), s_, 100)))
-            del s_
+            r = row("cfg2 padded fwd [8,16,1024,1024] fp16", fwd_bytes,
+                    *time_launches(lambda t: masked_fwd(t, b, heads, sq, sk, dtype, scale), s_, 100))
+            z = s_[0]
+            table.append(softmax_extras(r, z["x"][:1], z["y"][:1], z["mask"][:1], scale, dtype, b))
+            r = row("cfg2 padded bwd [8,16,1024,1024] fp16", bwd_bytes,
+                    *time_launches(lambda t: masked_bwd(t, b, heads, sq, sk, dtype, scale), s_, 100))
+            table.append(softmax_extras(r, z["x"][:1], z["y"][:1], z["mask"][:1], scale, dtype, b,
+                                        dy=z["dy"][:1], dx=z["dx"][:1]))
+            del s_, z
         # configs[2]: partial rotary
         if want("cfg3"):
             S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
             s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1236, nsets=10)
             nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-            table.append(row("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
-                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200)))
-            table.append(row("cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
-                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200)))
+            r = row("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
+                    *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200))
+            table.append(rope_extras(r, S, Bb, H, HN, DR, 0))
+            r = row("cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
+                    *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
+            table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
             del s_
         # configs[3]: 20B shape
         if want("cfg4"):
             B, n, dt, sc = 64, 2048, torch.float16, 96 ** -0.5
             s_ = causal_sets(B, n, dt, 1237, nsets=2, need_bwd=True)
-            table.append(row("cfg4 causal fwd [64,2048,2048] fp16", B * 2 * (tri(n) + n * n),
-                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100)))
-            table.append(row("cfg4 causal bwd [64,2048,2048] fp16", B * 2 * (2 * tri(n) + n * n),
-                             *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 100)))
-            del s_
+            cm = R.get_attn_mask(n, dev)
+            r = row("cfg4 causal fwd [64,2048,2048] fp16", B * 2 * (tri(n) + n * n),
+                    *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100))
+            z = s_[0]
+            table.append(softmax_extras(r, z["x"][:2], z["y"][:2], cm, sc, dt, B))
+            r = row("cfg4 causal bwd [64,2048,2048] fp16", B * 2 * (2 * tri(n) + n * n),
+                    *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 100))
+            table.append(softmax_extras(r, z["x"][:2], z["y"][:2], cm, sc, dt, B, dy=z["dy"][:2], dx=z["dx"][:2]))
+            del s_, z, cm
         # configs[4]: long context
         if want("cfg5"):
             torch.cuda.empty_cache()
             B, n, dt, sc = 32, 8192, torch.bfloat16, 128 ** -0.5
             s_ = causal_sets(B, n, dt, 1238, nsets=1, need_bwd=True)
-            table.append(row("cfg5 causal fwd [32,8192,8192] bf16", B * 2 * (tri(n) + n * n),
-                             *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 30, warm=5)))
-            table.append(row("cfg5 causal bwd [32,8192,8192] bf16", B * 2 * (2 * tri(n) + n * n),
-                             *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 30, warm=5)))
-            del s_
+            cm = R.get_attn_mask(n, dev)
+            r = row("cfg5 causal fwd [32,8192,8192] bf16", B * 2 * (tri(n) + n * n),
+                    *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 30, warm=5))
+            z = s_[0]
+            table.append(softmax_extras(r, z["x"][:1], z["y"][:1], cm, sc, dt, B))
+            r = row("cfg5 causal bwd [32,8192,8192] bf16", B * 2 * (2 * tri(n) + n * n),
+                    *time_launches(lambda t: causal_bwd(t, B, n, dt, sc), s_, 30, warm=5))
+            table.append(softmax_extras(r, z["x"][:1], z["y"][:1], cm, sc, dt, B, dy=z["dy"][:1], dx=z["dx"][:1]))
+            del s_, z, cm
             torch.cuda.empty_cache()
             S, Bb, H, HN, DR = 8192, 1, 32, 128, 128
             s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1239, nsets=6)
             nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-            table.append(row("cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
-                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200)))
-            table.append(row("cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
-                             *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200)))
+            r = row("cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
+                    *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 0), s_, 200))
+            table.append(rope_extras(r, S, Bb, H, HN, DR, 0))
+            r = row("cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128", nb,
+                    *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
+            table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
             del s_
         # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
         if want("copy"):
