@@ -28,6 +28,9 @@ SIGNATURES = {
     "neox_fused_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "neox_fused_last_error": (ctypes.c_char_p, []),
     "neox_causal_softmax_fwd": (ctypes.c_int, [_vp, _vp, _f32, _i64, _i32, _i32, _i32, _vp]),
+    "neox_causal_softmax_alibi_fwd": (
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _vp]
+    ),
     "neox_causal_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _i32, _vp]),
     "neox_masked_softmax_fwd": (
         ctypes.c_int,

@@ -98,6 +98,29 @@ int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches
     return check_launch(launch_softmax_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
 }
 
+int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, float scale, int32_t b,
+                                  int32_t np, int32_t sq, int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_causal_softmax_alibi_fwd";
+    if (!y || !x || !slopes) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(slopes, 4))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    a.out = y;
+    a.in0 = x;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)((int64_t)b * np * sq);
+    a.sq = sq;
+    a.sk = sk;
+    a.slopes = slopes;
+    a.np = (uint32_t)np;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
 int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
                             int32_t sq, int32_t sk, int32_t dtype, void* stream) {
     static const char* what = "neox_causal_softmax_bwd";

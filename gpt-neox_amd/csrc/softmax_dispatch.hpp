@@ -18,6 +18,12 @@
 
 namespace neox {
 
+// kernel flags: the causal forward has a second instantiation that adds the ALiBi bias
+template <Mask M, bool BWD>
+static bool wants_alibi(const SoftmaxArgs& a) {
+    return !BWD && M == Mask::Causal && a.slopes != nullptr;
+}
+
 template <typename T, Mask M, bool BWD, int NCH, int WPR, int RPB>
 static hipError_t launch_shape(const SoftmaxArgs& a, hipStream_t st) {
     const dim3 grid((a.rows + RPB - 1) / RPB);
@@ -25,6 +31,12 @@ static hipError_t launch_shape(const SoftmaxArgs& a, hipStream_t st) {
     if constexpr (BWD) {
         hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M>), grid, block, 0, st, a);
     } else {
+        if constexpr (M == Mask::Causal) {
+            if (wants_alibi<M, BWD>(a)) {
+                hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, kDefaultFlags | kAlibi>), grid, block, 0, st, a);
+                return hipGetLastError();
+            }
+        }
         hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M>), grid, block, 0, st, a);
     }
     return hipGetLastError();
@@ -49,6 +61,12 @@ static hipError_t launch_packed_shape(const SoftmaxArgs& a, hipStream_t st) {
     if constexpr (BWD) {
         hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
     } else {
+        if constexpr (M == Mask::Causal) {
+            if (wants_alibi<M, BWD>(a)) {
+                hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags | kAlibi, R, C>), grid, dim3(256), 0, st, a);
+                return hipGetLastError();
+            }
+        }
         hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
     }
     return hipGetLastError();

@@ -33,6 +33,8 @@ struct SoftmaxArgs {
     uint32_t rows_per_mask_batch;  // np*sq: rows sharing one mask sample
     int32_t mask_bcast;            // mask batch dim is 1
     uint32_t mask_bytes;           // size of the mask tensor, 0 if it does not fit 32 bits
+    const float* slopes;           // ALiBi (kAlibi kernels): one slope per head, fp32 [np]
+    uint32_t np;                   // heads per sample (kAlibi kernels)
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -40,6 +42,7 @@ enum class Mask { Causal, Bytes, None };
 // Compile-time tuning switches of the row kernels.
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
 constexpr int kNtStore = 2;  // non-temporal hint on the streaming stores
+constexpr int kAlibi = 4;    // causal forward adds the ALiBi bias -slope[head]*(i - j) to the scores
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
 
 // Where a wave works: the row, its position i inside its [sq, sk] matrix, the number of
@@ -105,6 +108,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     const int voff = lane * 16 + wir * kChunk * 2;
 
     const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    // ALiBi: scale*(x + slope*(j - i)) = x*scale + slope2*(j - i), slope2 wave-uniform
+    float slope2 = 0.f;
+    if constexpr ((FLAGS & kAlibi) != 0) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
     u32x4 raw[NCH];
     u32x2 mk[NCH];
     {
@@ -136,10 +142,16 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 if constexpr (MASK == Mask::Bytes) {
                     plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
                 }
+                float bias[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    bias[k] = 0.f;
+                    if constexpr ((FLAGS & kAlibi) != 0) bias[k] = slope2 * (float)(col + k - (int)pos.i);
+                }
                 if (plain) {
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
-                        v[c][k] *= a.scale;
+                        v[c][k] = fmaf(v[c][k], a.scale, bias[k]);  // bias 0: the plain product
                         mx = fmaxf(mx, v[c][k]);
                     }
                 } else {
@@ -150,7 +162,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                             const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
                             keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
                         }
-                        v[c][k] = keep ? v[c][k] * a.scale : ninf;
+                        v[c][k] = keep ? fmaf(v[c][k], a.scale, bias[k]) : ninf;
                         mx = fmaxf(mx, v[c][k]);
                     }
                 }
@@ -340,6 +352,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     u32x4 raw[R][C];
     u32x2 mk[R][C];
     int len[R];
+    int ipos[R];       // row position inside its matrix (ALiBi)
+    float slope2[R];   // slope[head] * scale of the lane's row (ALiBi)
     const uint32_t i0 = row0 % (uint32_t)a.sq;  // wave-uniform
 #pragma unroll
     for (int p = 0; p < R; ++p) {
@@ -348,6 +362,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
         const uint32_t i = wrap_row(i0 + lr, (uint32_t)a.sq);
         len[p] = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
         if (lr >= rows_here) len[p] = 0;
+        ipos[p] = (int)i;
+        slope2[p] = 0.f;
+        if constexpr ((FLAGS & kAlibi) != 0) {
+            const uint32_t safe_row = lr < rows_here ? row : row0;
+            slope2[p] = a.slopes[(safe_row / (uint32_t)a.sq) % a.np] * a.scale;
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
@@ -375,7 +395,9 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
                     const uint32_t w = (k < 4) ? mk[p][c].x : mk[p][c].y;
                     keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
                 }
-                v[c][k] = keep ? v[c][k] * a.scale : ninf;
+                float bias = 0.f;
+                if constexpr ((FLAGS & kAlibi) != 0) bias = slope2[p] * (float)(col + k - ipos[p]);
+                v[c][k] = keep ? fmaf(v[c][k], a.scale, bias) : ninf;
                 mx = fmaxf(mx, v[c][k]);
             }
         }
@@ -523,12 +545,18 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
         mrow = a.mask + ((size_t)mb * a.sq + i) * sk;
     }
     const float ninf = -__builtin_inff();
+    // ALiBi (causal only): slopes given -> scores get slope*(j - i) before the scale
+    const float slope2 = (MASK == Mask::Causal && a.slopes != nullptr)
+                             ? a.slopes[(row / (uint32_t)a.sq) % a.np] * a.scale : 0.f;
+    auto score = [&](int j) {
+        return fmaf(Elem<T>::load1(x + (size_t)j * 2), a.scale, slope2 * (float)(j - (int)i));
+    };
 
     float mx = ninf;
     for (int j = threadIdx.x; j < len; j += kGenericThreads) {
         bool keep = true;
         if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
-        if (keep) mx = fmaxf(mx, Elem<T>::load1(x + (size_t)j * 2) * a.scale);
+        if (keep) mx = fmaxf(mx, score(j));
     }
     mx = block_reduce<OpMax>(mx, red);
     const bool all_masked = (mx == ninf);
@@ -537,7 +565,7 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
     for (int j = threadIdx.x; j < len; j += kGenericThreads) {
         bool keep = true;
         if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
-        float e = keep ? fast_exp2(Elem<T>::load1(x + (size_t)j * 2) * a.scale - mx) : 0.f;
+        float e = keep ? fast_exp2(score(j) - mx) : 0.f;
         if (all_masked) e = 1.f;
         sum += e;
     }
@@ -550,7 +578,7 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
         if (j < len) {
             bool keep = true;
             if constexpr (MASK == Mask::Bytes) keep = (mrow[j] == 0);
-            float e = keep ? fast_exp2(Elem<T>::load1(x + (size_t)j * 2) * a.scale - mx) : 0.f;
+            float e = keep ? fast_exp2(score(j) - mx) : 0.f;
             if (all_masked) e = 1.f;
             o = e * inv;
         }

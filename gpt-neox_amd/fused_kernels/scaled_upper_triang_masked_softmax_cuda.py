@@ -35,6 +35,37 @@ def forward(input, scale_factor):
     return softmax_results
 
 
+def forward_alibi(input, slopes, scale_factor):
+    """Causal softmax of ``scale * (input + alibi_bias)`` without materialising the bias.
+
+    ``input``: ``[b, np, sq, sk]`` fp16/bf16; ``slopes``: ``[np]`` (any float dtype), the
+    per-head ALiBi slopes; the bias of head h is ``-slopes[h] * (i - j)`` for ``j <= i``
+    (megatron/model/positional_embeddings.py:161-176).  No counterpart in the reference's
+    extension: it adds the bias in a separate pass before calling ``forward``.
+    """
+    if input.dim() != 4:
+        raise RuntimeError("expected 4D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    b, np_, sq, sk = input.shape
+    if slopes.numel() != np_:
+        raise RuntimeError(f"expected {np_} ALiBi slopes (one per head), got {slopes.numel()}")
+    _lib.require_gpu(input, slopes)
+    input = input.contiguous()
+    slopes = slopes.detach().to(dtype=torch.float32).contiguous()
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_alibi_fwd(
+                softmax_results.data_ptr(), input.data_ptr(), slopes.data_ptr(), float(scale_factor),
+                b, np_, sq, sk, _lib.dtype_code(input.dtype), _lib.current_stream(input),
+            )
+        )
+    return softmax_results
+
+
 def backward(output_grads, softmax_results, scale_factor):
     """Returns d(input); like the reference, the result is written into
     ``output_grads`` itself when that tensor is contiguous."""

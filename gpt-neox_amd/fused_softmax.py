@@ -41,6 +41,20 @@ from .fused_kernels import scaled_masked_softmax_cuda as _masked_ext
 from .fused_kernels import scaled_upper_triang_masked_softmax_cuda as _causal_ext
 
 
+def alibi_bias(slopes, sq, sk, device, dtype):
+    """The ALiBi bias ``[np, sq, sk]`` (``[np, 1, sk]`` for a one-query decode step) as the
+    reference's ``AliBi`` module builds it, in ``dtype``: ``-slope_h * (i - j)`` for ``j <= i``,
+    0 above the diagonal (megatron/model/positional_embeddings.py:161-206)."""
+    rows = torch.arange(sk, device=device).view(sk, 1)
+    cols = torch.arange(sk, device=device).view(1, sk)
+    dist = (-torch.tril(rows - cols)).to(dtype)
+    bias = dist * slopes.to(device=device, dtype=dtype).view(-1, 1, 1)
+    if sq != sk:
+        assert sq == 1, "assumption sq == sk unless at inference time with cache in layer_past with sq == 1"
+        bias = bias[:, sk - 1, :].view(bias.shape[0], 1, sk)
+    return bias
+
+
 def _remember(ctx, probs, scale_t):
     ctx.save_for_backward(probs, scale_t)
     return probs
@@ -114,6 +128,27 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         return _causal_ext.backward(output_grads, probs, scale), None
 
 
+class ScaledUpperTriangMaskedSoftmaxAlibi(torch.autograd.Function):
+    """Causal softmax of ``scale * (inputs + alibi_bias(slopes))`` in one kernel; the bias is
+    computed from the per-head slopes inside the kernel instead of being added to the scores
+    in a pass of its own (megatron/model/transformer.py:529-534).
+
+    ``inputs``: ``[b, np, sq, sk]`` fp16/bf16; ``slopes``: ``[np]``.  Gradient with respect to
+    ``inputs`` only (the bias is a constant)."""
+
+    @staticmethod
+    def forward(ctx, inputs, slopes, scale):
+        scale_t = _scale_tensor(scale)
+        return _remember(ctx, _causal_ext.forward_alibi(inputs, slopes, scale_t[0].item()), scale_t)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        b, np, sq, sk = probs.shape
+        grads = _causal_ext.backward(output_grads.reshape(-1, sq, sk), probs.view(-1, sq, sk), scale)
+        return grads.view(b, np, sq, sk), None, None
+
+
 class ScaledMaskedSoftmax(torch.autograd.Function):
     """scale -> mask tensor -> softmax, in one kernel.
 
@@ -168,9 +203,19 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         if self.fusion:
             load_fused_kernels()  # ImportError here, not at the first forward
 
-    def forward(self, input, mask):
+    def forward(self, input, mask, alibi_slopes=None):
+        """``alibi_slopes`` (optional, ``[np]``) is an addition to the reference signature:
+        ``forward(scores, mask, alibi_slopes=alibi.slopes)`` equals
+        ``forward(alibi(scores), mask)`` (megatron/model/transformer.py:529-534) with the bias
+        evaluated in fp32 inside the causal kernel instead of a separate pass in half precision."""
         assert input.dim() == 4  # [b, np, sq, sk]
         fused = self.is_kernel_available(mask, *input.size())
+        if alibi_slopes is not None:
+            b, np, sq, sk = input.size()
+            if fused and self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
+                scale = 1.0 if self.scale is None else self.scale
+                return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
+            input = input + alibi_bias(alibi_slopes, sq, sk, input.device, input.dtype)
         return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
 
     def is_kernel_available(self, mask, b, np, sq, sk):

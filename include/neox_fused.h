@@ -62,6 +62,17 @@ int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches
                             int32_t sk, int32_t dtype, void* stream);
 
 /*
+ * Causal softmax with the ALiBi bias folded in (no separate pass over the scores):
+ *   y[n,h,i,j] = softmax_j(scale * (x[n,h,i,j] - slopes[h] * (i - j))) over j <= i ; 0 for j > i
+ * x, y: [b, np, sq, sk] contiguous; slopes: fp32 [np] in device memory.  The gradient with
+ * respect to x is neox_causal_softmax_bwd (the bias is a constant).
+ * Replaces AliBi.forward followed by scaled_upper_triang_masked_softmax_cuda.forward
+ *   megatron/model/positional_embeddings.py:210-257, megatron/model/transformer.py:529-534
+ */
+int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, float scale, int32_t b,
+                                  int32_t np, int32_t sq, int32_t sk, int32_t dtype, void* stream);
+
+/*
  * Causal softmax backward:  dx = scale * y * (dy - sum_j(dy*y)) over j <= i,
  * dx = 0 for j > i.  dx may alias dy (the reference overwrites dy in place).
  * Replaces scaled_upper_triang_masked_softmax_cuda.backward

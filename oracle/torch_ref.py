@@ -100,6 +100,32 @@ def softmax_autograd_fp32(x, mask, scale, grad_out):
     return y.detach(), xf.grad
 
 
+def alibi_slopes(n):
+    """Head slopes of ALiBi: 2^(-8/n * (k+1)) for a power-of-two n, otherwise the slopes of the
+    power of two below plus every second slope of the one above.
+    Follows AliBi._get_slopes, megatron/model/positional_embeddings.py:147-170."""
+    import math
+
+    def power_of_two(m):
+        start = 2 ** (-(2 ** -(math.log2(m) - 3)))
+        return [start * start**k for k in range(m)]
+
+    if math.log2(n).is_integer():
+        return power_of_two(n)
+    below = 2 ** math.floor(math.log2(n))
+    return power_of_two(below) + alibi_slopes(2 * below)[0::2][: n - below]
+
+
+def alibi_bias_fp32(slopes, sq, sk):
+    """fp32 ALiBi bias [np, sq, sk]: -slope_h * (i - j) on j <= i, 0 above the diagonal.
+    Follows AliBi.forward, megatron/model/positional_embeddings.py:210-257 (sq == sk)."""
+    assert sq == sk
+    i = torch.arange(sq).view(sq, 1)
+    j = torch.arange(sk).view(1, sk)
+    dist = -torch.tril(i - j).float()
+    return dist * torch.as_tensor(slopes, dtype=torch.float32).view(-1, 1, 1)
+
+
 # --- rotary ------------------------------------------------------------------------
 
 

@@ -106,3 +106,24 @@ def test_alibi_slopes_and_bias():
     a(torch.zeros(1, 2, 7, 7))
     assert a.cached_seq_len == 20  # grown 4x
     assert torch.equal(a.bias(7, 7, "cpu", torch.float32), a(torch.zeros(1, 2, 7, 7))[0])
+
+
+def test_alibi_bias_helper_equals_the_alibi_module_and_the_oracle():
+    from gpt_neox_amd.fused_softmax import alibi_bias
+
+    mod = AliBi(6, mp_size=1, mp_rank=0)
+    assert mod.slopes.tolist() == pytest.approx(R.alibi_slopes(6))
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.zeros(2, 6, 9, 9, dtype=dtype)
+        assert torch.equal(mod(x)[0], alibi_bias(mod.slopes, 9, 9, "cpu", dtype))
+    assert torch.equal(alibi_bias(mod.slopes, 9, 9, "cpu", torch.float32), R.alibi_bias_fp32(mod.slopes, 9, 9))
+    one = AliBi(6, mp_size=1, mp_rank=0)
+    assert torch.equal(one(torch.zeros(2, 6, 1, 9))[0], alibi_bias(mod.slopes, 1, 9, "cpu", torch.float32))
+
+
+def test_alibi_slopes_argument_on_the_unfused_branch():
+    mod = AliBi(4, mp_size=1, mp_rank=0)
+    x = torch.randn(2, 4, 8, 8)
+    mask = R.get_attn_mask(8)
+    sm = FusedScaleMaskSoftmax(False, False, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
+    assert torch.equal(sm(x.clone(), mask, alibi_slopes=mod.slopes), sm(mod(x.clone()), mask))

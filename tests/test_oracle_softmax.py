@@ -180,3 +180,29 @@ def test_fixtures_backward(golden):
         f = golden[name]
         dx = R.softmax_backward_fp32(torch.tensor(f["g"]), torch.tensor(f["y"]), float(f["scale"]))
         assert np.allclose(dx.numpy(), f["dx"], atol=1e-5), name
+
+
+# ---- ALiBi bias -----------------------------------------------------------------------
+
+
+def test_alibi_slopes_and_bias_closed_forms():
+    assert R.alibi_slopes(8) == pytest.approx([2.0 ** -(k + 1) for k in range(8)])
+    assert R.alibi_slopes(4) == pytest.approx([2.0 ** -2, 2.0 ** -4, 2.0 ** -6, 2.0 ** -8])
+    s6 = R.alibi_slopes(6)  # 4 slopes of n=4, then slopes 0 and 2 of n=8
+    assert s6 == pytest.approx([2.0 ** -2, 2.0 ** -4, 2.0 ** -6, 2.0 ** -8, 2.0 ** -1, 2.0 ** -3])
+    bias = R.alibi_bias_fp32([0.5, 0.25], 4, 4)
+    assert bias.shape == (2, 4, 4)
+    for h, m in enumerate((0.5, 0.25)):
+        for i in range(4):
+            for j in range(4):
+                assert bias[h, i, j].item() == (-m * (i - j) if j <= i else 0.0)
+
+
+def test_alibi_softmax_row_closed_form():
+    # zero scores: row i of head h is softmax_j(-m (i - j)) = a geometric distribution
+    m, s = 0.5, 6
+    y = R.softmax_fp32(torch.zeros(1, 1, s, s) + R.alibi_bias_fp32([m], s, s), R.get_attn_mask(s), 1.0)
+    for i in range(s):
+        w = [math.exp(-m * (i - j)) for j in range(i + 1)]
+        for j in range(i + 1):
+            assert y[0, 0, i, j].item() == pytest.approx(w[j] / sum(w), abs=1e-6)

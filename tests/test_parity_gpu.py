@@ -350,6 +350,53 @@ def test_causal_module_honours_masks_that_are_not_plain_causal(device):
         assert max_err(fused(x, plain), R.softmax_fp32(x, plain, 0.25)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 4, 8), (1, 6, 40), (2, 3, 136), (1, 8, 520), (2, 2, 1000), (1, 4, 2048),
+                                   (1, 2, 2568), (1, 2, 4104), (1, 3, 37)])
+def test_alibi_folded_into_the_causal_kernel(device, shape, dtype):
+    # scale * (x + alibi) evaluated in fp32, against the fp32 oracle; every kernel family
+    # (packed, one/several waves per row, element-wise)
+    b, heads, s = shape
+    x = scores((b, heads, s, s), dtype, device, s)
+    slopes = torch.tensor(R.alibi_slopes(heads), device=device)
+    mask = R.get_attn_mask(s, device)
+    want = R.softmax_fp32(x.float() + R.alibi_bias_fp32(slopes.cpu(), s, s).to(device), mask, 0.25)
+    got = causal_ext.forward_alibi(x, slopes, 0.25)
+    assert max_err(got, want) <= TOL[dtype]
+    assert (got[mask.expand_as(got)] == 0).all()
+    zero = causal_ext.forward_alibi(x, torch.zeros_like(slopes), 0.25)  # zero slopes: the plain kernel's result
+    assert max_err(zero, causal_ext.forward(x.view(-1, s, s), 0.25).view_as(x)) <= 2.0 ** -8
+
+
+def test_alibi_module_argument_and_gradient(device):
+    from gpt_neox_amd.positional_embeddings import AliBi
+
+    b, heads, s, dtype = 2, 4, 72, torch.bfloat16
+    alibi = AliBi(heads, mp_size=1, mp_rank=0).to(device)
+    mask = R.get_attn_mask(s, device)
+    fused = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang,
+                                  R.gpt2_attention_mask_func, True, 0.5)
+    x = scores((b, heads, s, s), dtype, device, 3)
+    xf = x.clone().requires_grad_(True)
+    y = fused(xf, mask, alibi_slopes=alibi.slopes)
+    # fp32 oracle, forward and autograd backward
+    xr = x.float().requires_grad_(True)
+    bias = R.alibi_bias_fp32(alibi.slopes.cpu(), s, s).to(device)
+    yr = torch.softmax(R.gpt2_attention_mask_func((xr + bias) * 0.5, mask), -1)
+    assert max_err(y, yr) <= TOL[dtype]
+    g = normal(y.shape, dtype, device, 4)
+    y.backward(g.clone())
+    yr.backward(g.float())
+    assert max_err(xf.grad, xr.grad) <= 4 * TOL[dtype] * max(1.0, xr.grad.abs().max().item())
+    # the reference's two-pass sequence (bias added in bf16) stays within bf16 noise of it
+    two_pass = fused(alibi(x), mask)
+    assert max_err(y, two_pass) <= 0.06
+    # a sliding-window mask cannot use the causal kernel: bias added first, mask honoured
+    window = R.get_attn_mask(s, device, sliding_window_width=5)
+    yw = fused(x, window, alibi_slopes=alibi.slopes)
+    assert max_err(yw, fused(alibi(x), window)) == 0.0
+
+
 def test_causal_decode_step_takes_the_torch_branch(device):
     fused = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang,
                                   R.gpt2_attention_mask_func, True, None)
