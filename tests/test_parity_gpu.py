@@ -553,6 +553,35 @@ def test_rotary_half_precision_tables(device, dtype):
     assert emb(q, seq_len=s)[0].data_ptr() == cos.data_ptr()  # device copy is kept, not re-made
 
 
+@pytest.mark.parametrize("d_rot", [64, 48, 24, 6])
+def test_rotary_head_loop_split_over_blocks(device, d_rot):
+    # few positions, many heads: the head loop of a position is split over blockIdx.z
+    # (contiguous-span kernel for d_rot = 64, the per-pair kernel with 8/4/1-element slots otherwise)
+    s, b, h, hn = 2, 1, 600, 64
+    q, k = normal((s, b, h, hn), torch.float16, device, 1), normal((s, b, 77, hn), torch.float16, device, 2)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s))
+    oq, ok = apply_rotary_pos_emb(q[..., :d_rot], k[..., :d_rot], cos, sin)
+    rq, rk = R.rotary_fp32(q[..., :d_rot], k[..., :d_rot], cos, sin)
+    assert torch.equal(oq, rq.half()) and torch.equal(ok, rk.half())
+
+
+@pytest.mark.parametrize("d_rot", [32, 24, 48])
+def test_rotary_strided_batch_and_half_tables_on_every_kernel(device, d_rot):
+    # [s, b, h, d] view of a [b, s, h, d] buffer (batch stride cannot be folded into the head
+    # stride) with tables stored in the dtype of q
+    s, b, h, hn = 10, 3, 4, 64
+    for dtype in DTYPES:
+        q = normal((b, s, h, hn), dtype, device, 1).transpose(0, 1)
+        k = normal((b, s, h, hn), dtype, device, 2).transpose(0, 1)
+        cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + 2, 10000, dtype))
+        oq, ok = apply_rotary_pos_emb(q[..., :d_rot], k[..., :d_rot], cos, sin, offset=2)
+        rq, rk = R.rotary_fp32(q[..., :d_rot], k[..., :d_rot], cos, sin, offset=2)
+        assert torch.equal(oq, rq.to(dtype)) and torch.equal(ok, rk.to(dtype))
+        q2, k2 = q.clone(memory_format=torch.preserve_format), k.clone(memory_format=torch.preserve_format)
+        apply_rotary_pos_emb_(q2, k2, cos, sin, 2, d_rot)
+        assert torch.equal(q2[..., :d_rot], oq) and torch.equal(q2[..., d_rot:], q[..., d_rot:])
+
+
 def test_rotary_non_collapsible_layout(device):
     # [s, b, h, d] view of a [b, s, h, d] buffer: stride_b != h * stride_h
     s, b, h, d = 10, 3, 4, 32
