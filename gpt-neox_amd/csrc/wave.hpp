@@ -1,6 +1,7 @@
 // Device-side building blocks shared by the gfx950 kernels: 128-bit packed
-// half/bfloat16 access, fp32 <-> 16-bit conversion, and wave64 reductions done
-// with DPP row operations plus four lane reads (no LDS traffic).
+// half/bfloat16 access (flat and range-checked buffer forms), fp32 <-> 16-bit
+// conversion, and reductions over a wave64 or over lane groups inside it done with
+// DPP row operations, one swizzle and four lane reads (no LDS traffic).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -91,16 +92,6 @@ __device__ __forceinline__ u32x4 ld128(const void* p) {
 }
 __device__ __forceinline__ void st128(void* p, const u32x4& v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
-}
-__device__ __forceinline__ u32x2 ld64(const void* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
-}
-// cached variants (data that several waves re-read: masks, cos/sin tables)
-__device__ __forceinline__ u32x4 ld128_cached(const void* p) {
-    return *reinterpret_cast<const u32x4*>(p);
-}
-__device__ __forceinline__ u32x2 ld64_cached(const void* p) {
-    return *reinterpret_cast<const u32x2*>(p);
 }
 
 // ---- buffer (range-checked) access --------------------------------------------------
