@@ -37,8 +37,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel (configs[1] backward), from the rocprofv3 counter
 # runs of this same script summarised in profiles/bench_all_configs_hbm_counters.txt:
-# fetched 536.9 MB (TCC_EA0_RDREQ x 128 B) + written 268.5 MB (WRITE_SIZE); cannot be read live.
-MEASURED_TRAFFIC_BWD_BYTES = 805.4e6
+# fetched 536.9 MB (TCC_EA0_RDREQ x 128 B) + written 268.4 MB (WRITE_SIZE); cannot be read live.
+MEASURED_TRAFFIC_BWD_BYTES = 805.3e6
 METRIC = "softmax/rotary fwd+bwd achieved GB/s and % of MI355X HBM peak; µs per call"
 
 
@@ -228,7 +228,7 @@ def main():
         "us_per_call": {"fwd": round(fwd_us, 2), "bwd": round(bwd_us, 2)},
         "roofline": {
             "bound": "hbm",
-            "kernel": "softmax_bwd_kernel<F16, 2 chunks/wave, 1 wave/row, 4 rows/block, no mask>",
+            "kernel": "softmax_bwd_packed_kernel<F16, 64 lanes/row, no mask, 2 row passes/wave, 2 chunks of 512 columns>",
             "achieved": round(bwd_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
