@@ -431,6 +431,78 @@ def main():
             table.append(row("copy 1 GiB (read + write)", 2 * nbytes,
                              *time_launches(lambda t: ok(lib.neox_copy_bytes(dst.data_ptr(), src.data_ptr(),
                                                                             nbytes, stream)), [None], 50)))
+        # softmax + attention dropout in one kernel per pass (the op that follows the softmax in
+        # the model), on the padded, the 20B and the long-context shapes; p = 0.1
+        if want("dropout"):
+            from gpt_neox_amd.fused_kernels import attention_dropout as rng
+
+            extras, p_drop, seed = [], 0.1, 1234
+
+            def drop_extras(r, z, k, mask, sc, fwd):
+                """Slice [:k] along dim 0: the dropped output against torch's dropout expression
+                on the kernel's own probabilities and keep pattern (bit-equality), or the
+                backward against the fp32 closed form."""
+                y = z["y"][:k]
+                keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
+                if fwd:
+                    r["dropped_bit_equal_to_torch_expression"] = bool(
+                        torch.equal(z["y2"][:k], R.dropout_with_mask(y, keep, p_drop)))
+                    r["kept_fraction"] = round(float(keep.float().mean()), 5)
+                else:
+                    ref = R.softmax_dropout_backward_fp32(z["dy"][:k], y, keep, p_drop, sc)
+                    r["max_abs_err"] = float((z["dx"][:k].float() - ref).abs().max())
+                    r["masked_nonzero"] = int((z["dx"][:k][mask.expand_as(y)] != 0).sum())
+                return r
+
+            s_ = masked_sets(b, heads, sq, sk, dtype, 1240, nsets=3)
+            for z in s_:
+                z["y2"] = torch.empty_like(z["x"])
+
+            def md_fwd(t):
+                ok(lib.neox_masked_softmax_dropout_fwd(
+                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), scale,
+                    p_drop, seed, 0, b, heads, sq, sk, b, code[dtype], stream))
+
+            def md_bwd(t):
+                ok(lib.neox_masked_softmax_dropout_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0,
+                    b * heads * sq, sk, code[dtype], stream))
+
+            z = s_[0]
+            r = row("cfg2 padded fwd + dropout [8,16,1024,1024] fp16", 3 * n_elem * 2 + b * sq * sk,
+                    *time_launches(md_fwd, s_, 100))
+            extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, True))
+            r = row("cfg2 padded bwd + dropout [8,16,1024,1024] fp16", bwd_bytes, *time_launches(md_bwd, s_, 100))
+            extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, False))
+            del s_, z
+            for label, B, n, dt, sc, nl in (("cfg4", 64, 2048, torch.float16, 96 ** -0.5, 100),
+                                            ("cfg5", 32, 8192, torch.bfloat16, 128 ** -0.5, 30)):
+                torch.cuda.empty_cache()
+                s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
+                for z in s_:
+                    z["y2"] = torch.empty_like(z["x"])
+                cm = R.get_attn_mask(n, dev)[0]
+
+                def cd_fwd(t):
+                    ok(lib.neox_causal_softmax_dropout_fwd(
+                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), sc, p_drop, seed, 0, B, n, n,
+                        code[dt], stream))
+
+                def cd_bwd(t):
+                    ok(lib.neox_causal_softmax_dropout_bwd(
+                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, B, n, n,
+                        code[dt], stream))
+
+                z = s_[0]
+                shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'}"
+                r = row(f"{label} causal fwd + dropout {shape}", B * 2 * (tri(n) + 2 * n * n),
+                        *time_launches(cd_fwd, s_, nl, warm=5))
+                extras.append(drop_extras(r, z, 1, cm, sc, True))
+                r = row(f"{label} causal bwd + dropout {shape}", B * 2 * (2 * tri(n) + n * n),
+                        *time_launches(cd_bwd, s_, nl, warm=5))
+                extras.append(drop_extras(r, z, 1, cm, sc, False))
+                del s_, z, cm
+            result["fused_dropout"] = extras
         result["all_configs"] = table
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
         if pcts:

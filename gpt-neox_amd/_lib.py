@@ -21,6 +21,7 @@ _DTYPE_CODE = {torch.float16: NEOX_F16, torch.bfloat16: NEOX_BF16, torch.float32
 
 _c_i64p = ctypes.POINTER(ctypes.c_int64)
 _vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
+_u64 = ctypes.c_uint64
 
 # name -> (restype, argtypes); one entry per declaration of include/neox_fused.h
 SIGNATURES = {
@@ -37,6 +38,20 @@ SIGNATURES = {
         [_vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_masked_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _vp]),
+    "neox_causal_softmax_dropout_fwd": (
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _i32, _vp]
+    ),
+    "neox_causal_softmax_dropout_bwd": (
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _i32, _vp]
+    ),
+    "neox_masked_softmax_dropout_fwd": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _f32, _f32, _u64, _u64, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+    ),
+    "neox_masked_softmax_dropout_bwd": (
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _vp]
+    ),
+    "neox_dropout_keep_mask": (ctypes.c_int, [_vp, _f32, _u64, _u64, _i64, _vp]),
     "neox_get_batch_per_block": (ctypes.c_int, [_i32, _i32, _i32, _i32]),
     "neox_rope_apply": (
         ctypes.c_int,

@@ -42,6 +42,30 @@ static int check_rows(int64_t rows, int sq, int sk, const char* what) {
     return NEOX_OK;
 }
 
+// Dropout parameters of a call: threshold in 16-bit units and the fp32 factor 1/(1-p)
+// formed as torch's dropout kernel forms it (fp32 keep probability, then the quotient).
+static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset, const char* what) {
+    if (!(p >= 0.f && p <= 1.f))
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: dropout probability has to be between 0 and 1, but got %g", what, (double)p);
+    d.seed_lo = (uint32_t)seed;
+    d.seed_hi = (uint32_t)(seed >> 32);
+    d.off_lo = (uint32_t)offset;
+    d.off_hi = (uint32_t)(offset >> 32);
+    d.threshold = (uint32_t)__builtin_rint((double)p * 65536.0);
+    const float keep = (float)(1.0 - (double)p);
+    d.scale = p >= 1.f ? 0.f : (float)(1.0 / (double)keep);
+    return NEOX_OK;
+}
+
+// The keep pattern of the dropout kernels, one byte per element (1 = kept).
+__global__ __launch_bounds__(256) void keep_mask_kernel(uint8_t* keep, DropoutArgs d, uint64_t n) {
+    const uint64_t group = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (group * 8 >= n) return;
+    const uint32_t bits = keep_bits8(d, group);
+    for (int k = 0; k < 8; ++k)
+        if (group * 8 + k < n) keep[group * 8 + k] = (bits >> k) & 1u;
+}
+
 // Plain copy with the same access shape (measurement aid).
 __global__ __launch_bounds__(256) void copy_kernel(u32x4* dst, const u32x4* src, size_t n16) {
     size_t idx = (size_t)blockIdx.x * 1024 + threadIdx.x;
@@ -190,6 +214,125 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     a.sk = sk;
     const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
     return check_launch(launch_softmax_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_causal_softmax_dropout_fwd";
+    if (!y_drop || !y || !x) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (y_drop == y) return fail(NEOX_ERR_BAD_STRIDE, "%s: y_drop must not alias y", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
+    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(y_drop, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
+    a.out = y;
+    a.out2 = y_drop;
+    a.in0 = x;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)(batches * sq);
+    a.sq = sq;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(y_drop, 16);
+    return check_launch(launch_softmax_dropout_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    int32_t sk, int32_t dtype, void* stream) {
+    static const char* what = "neox_causal_softmax_dropout_bwd";
+    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
+    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
+    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
+    a.out = dx;
+    a.in0 = dy;
+    a.in1 = y;
+    a.scale = scale;
+    a.rows = (uint32_t)(batches * sq);
+    a.sq = sq;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_dropout_bwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
+                                    float scale, float p, uint64_t seed, uint64_t offset, int32_t b,
+                                    int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                    int32_t dtype, void* stream) {
+    static const char* what = "neox_masked_softmax_dropout_fwd";
+    if (!y_drop || !y || !x || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (y_drop == y) return fail(NEOX_ERR_BAD_STRIDE, "%s: y_drop must not alias y", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+    if (mask_b != 1 && mask_b != b)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
+    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(y_drop, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
+    a.out = y;
+    a.out2 = y_drop;
+    a.in0 = x;
+    a.mask = mask;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)((int64_t)b * np * sq);
+    a.sq = sq;
+    a.sk = sk;
+    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
+    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
+    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(y_drop, 16) &&
+                        aligned(mask, 8);
+    return check_launch(launch_softmax_dropout_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t rows, int32_t sk,
+                                    int32_t dtype, void* stream) {
+    static const char* what = "neox_masked_softmax_dropout_bwd";
+    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (int e = check_rows(rows, 1, sk, what)) return e;
+    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
+    a.out = dx;
+    a.in0 = dy;
+    a.in1 = y;
+    a.scale = scale;
+    a.rows = (uint32_t)rows;
+    a.sq = 1;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
+    return check_launch(launch_softmax_dropout_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset, int64_t n,
+                           void* stream) {
+    static const char* what = "neox_dropout_keep_mask";
+    if (!keep) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
+    if (n < 1 || n > (int64_t)1 << 40) return fail(NEOX_ERR_BAD_SHAPE, "%s: n=%lld outside [1, 2^40]", what, (long long)n);
+    DropoutArgs d{};
+    if (int e = make_dropout(d, p, seed, offset, what)) return e;
+    const uint64_t groups = ((uint64_t)n + 7) / 8;
+    hipLaunchKernelGGL(keep_mask_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, keep, d, (uint64_t)n);
+    return check_launch(hipGetLastError(), what);
 }
 
 int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np) {

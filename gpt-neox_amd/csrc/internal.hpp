@@ -19,6 +19,11 @@ hipError_t launch_softmax_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool v
                               hipStream_t stream);
 hipError_t launch_softmax_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                               hipStream_t stream);
+// The same with attention dropout fused in (a.drop, and a.out2 for the forward pass).
+hipError_t launch_softmax_dropout_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                      hipStream_t stream);
+hipError_t launch_softmax_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                      hipStream_t stream);
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream);
 

@@ -24,118 +24,120 @@ static bool wants_alibi(const SoftmaxArgs& a) {
     return !BWD && M == Mask::Causal && a.slopes != nullptr;
 }
 
-template <typename T, Mask M, bool BWD, int NCH, int WPR, int RPB>
+template <typename T, Mask M, bool BWD, int EXTRA, int NCH, int WPR, int RPB>
 static hipError_t launch_shape(const SoftmaxArgs& a, hipStream_t st) {
     const dim3 grid((a.rows + RPB - 1) / RPB);
     const dim3 block(kWave * WPR * RPB);
+    constexpr int FLAGS = kDefaultFlags | EXTRA;
     if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M>), grid, block, 0, st, a);
+        hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
     } else {
-        if constexpr (M == Mask::Causal) {
+        if constexpr (M == Mask::Causal && EXTRA == 0) {
             if (wants_alibi<M, BWD>(a)) {
-                hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, kDefaultFlags | kAlibi>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS | kAlibi>), grid, block, 0, st, a);
                 return hipGetLastError();
             }
         }
-        hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M>), grid, block, 0, st, a);
+        hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
     }
     return hipGetLastError();
 }
 
-template <typename T, Mask M, bool BWD>
+template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t launch_generic(const SoftmaxArgs& a, hipStream_t st) {
     const dim3 grid(a.rows);
     const dim3 block(kGenericThreads);
     if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_generic_kernel<T, M>), grid, block, 0, st, a);
+        hipLaunchKernelGGL((softmax_bwd_generic_kernel<T, M, EXTRA>), grid, block, 0, st, a);
     } else {
-        hipLaunchKernelGGL((softmax_fwd_generic_kernel<T, M>), grid, block, 0, st, a);
+        hipLaunchKernelGGL((softmax_fwd_generic_kernel<T, M, EXTRA>), grid, block, 0, st, a);
     }
     return hipGetLastError();
 }
 
-template <typename T, Mask M, bool BWD, int G, int R, int C>
+template <typename T, Mask M, bool BWD, int EXTRA, int G, int R, int C>
 static hipError_t launch_packed_shape(const SoftmaxArgs& a, hipStream_t st) {
     const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
     const dim3 grid((a.rows + per_block - 1) / per_block);
+    constexpr int FLAGS = kDefaultFlags | EXTRA;
     if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
     } else {
-        if constexpr (M == Mask::Causal) {
+        if constexpr (M == Mask::Causal && EXTRA == 0) {
             if (wants_alibi<M, BWD>(a)) {
-                hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags | kAlibi, R, C>), grid, dim3(256), 0, st, a);
+                hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS | kAlibi, R, C>), grid, dim3(256), 0, st, a);
                 return hipGetLastError();
             }
         }
-        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, kDefaultFlags, R, C>), grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
     }
     return hipGetLastError();
 }
 
-template <typename T, Mask M, bool BWD, int G>
+template <typename T, Mask M, bool BWD, int EXTRA, int G>
 static hipError_t launch_packed(const SoftmaxArgs& a, hipStream_t st) {
     // passes per wave: 4 everywhere except the causal forward of the longer packed rows,
     // which measured 15 % faster with 2
     constexpr int R = (!BWD && M == Mask::Causal && G >= 32) ? 2 : kPackedPasses;
-    return launch_packed_shape<T, M, BWD, G, R, 1>(a, st);
+    return launch_packed_shape<T, M, BWD, EXTRA, G, R, 1>(a, st);
 }
 
 // sk <= 512: lane groups of G = pow2 >= sk/8 lanes per row
-template <typename T, Mask M, bool BWD>
+template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
     const int lanes = (a.sk + kVec - 1) / kVec;
-    if (lanes <= 1) return launch_packed<T, M, BWD, 1>(a, st);
-    if (lanes <= 2) return launch_packed<T, M, BWD, 2>(a, st);
-    if (lanes <= 4) return launch_packed<T, M, BWD, 4>(a, st);
-    if (lanes <= 8) return launch_packed<T, M, BWD, 8>(a, st);
-    if (lanes <= 16) return launch_packed<T, M, BWD, 16>(a, st);
-    if (lanes <= 32) return launch_packed<T, M, BWD, 32>(a, st);
-    return launch_packed<T, M, BWD, 64>(a, st);
+    if (lanes <= 1) return launch_packed<T, M, BWD, EXTRA, 1>(a, st);
+    if (lanes <= 2) return launch_packed<T, M, BWD, EXTRA, 2>(a, st);
+    if (lanes <= 4) return launch_packed<T, M, BWD, EXTRA, 4>(a, st);
+    if (lanes <= 8) return launch_packed<T, M, BWD, EXTRA, 8>(a, st);
+    if (lanes <= 16) return launch_packed<T, M, BWD, EXTRA, 16>(a, st);
+    if (lanes <= 32) return launch_packed<T, M, BWD, EXTRA, 32>(a, st);
+    return launch_packed<T, M, BWD, EXTRA, 64>(a, st);
 }
 
-template <typename T, Mask M, bool BWD>
+template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     const int chunks = (a.sk + kChunk - 1) / kChunk;
-    if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD>(a, st);
+    if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD, EXTRA>(a, st);
     if (chunks == 1) {
         // the forward mask kernel addresses the mask through one 32-bit-sized buffer
         const bool mask_ok = BWD || M != Mask::Bytes || a.mask_bytes != 0;
-        if (mask_ok) return dispatch_packed<T, M, BWD>(a, st);
-        return launch_shape<T, M, BWD, 1, 1, 4>(a, st);
+        if (mask_ok) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
+        return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
     }
     if constexpr (BWD && M == Mask::None) {
         // full rows up to 2048 columns: straight-line packed kernel, R x C = 4 accesses per tensor
-        if (chunks == 2) return launch_packed_shape<T, M, BWD, kWave, 2, 2>(a, st);
-        if (chunks == 3) return launch_packed_shape<T, M, BWD, kWave, 1, 3>(a, st);
-        if (chunks == 4) return launch_packed_shape<T, M, BWD, kWave, 1, 4>(a, st);
+        if (chunks == 2) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
+        if (chunks == 3) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
+        if (chunks == 4) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 4>(a, st);
     }
-    if (chunks == 2) return launch_shape<T, M, BWD, 2, 1, 4>(a, st);
-    if (chunks <= 4) return launch_shape<T, M, BWD, 2, 2, 2>(a, st);
-    if (chunks <= 8) return launch_shape<T, M, BWD, 2, 4, 1>(a, st);
-    if (chunks <= 16) return launch_shape<T, M, BWD, 2, 8, 1>(a, st);
-    if (chunks <= 32) return launch_shape<T, M, BWD, 2, 16, 1>(a, st);
-    if (chunks <= 48) return launch_shape<T, M, BWD, 3, 16, 1>(a, st);
-    return launch_shape<T, M, BWD, 4, 16, 1>(a, st);
+    if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
+    if (chunks <= 4) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
+    if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
+    if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);
+    if (chunks <= 32) return launch_shape<T, M, BWD, EXTRA, 2, 16, 1>(a, st);
+    if (chunks <= 48) return launch_shape<T, M, BWD, EXTRA, 3, 16, 1>(a, st);
+    return launch_shape<T, M, BWD, EXTRA, 4, 16, 1>(a, st);
 }
 
-template <bool BWD>
+template <bool BWD, int EXTRA = 0>
 static hipError_t dispatch_softmax(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                    hipStream_t st) {
     const bool f16 = (dtype == NEOX_F16);
     switch (mask) {
         case Mask::Causal:
-            return f16 ? dispatch_rows<F16, Mask::Causal, BWD>(a, vec_ok, st)
-                       : dispatch_rows<BF16, Mask::Causal, BWD>(a, vec_ok, st);
+            return f16 ? dispatch_rows<F16, Mask::Causal, BWD, EXTRA>(a, vec_ok, st)
+                       : dispatch_rows<BF16, Mask::Causal, BWD, EXTRA>(a, vec_ok, st);
         case Mask::Bytes:
             if constexpr (!BWD) {
-                return f16 ? dispatch_rows<F16, Mask::Bytes, BWD>(a, vec_ok, st)
-                           : dispatch_rows<BF16, Mask::Bytes, BWD>(a, vec_ok, st);
+                return f16 ? dispatch_rows<F16, Mask::Bytes, BWD, EXTRA>(a, vec_ok, st)
+                           : dispatch_rows<BF16, Mask::Bytes, BWD, EXTRA>(a, vec_ok, st);
             }
             [[fallthrough]];  // the backward pass needs no mask: masked probabilities are 0
         case Mask::None:
             if constexpr (BWD) {
-                return f16 ? dispatch_rows<F16, Mask::None, BWD>(a, vec_ok, st)
-                           : dispatch_rows<BF16, Mask::None, BWD>(a, vec_ok, st);
+                return f16 ? dispatch_rows<F16, Mask::None, BWD, EXTRA>(a, vec_ok, st)
+                           : dispatch_rows<BF16, Mask::None, BWD, EXTRA>(a, vec_ok, st);
             }
             break;
     }

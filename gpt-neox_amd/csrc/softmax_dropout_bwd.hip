@@ -1,0 +1,11 @@
+// Backward softmax kernels with attention dropout fused in, and their launcher.
+#include "softmax_dispatch.hpp"
+
+namespace neox {
+
+hipError_t launch_softmax_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                      hipStream_t stream) {
+    return dispatch_softmax<true, kDropout>(a, mask, dtype, vec_ok, stream);
+}
+
+}  // namespace neox

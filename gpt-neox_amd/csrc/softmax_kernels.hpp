@@ -17,6 +17,7 @@
 // one reciprocal per row, one rounding to the storage type on store.
 #pragma once
 
+#include "philox.hpp"
 #include "wave.hpp"
 
 namespace neox {
@@ -35,6 +36,8 @@ struct SoftmaxArgs {
     uint32_t mask_bytes;           // size of the mask tensor, 0 if it does not fit 32 bits
     const float* slopes;           // ALiBi (kAlibi kernels): one slope per head, fp32 [np]
     uint32_t np;                   // heads per sample (kAlibi kernels)
+    void* out2;                    // kDropout forward: the probabilities after dropout
+    DropoutArgs drop;              // kDropout kernels
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -43,7 +46,17 @@ enum class Mask { Causal, Bytes, None };
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
 constexpr int kNtStore = 2;  // non-temporal hint on the streaming stores
 constexpr int kAlibi = 4;    // causal forward adds the ALiBi bias -slope[head]*(i - j) to the scores
+// Attention dropout fused in.  Forward: besides y (kept for the backward pass) the kernel
+// stores dropout(y) = keep ? round(y)*1/(1-p) : 0 to out2.  Backward: the incoming gradient is
+// the gradient of dropout(y); the kernel regenerates the keep pattern and uses
+// dy*keep/(1-p) in fp32 where the plain kernel uses dy.
+constexpr int kDropout = 8;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
+
+// Philox group (8 consecutive elements) of column `col` (a multiple of 8) of row `row`
+__device__ __forceinline__ uint64_t drop_group(uint32_t row, int sk, int col) {
+    return (uint64_t)row * (uint32_t)(sk >> 3) + (uint32_t)(col >> 3);
+}
 
 // Where a wave works: the row, its position i inside its [sq, sk] matrix, the number of
 // columns that take part, and whether the result is stored (surplus waves of the last
@@ -207,16 +220,34 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         // ---- normalise and store; chunks above the diagonal store zeros
         char* y = static_cast<char*>(a.out) + (size_t)pos.row * sk * 2;
         const rsrc_t ry = make_rsrc(y, pos.store ? (uint32_t)sk * 2u : 0u);
+        rsrc_t ry2 = ry;
+        if constexpr ((FLAGS & kDropout) != 0) {
+            ry2 = make_rsrc(static_cast<char*>(a.out2) + (size_t)pos.row * sk * 2, pos.store ? (uint32_t)sk * 2u : 0u);
+        }
+        u32x4 o[NCH];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
-            u32x4 o = u32x4{0, 0, 0, 0};
+            o[c] = u32x4{0, 0, 0, 0};
             if (c0 < len) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) v[c][k] *= inv;
-                o = pack8<T>(v[c]);
+                o[c] = pack8<T>(v[c]);
             }
-            buf_st128<kStNt>(ry, o, voff + c * WPR * kChunk * 2, 0);
+            buf_st128<kStNt>(ry, o[c], voff + c * WPR * kChunk * 2, 0);
+        }
+        if constexpr ((FLAGS & kDropout) != 0) {
+            // second output after the first: each stream is written in runs of whole rows
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const int c0 = (wir + WPR * c) * kChunk;
+                u32x4 o2 = u32x4{0, 0, 0, 0};
+                if (c0 < len) {
+                    const uint32_t bits = keep_bits8(a.drop, drop_group(pos.row, sk, c0) + lane);
+                    o2 = dropout8<T>(o[c], bits, a.drop.scale);
+                }
+                buf_st128<kStNt>(ry2, o2, voff + c * WPR * kChunk * 2, 0);
+            }
         }
     }
 }
@@ -254,14 +285,21 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
 
         // the row stays packed; it is unpacked once for the dot product and once for dx
         float dot = 0.f;
+        uint32_t kb[NCH];  // keep bits of the lane's 8 columns per chunk (kDropout)
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
+            kb[c] = 0xffu;
             if (c0 < len) {
                 float gv[8], pv[8];
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
                 const int col = c0 + lane * kVec;
+                if constexpr ((FLAGS & kDropout) != 0) {
+                    kb[c] = keep_bits8(a.drop, drop_group(pos.row, sk, c0) + lane);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
+                }
                 if (c0 + kChunk > len) {
                     // the lane holding the diagonal may have loaded columns past it
 #pragma unroll
@@ -288,6 +326,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                 const int col = c0 + lane * kVec;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
+                    if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
                     gv[k] = a.scale * (pv[k] * (gv[k] - dot));
                     if ((c0 + kChunk > len) && (col + k) >= len) gv[k] = 0.f;
                 }
@@ -348,6 +387,10 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)row0 * sk * 2, rows_here * sk * 2);
     const rsrc_t ry = make_rsrc(static_cast<char*>(a.out) + (size_t)row0 * sk * 2, rows_here * sk * 2);
     const rsrc_t rm = make_rsrc(a.mask, a.mask_bytes);
+    rsrc_t ry2 = ry;
+    if constexpr ((FLAGS & kDropout) != 0) {
+        ry2 = make_rsrc(static_cast<char*>(a.out2) + (size_t)row0 * sk * 2, rows_here * sk * 2);
+    }
 
     u32x4 raw[R][C];
     u32x2 mk[R][C];
@@ -435,7 +478,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[c][k] *= inv;  // lanes of absent rows hold NaN and store nothing
             const bool st = lr < rows_here && col < sk;
-            buf_st128<kStNt>(ry, pack8<T>(v[c]), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            const u32x4 o = pack8<T>(v[c]);
+            buf_st128<kStNt>(ry, o, st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            if constexpr ((FLAGS & kDropout) != 0) {
+                const uint32_t bits = keep_bits8(a.drop, drop_group(row0 + lr, sk, col));
+                buf_st128<kStNt>(ry2, dropout8<T>(o, bits, a.drop.scale), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            }
         }
     }
 }
@@ -479,19 +527,23 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     for (int p = 0; p < R; ++p) {
         // the row stays packed; it is unpacked once for the dot product and once for dx
         float dot = 0.f;
+        uint32_t kb[C];  // keep bits of the lane's 8 columns per chunk (kDropout)
+        const uint32_t lr = p * RPP + grp;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             float gv[8], pv[8];
             unpack8<T>(rg[p][c], gv);
             unpack8<T>(rp[p][c], pv);
+            kb[c] = 0xffu;
+            if constexpr ((FLAGS & kDropout) != 0) kb[c] = keep_bits8(a.drop, drop_group(row0 + lr, sk, col0 + c * kChunk));
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
+                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
                 if ((col0 + c * kChunk + k) >= len[p]) pv[k] = 0.f;  // past the diagonal / row end
                 dot = fmaf(gv[k], pv[k], dot);
             }
         }
         dot = group_reduce<OpSum, G>(dot);
-        const uint32_t lr = p * RPP + grp;
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
@@ -500,6 +552,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             unpack8<T>(rp[p][c], pv);
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
+                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
                 gv[k] = a.scale * (pv[k] * (gv[k] - dot));
                 if ((col + k) >= len[p]) gv[k] = 0.f;
             }
@@ -530,7 +583,13 @@ __device__ __forceinline__ float block_reduce(float v, float* red) {
     return Op::dec(r);
 }
 
-template <typename T, Mask MASK>
+// keep bit of one element (any alignment): its group's block, its 16-bit field
+__device__ __forceinline__ bool keep_element(const DropoutArgs& d, uint32_t row, int sk, int j) {
+    const uint64_t e = (uint64_t)row * (uint32_t)sk + (uint32_t)j;
+    return (keep_bits8(d, e >> 3) >> (uint32_t)(e & 7u)) & 1u;
+}
+
+template <typename T, Mask MASK, int FLAGS = 0>
 __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(SoftmaxArgs a) {
     __shared__ float red[kGenericThreads / kWave];
     const uint32_t row = blockIdx.x;
@@ -583,10 +642,16 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
             o = e * inv;
         }
         Elem<T>::store1(y + (size_t)j * 2, o);
+        if constexpr ((FLAGS & kDropout) != 0) {
+            float rounded, unused;
+            Elem<T>::unpack(Elem<T>::pack(o, 0.f), rounded, unused);
+            const bool keep = j < len && keep_element(a.drop, row, sk, j);
+            Elem<T>::store1(static_cast<char*>(a.out2) + ((size_t)row * sk + j) * 2, keep ? rounded * a.drop.scale : 0.f);
+        }
     }
 }
 
-template <typename T, Mask MASK>
+template <typename T, Mask MASK, int FLAGS = 0>
 __global__ __launch_bounds__(kGenericThreads) void softmax_bwd_generic_kernel(SoftmaxArgs a) {
     __shared__ float red[kGenericThreads / kWave];
     const uint32_t row = blockIdx.x;
@@ -597,15 +662,20 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_bwd_generic_kernel(So
     const char* p = static_cast<const char*>(a.in1) + (size_t)row * sk * 2;
     char* dx = static_cast<char*>(a.out) + (size_t)row * sk * 2;
 
+    auto grad = [&](int j) {
+        float gj = Elem<T>::load1(g + (size_t)j * 2);
+        if constexpr ((FLAGS & kDropout) != 0) gj = keep_element(a.drop, row, sk, j) ? gj * a.drop.scale : 0.f;
+        return gj;
+    };
     float dot = 0.f;
     for (int j = threadIdx.x; j < len; j += kGenericThreads)
-        dot = fmaf(Elem<T>::load1(g + (size_t)j * 2), Elem<T>::load1(p + (size_t)j * 2), dot);
+        dot = fmaf(grad(j), Elem<T>::load1(p + (size_t)j * 2), dot);
     dot = block_reduce<OpSum>(dot, red);
 
     for (int j = threadIdx.x; j < sk; j += kGenericThreads) {
         float o = 0.f;
         if (j < len) {
-            const float gj = Elem<T>::load1(g + (size_t)j * 2);
+            const float gj = grad(j);
             const float pj = Elem<T>::load1(p + (size_t)j * 2);
             o = a.scale * (pj * (gj - dot));
         }

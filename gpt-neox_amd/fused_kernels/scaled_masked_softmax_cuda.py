@@ -15,7 +15,7 @@ from .. import _lib
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def forward(input, mask, scale_factor):
+def _check_forward(input, mask):
     if input.dim() != 4:
         raise RuntimeError("expected 4D tensor")
     if input.dtype not in _HALF:
@@ -31,8 +31,13 @@ def forward(input, mask, scale_factor):
     if mask.dtype not in (torch.bool, torch.uint8):
         raise RuntimeError("mask must be a bool or uint8 tensor")
     _lib.require_gpu(input, mask)
-    input = input.contiguous()
-    mask = mask.contiguous()
+    return input.contiguous(), mask.contiguous()
+
+
+def forward(input, mask, scale_factor):
+    input, mask = _check_forward(input, mask)
+    b, np_, sq, sk = input.shape
+    pad_batches = mask.size(0)
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
@@ -47,8 +52,7 @@ def forward(input, mask, scale_factor):
     return softmax_results
 
 
-def backward(output_grads, softmax_results, scale_factor):
-    """Returns d(input), written into ``output_grads`` itself when it is contiguous."""
+def _check_backward(output_grads, softmax_results):
     if output_grads.dim() != 4 or softmax_results.dim() != 4:
         raise RuntimeError("expected 4D tensor")
     if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
@@ -56,8 +60,12 @@ def backward(output_grads, softmax_results, scale_factor):
     if output_grads.dtype != softmax_results.dtype or output_grads.shape != softmax_results.shape:
         raise RuntimeError("output_grads and softmax_results must have the same dtype and shape")
     _lib.require_gpu(output_grads, softmax_results)
-    output_grads = output_grads.contiguous()
-    softmax_results = softmax_results.contiguous()
+    return output_grads.contiguous(), softmax_results.contiguous()
+
+
+def backward(output_grads, softmax_results, scale_factor):
+    """Returns d(input), written into ``output_grads`` itself when it is contiguous."""
+    output_grads, softmax_results = _check_backward(output_grads, softmax_results)
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
@@ -67,6 +75,49 @@ def backward(output_grads, softmax_results, scale_factor):
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
                 float(scale_factor), b * np_ * sq, sk, _lib.dtype_code(output_grads.dtype),
                 _lib.current_stream(output_grads),
+            )
+        )
+    return output_grads
+
+
+def forward_dropout(input, mask, scale_factor, p, seed, offset):
+    """Mask-tensor softmax and the attention dropout that follows it, in one kernel.
+
+    Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
+    and ``dropout(softmax_results, p)`` as ``torch.nn.Dropout`` computes it from them, with
+    the keep pattern drawn from Philox state ``(seed, offset)``
+    (megatron/model/transformer.py:533-539).  No counterpart in the reference's extension.
+    """
+    input, mask = _check_forward(input, mask)
+    b, np_, sq, sk = input.shape
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    dropped = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results, dropped
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_masked_softmax_dropout_fwd(
+                dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
+                float(scale_factor), float(p), int(seed), int(offset), b, np_, sq, sk, mask.size(0),
+                _lib.dtype_code(input.dtype), _lib.current_stream(input),
+            )
+        )
+    return softmax_results, dropped
+
+
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset):
+    """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
+    that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
+    output_grads, softmax_results = _check_backward(output_grads, softmax_results)
+    b, np_, sq, sk = output_grads.shape
+    if output_grads.numel() == 0:
+        return output_grads
+    with torch.cuda.device(output_grads.device):
+        _lib.check(
+            _lib.lib().neox_masked_softmax_dropout_bwd(
+                output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
+                float(scale_factor), float(p), int(seed), int(offset), b * np_ * sq, sk,
+                _lib.dtype_code(output_grads.dtype), _lib.current_stream(output_grads),
             )
         )
     return output_grads

@@ -90,3 +90,59 @@ def backward(output_grads, softmax_results, scale_factor):
             )
         )
     return output_grads
+
+
+def forward_dropout(input, scale_factor, p, seed, offset):
+    """Causal softmax and the attention dropout that follows it, in one kernel.
+
+    Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
+    and ``dropout(softmax_results, p)`` as ``torch.nn.Dropout`` computes it from them, with
+    the keep pattern drawn from Philox state ``(seed, offset)``
+    (megatron/model/transformer.py:533-539).  No counterpart in the reference's extension.
+    """
+    if input.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    _lib.require_gpu(input)
+    input = input.contiguous()
+    attn_batches, sq, sk = input.shape
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    dropped = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results, dropped
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_dropout_fwd(
+                dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), float(scale_factor),
+                float(p), int(seed), int(offset), attn_batches, sq, sk, _lib.dtype_code(input.dtype),
+                _lib.current_stream(input),
+            )
+        )
+    return softmax_results, dropped
+
+
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset):
+    """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
+    that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
+    if output_grads.dim() != 3 or softmax_results.dim() != 3:
+        raise RuntimeError("expected 3D tensor")
+    if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    if output_grads.dtype != softmax_results.dtype or output_grads.shape != softmax_results.shape:
+        raise RuntimeError("output_grads and softmax_results must have the same dtype and shape")
+    _lib.require_gpu(output_grads, softmax_results)
+    output_grads = output_grads.contiguous()
+    softmax_results = softmax_results.contiguous()
+    attn_batches, sq, sk = output_grads.shape
+    if output_grads.numel() == 0:
+        return output_grads
+    with torch.cuda.device(output_grads.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_dropout_bwd(
+                output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
+                float(scale_factor), float(p), int(seed), int(offset), attn_batches, sq, sk,
+                _lib.dtype_code(output_grads.dtype), _lib.current_stream(output_grads),
+            )
+        )
+    return output_grads

@@ -36,6 +36,7 @@ import weakref
 
 import torch
 
+from .fused_kernels import attention_dropout as _rng
 from .fused_kernels import load_fused_kernels
 from .fused_kernels import scaled_masked_softmax_cuda as _masked_ext
 from .fused_kernels import scaled_upper_triang_masked_softmax_cuda as _causal_ext
@@ -168,6 +169,50 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
         return _masked_ext.backward(output_grads, probs, scale), None, None
 
 
+class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
+    """Causal softmax followed by dropout with probability ``p``, in one kernel per pass.
+
+    Returns ``dropout(softmax(scale * inputs))`` -- what the reference obtains from the
+    softmax and ``self.attention_dropout`` (megatron/model/transformer.py:533-539).  The keep
+    pattern comes from the device's default generator (see ``fused_kernels.attention_dropout``),
+    so call it where the reference calls the dropout: inside the RNG tracker's ``fork()``.
+    The undropped probabilities are kept for the backward pass; the pattern is regenerated
+    there from the saved generator state instead of being stored."""
+
+    @staticmethod
+    def forward(ctx, inputs, scale, p):
+        scale_t = _scale_tensor(scale)
+        seed, offset = _rng.take_philox_state(inputs.device)
+        probs, dropped = _causal_ext.forward_dropout(inputs, scale_t[0].item(), p, seed, offset)
+        ctx.save_for_backward(probs, scale_t)
+        ctx.dropout = (p, seed, offset)
+        return dropped
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        return _causal_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout), None, None
+
+
+class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
+    """Mask-tensor softmax followed by dropout with probability ``p``, in one kernel per
+    pass; see ``ScaledUpperTriangMaskedSoftmaxDropout``."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale, p):
+        scale_t = _scale_tensor(scale)
+        seed, offset = _rng.take_philox_state(inputs.device)
+        probs, dropped = _masked_ext.forward_dropout(inputs, mask, scale_t[0].item(), p, seed, offset)
+        ctx.save_for_backward(probs, scale_t)
+        ctx.dropout = (p, seed, offset)
+        return dropped
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        return _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout), None, None, None
+
+
 class SoftmaxFusionTypes(enum.Enum):
     upper_triang = 1  # causal mask
     general = 2  # general mask
@@ -203,12 +248,19 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         if self.fusion:
             load_fused_kernels()  # ImportError here, not at the first forward
 
-    def forward(self, input, mask, alibi_slopes=None):
+    def forward(self, input, mask, alibi_slopes=None, dropout_p=0.0):
         """``alibi_slopes`` (optional, ``[np]``) is an addition to the reference signature:
         ``forward(scores, mask, alibi_slopes=alibi.slopes)`` equals
         ``forward(alibi(scores), mask)`` (megatron/model/transformer.py:529-534) with the bias
-        evaluated in fp32 inside the causal kernel instead of a separate pass in half precision."""
+        evaluated in fp32 inside the causal kernel instead of a separate pass in half precision.
+
+        ``dropout_p`` (optional, training only) is the second addition:
+        ``forward(scores, mask, dropout_p=p)`` equals ``dropout(forward(scores, mask), p)``
+        (megatron/model/transformer.py:533-539) and is to be called where the reference calls
+        the dropout, inside the RNG tracker's ``fork()``."""
         assert input.dim() == 4  # [b, np, sq, sk]
+        if dropout_p:
+            return self.forward_with_dropout(input, mask, alibi_slopes, dropout_p)
         fused = self.is_kernel_available(mask, *input.size())
         if alibi_slopes is not None:
             b, np, sq, sk = input.size()
@@ -217,6 +269,24 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
                 return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
             input = input + alibi_bias(alibi_slopes, sq, sk, input.device, input.dtype)
         return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
+
+    def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p):
+        """Softmax and dropout in one kernel when the fused softmax serves the call, there is
+        no ALiBi bias and no HIP graph is being captured (the generator state would be frozen
+        into the graph); otherwise the softmax above followed by torch's dropout."""
+        b, np, sq, sk = input.size()
+        fusable = (
+            alibi_slopes is None
+            and self.is_kernel_available(mask, b, np, sq, sk)
+            and not torch.cuda.is_current_stream_capturing()
+        )
+        if not fusable:
+            return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes), dropout_p, True)
+        scale = 1.0 if self.scale is None else self.scale
+        if self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
+            probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(-1, sq, sk), scale, dropout_p)
+            return probs.view(b, np, sq, sk)
+        return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """Whether the fused branch serves this call.

@@ -107,6 +107,39 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
                             int32_t sk, int32_t dtype, void* stream);
 
 /*
+ * Softmax with the attention dropout that follows it folded in (training only).
+ * Forward stores two tensors: y, the probabilities exactly as neox_*_softmax_fwd gives
+ * them (the backward pass needs them), and y_drop = keep ? round(float(y) / (1-p)) : 0,
+ * which is what torch.nn.Dropout computes from y; y_drop must not alias y.  Backward
+ * takes dy = the gradient of y_drop, regenerates the keep pattern and returns
+ *   dx = scale * y * (g - sum_j(g*y)),  g = keep ? dy / (1-p) : 0  (fp32, never stored).
+ * Keep pattern: Philox4x32-10 with key = seed and counter = (offset, e / 8), e the
+ * row-major element index into the score tensor; element e owns the 16-bit field e % 8 of
+ * its block and is kept iff field >= round(p * 65536).  neox_dropout_keep_mask writes that
+ * pattern as bytes (1 = kept) for n elements.  (seed, offset) are the device generator's
+ * Philox state; a call consumes one counter value per group, so the caller advances the
+ * generator's offset by 4 (torch's granularity) per call.  0 <= p <= 1.
+ * Replaces scaled_*_softmax_cuda.forward/backward followed by the attention dropout
+ *   megatron/model/transformer.py:533-539 (softmax, then dropout under the RNG tracker)
+ *   megatron/mpu/random.py:20-37 (the tracker that selects the generator state)
+ */
+int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    int32_t sk, int32_t dtype, void* stream);
+int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    int32_t sk, int32_t dtype, void* stream);
+int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
+                                    float scale, float p, uint64_t seed, uint64_t offset, int32_t b,
+                                    int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                    int32_t dtype, void* stream);
+int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int64_t rows, int32_t sk,
+                                    int32_t dtype, void* stream);
+int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset, int64_t n,
+                           void* stream);
+
+/*
  * Rows-per-block figure the reference's dispatcher predicate consumes; kept for
  * API compatibility (wave64 values).  Pure host arithmetic.
  * Replaces scaled_masked_softmax_cuda.get_batch_per_block

@@ -7,6 +7,10 @@ it is used by ``tests/``, by ``__graft_entry__.smoke()`` and by the
 * ``torch_ref``  -- the reference's torch expressions, restated op for op.
 * ``brute``      -- an independent float64 evaluation with Python/numpy loops, used
                     to pin ``torch_ref`` on small inputs.
+* ``philox``     -- Philox4x32-10 and the element -> random bits assignment of the fused
+                    attention-dropout kernels, in numpy; pinned by Random123's published
+                    known-answer vectors, a per-element pure-Python restatement, and (on
+                    the GPU) ``torch.rand``, which consumes the same block function.
 
 Pins (tests/test_oracle_*.py): the reference ships no golden vectors, fixtures or
 asserting tests for this path, so every function here is pinned by closed forms,

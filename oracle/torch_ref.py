@@ -100,6 +100,34 @@ def softmax_autograd_fp32(x, mask, scale, grad_out):
     return y.detach(), xf.grad
 
 
+# --- attention dropout ----------------------------------------------------------------
+
+
+def dropout_scale(p):
+    """``1/(1-p)`` as torch's device dropout kernel forms it: the keep probability is
+    narrowed to fp32 and the quotient is taken from that (0 for ``p == 1``)."""
+    if p >= 1.0:
+        return 0.0
+    keep = torch.tensor(1.0 - p, dtype=torch.float32)
+    return float((1.0 / keep.double()).float())
+
+
+def dropout_with_mask(probs, keep, p):
+    """``torch.nn.Dropout(p)`` on ``probs`` for a given keep pattern, as the attention
+    dropout of megatron/model/transformer.py:536-539 computes it on the device:
+    ``probs * keep * 1/(1-p)`` in fp32, rounded once to the dtype of ``probs``."""
+    scale = torch.tensor(dropout_scale(p), dtype=torch.float32, device=probs.device)
+    return torch.where(keep, probs.float() * scale, torch.zeros((), device=probs.device)).to(probs.dtype)
+
+
+def softmax_dropout_backward_fp32(grad_out, probs, keep, p, scale):
+    """Gradient of ``dropout(softmax(scale * x))`` with respect to ``x`` in fp32:
+    the dropout's backward ``g = grad_out * keep / (1-p)`` followed by
+    ``softmax_backward_fp32`` (autograd of transformer.py:533-539)."""
+    g = torch.where(keep, grad_out.float() * dropout_scale(p), torch.zeros((), device=grad_out.device))
+    return softmax_backward_fp32(g, probs, scale)
+
+
 def alibi_slopes(n):
     """Head slopes of ALiBi: 2^(-8/n * (k+1)) for a power-of-two n, otherwise the slopes of the
     power of two below plus every second slope of the one above.

@@ -1,0 +1,351 @@
+"""Parity of the fused softmax + attention-dropout kernels (through the C-ABI) with the oracle.
+
+Bars: the keep pattern is bit-equal to oracle/philox.py; the undropped probabilities are
+bit-equal to the plain softmax kernels'; the dropped output is bit-equal to torch's
+dropout expression evaluated on those probabilities with that pattern; the backward pass
+meets the softmax bars (2e-3 bf16 / 1e-3 fp16, masked positions exactly 0) against the
+fp32 closed form.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpt_neox_amd.fused_kernels import attention_dropout as rng
+from gpt_neox_amd.fused_kernels import scaled_masked_softmax_cuda as masked_ext
+from gpt_neox_amd.fused_kernels import scaled_upper_triang_masked_softmax_cuda as causal_ext
+from gpt_neox_amd.fused_softmax import (
+    FusedScaleMaskSoftmax,
+    ScaledMaskedSoftmaxDropout,
+    ScaledUpperTriangMaskedSoftmaxDropout,
+    SoftmaxFusionTypes,
+)
+from oracle import philox
+from oracle import torch_ref as R
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-3, torch.float16: 1e-3}
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+def gen(device, seed):
+    return torch.Generator(device=device).manual_seed(seed)
+
+
+def scores(shape, dtype, device, seed):
+    return (torch.randn(shape, device=device, generator=gen(device, seed)) * 8).to(dtype)
+
+
+def normal(shape, dtype, device, seed):
+    return torch.randn(shape, device=device, generator=gen(device, seed)).to(dtype)
+
+
+def max_err(a, b):
+    return (a.float() - b.float()).abs().max().item()
+
+
+# ---------------------------------------------------------------------------------
+# the generator
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 4099, 1 << 20])
+@pytest.mark.parametrize("p,seed,offset", [(0.1, 1234, 0), (0.5, 2**63 + 5, 2**40 + 8), (0.9, 0, 4)])
+def test_keep_mask_kernel_is_bit_equal_to_the_oracle(device, n, p, seed, offset):
+    got = rng.keep_mask(n, p, seed, offset, device).cpu().numpy()
+    assert np.array_equal(got, philox.keep_mask(n, p, seed, offset))
+
+
+def test_keep_mask_edge_probabilities(device):
+    assert rng.keep_mask(5000, 0.0, 3, 0, device).all()
+    assert not rng.keep_mask(5000, 1.0, 3, 0, device).any()
+    with pytest.raises(RuntimeError, match="between 0 and 1"):
+        rng.keep_mask(8, 1.25, 3, 0, device)
+
+
+def test_oracle_philox_agrees_with_the_device_library_generator(device):
+    # torch.rand on the device draws Philox4x32-10 blocks with key = seed and
+    # counter = (offset, thread index); in a launch with one element per thread, thread t
+    # converts the first word of its block to a float in (0, 1].
+    torch.manual_seed(987654321)
+    u = torch.rand(256, device=device, dtype=torch.float32).cpu().numpy().astype(np.float64)
+    ctr = np.zeros((256, 4), dtype=np.uint64)
+    ctr[:, 2] = np.arange(256, dtype=np.uint64)
+    words = philox.philox4x32_10(ctr, (987654321, 0)).astype(np.float64)  # [256, 4]
+    want = words[:, 0] / 2.0**32  # element t <- first word of thread t's first block
+    assert np.abs(u - want).max() < 2.0**-23
+
+
+def test_dropout_scale_is_the_device_library_s(device):
+    # kept entries of torch's own dropout equal round(float(y) * scale) for the oracle's scale
+    y = torch.rand(1 << 16, device=device).to(torch.bfloat16)
+    for p in (0.1, 0.25, 0.3):
+        out = torch.nn.functional.dropout(y, p, True)
+        kept = out != 0
+        want = R.dropout_with_mask(y, kept, p)
+        assert torch.equal(out, want)
+
+
+# ---------------------------------------------------------------------------------
+# forward
+# ---------------------------------------------------------------------------------
+def check_forward(y, dropped, y_plain, p, seed, offset, device):
+    assert torch.equal(y, y_plain)  # the saved probabilities are the plain kernels'
+    keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
+    assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
+    return keep
+
+
+CAUSAL_SHAPES = [(3, 8, 8), (5, 24, 24), (2, 72, 72), (3, 128, 128), (2, 264, 264), (2, 512, 512),
+                 (2, 1024, 1024), (1, 1032, 1032), (2, 2048, 2048), (1, 4096, 4096), (1, 8192, 8192),
+                 (3, 7, 7), (2, 100, 100), (1, 1001, 1001)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", CAUSAL_SHAPES)
+def test_causal_forward(device, shape, dtype):
+    x = scores(shape, dtype, device, 3)
+    p, seed, offset = 0.1, 1234 + shape[1], 4 * shape[0]
+    y, dropped = causal_ext.forward_dropout(x, 0.125, p, seed, offset)
+    keep = check_forward(y, dropped, causal_ext.forward(x, 0.125), p, seed, offset, device)
+    if shape[1] <= 1024:
+        # the device-side pattern is the oracle's (row-major element index of the [B, sq, sk] tensor)
+        want = philox.keep_mask(x.numel(), p, seed, offset).reshape(shape)
+        assert np.array_equal(keep.cpu().numpy(), want)
+    upper = torch.triu(torch.ones(shape[1:], dtype=torch.bool, device=device), 1).expand(shape)
+    assert (dropped[upper] == 0).all()
+
+
+MASKED_SHAPES = [(2, 3, 5, 8), (2, 2, 9, 40), (1, 3, 16, 136), (2, 2, 8, 512), (2, 2, 16, 1024),
+                 (1, 2, 8, 1536), (1, 2, 8, 2048), (1, 1, 4, 4096), (1, 1, 2, 16384), (1, 1, 2, 32768),
+                 (2, 2, 5, 37), (1, 2, 3, 1001), (1, 1, 2, 40000)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", MASKED_SHAPES)
+def test_masked_forward(device, shape, dtype):
+    b, np_, sq, sk = shape
+    x = scores(shape, dtype, device, 4)
+    lengths = torch.randint(1, sk + 1, (b,), generator=gen(device, 5), device=device)
+    mask = R.padding_mask(lengths, sq, sk, device)
+    mask[0, 0, 0, :] = True  # one fully hidden row: uniform 1/sk, then dropout
+    p, seed, offset = 0.25, 99, 8
+    y, dropped = masked_ext.forward_dropout(x, mask, 0.5, p, seed, offset)
+    check_forward(y, dropped, masked_ext.forward(x, mask, 0.5), p, seed, offset, device)
+    hidden = mask.expand(shape).clone()
+    hidden[0, :, 0, :] = False
+    assert (dropped[hidden] == 0).all()
+
+
+@pytest.mark.parametrize("p", [0.0, 1.0])
+def test_forward_edge_probabilities(device, p):
+    x = scores((2, 64, 64), torch.bfloat16, device, 6)
+    y, dropped = causal_ext.forward_dropout(x, 1.0, p, 1, 0)
+    assert torch.equal(dropped, y if p == 0.0 else torch.zeros_like(y))
+
+
+# ---------------------------------------------------------------------------------
+# backward
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", CAUSAL_SHAPES)
+def test_causal_backward(device, shape, dtype):
+    x = scores(shape, dtype, device, 7)
+    g = normal(shape, dtype, device, 8)
+    p, seed, offset, scale = 0.2, 4321, 12, 0.125
+    y, _ = causal_ext.forward_dropout(x, scale, p, seed, offset)
+    keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(shape)
+    ref = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
+    dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+    assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    assert (dx[y == 0] == 0).all()
+    # in place on the gradient buffer, as the plain backward
+    buf = g.clone()
+    out = causal_ext.backward_dropout(buf, y, scale, p, seed, offset)
+    assert out.data_ptr() == buf.data_ptr() and torch.equal(out, dx)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", MASKED_SHAPES)
+def test_masked_backward(device, shape, dtype):
+    b, np_, sq, sk = shape
+    x = scores(shape, dtype, device, 9)
+    g = normal(shape, dtype, device, 10)
+    mask = R.padding_mask(torch.randint(1, sk + 1, (b,), generator=gen(device, 11), device=device), sq, sk, device)
+    p, seed, offset, scale = 0.1, 2**50 + 3, 2**33, 1.0
+    y, _ = masked_ext.forward_dropout(x, mask, scale, p, seed, offset)
+    keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(shape)
+    ref = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
+    dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+    assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    assert (dx[mask.expand(shape)] == 0).all()
+
+
+def test_backward_against_fp64_autograd_of_the_unfused_expression(device):
+    shape = (2, 3, 48, 48)
+    x = scores(shape, torch.float16, device, 12)
+    g = normal(shape, torch.float16, device, 13)
+    mask = R.get_attn_mask(48, device)
+    p, seed, offset, scale = 0.3, 5, 0, 0.25
+    y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset)
+    keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(shape)
+    xd = x.double().requires_grad_(True)
+    probs = torch.softmax((scale * xd).masked_fill(mask, float("-inf")), -1)
+    out = probs * keep / (1 - p)
+    (want,) = torch.autograd.grad(out, xd, g.double())
+    assert max_err(dropped, out) <= 2 * TOL[torch.float16] / (1 - p)
+    dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+    assert max_err(dx, want) <= 4 * TOL[torch.float16] * max(1.0, want.abs().max().item())
+
+
+# ---------------------------------------------------------------------------------
+# BASELINE shapes at full size
+# ---------------------------------------------------------------------------------
+def test_full_size_padded_config(device):
+    shape = (8, 16, 1024, 1024)
+    x = scores(shape, torch.float16, device, 1235)
+    g = normal(shape, torch.float16, device, 1236)
+    lengths = torch.randint(256, 1025, (8,), generator=gen(device, 1237), device=device)
+    mask = R.padding_mask(lengths, 1024, 1024, device)
+    p, seed, offset = 0.1, 17, 400
+    y, dropped = masked_ext.forward_dropout(x, mask, 0.125, p, seed, offset)
+    keep = check_forward(y, dropped, masked_ext.forward(x, mask, 0.125), p, seed, offset, device)
+    frac = keep.float().mean().item()
+    assert abs(frac - 0.9) < 5 * (0.09 / keep.numel()) ** 0.5 + 2.0**-16
+    dx = masked_ext.backward_dropout(g.clone(), y, 0.125, p, seed, offset)
+    for s in range(0, 8, 4):  # fp32 reference in slices
+        ref = R.softmax_dropout_backward_fp32(g[s:s + 4], y[s:s + 4], keep[s:s + 4], p, 0.125)
+        assert max_err(dx[s:s + 4], ref) <= TOL[torch.float16] * max(1.0, ref.abs().max().item())
+
+
+def test_full_size_long_causal_config(device):
+    shape = (32, 8192, 8192)
+    x = scores((4, 8192, 8192), torch.bfloat16, device, 1238).repeat(8, 1, 1)
+    p, seed, offset = 0.1, 23, 2**35
+    y, dropped = causal_ext.forward_dropout(x, 0.0884, p, seed, offset)
+    assert y.shape == shape
+    y_plain = causal_ext.forward(x, 0.0884)
+    assert torch.equal(y, y_plain)
+    del y_plain
+    for s in range(0, 32, 8):  # element indices beyond 2^31: groups are 64-bit
+        n0 = s * 8192 * 8192
+        keep = rng.keep_mask(n0 + 8 * 8192 * 8192, p, seed, offset, device)[n0:].view(8, 8192, 8192)
+        assert torch.equal(dropped[s:s + 8], R.dropout_with_mask(y[s:s + 8], keep, p))
+        del keep
+    g = normal((4, 8192, 8192), torch.bfloat16, device, 1239).repeat(8, 1, 1)
+    dx = causal_ext.backward_dropout(g.clone(), y, 0.0884, p, seed, offset)
+    s = 24
+    n0 = s * 8192 * 8192
+    keep = rng.keep_mask(n0 + 2 * 8192 * 8192, p, seed, offset, device)[n0:].view(2, 8192, 8192)
+    ref = R.softmax_dropout_backward_fp32(g[s:s + 2], y[s:s + 2], keep, p, 0.0884)
+    assert max_err(dx[s:s + 2], ref) <= TOL[torch.bfloat16] * max(1.0, ref.abs().max().item())
+    assert (dx[s:s + 2][y[s:s + 2] == 0] == 0).all()
+
+
+# ---------------------------------------------------------------------------------
+# autograd Functions, module, generator plumbing
+# ---------------------------------------------------------------------------------
+def test_functions_follow_the_default_generator(device):
+    x = scores((4, 256, 256), torch.bfloat16, device, 20).requires_grad_(True)
+    gen0 = torch.cuda.default_generators[device.index]
+    torch.manual_seed(555)
+    off0 = gen0.get_offset()
+    a = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    assert gen0.get_offset() == off0 + rng.OFFSET_STEP
+    b = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    assert not torch.equal(a, b)  # the generator moved on
+    torch.manual_seed(555)
+    c = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    assert torch.equal(a, c)  # same generator state, same pattern
+    # the call with the state spelled out
+    _, want = causal_ext.forward_dropout(x.detach(), 0.5, 0.1, 555, off0)
+    assert torch.equal(a, want)
+    # a torch random call in between shifts the pattern: the state is shared, not private
+    torch.manual_seed(555)
+    torch.rand(4, device=device)
+    d = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    assert not torch.equal(a, d)
+    # saved and restored generator state (what the RNG tracker's fork() does)
+    torch.manual_seed(777)
+    state = torch.cuda.get_rng_state(device)
+    e = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    torch.cuda.set_rng_state(state, device)
+    f = ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.1)
+    assert torch.equal(e, f)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_function_gradients(device, dtype):
+    shape = (2, 4, 128, 128)
+    x = scores(shape, dtype, device, 21).requires_grad_(True)
+    g = normal(shape, dtype, device, 22)
+    mask = R.padding_mask(torch.tensor([100, 128]), 128, 128, device)
+    torch.manual_seed(31)
+    off = torch.cuda.default_generators[device.index].get_offset()
+    out = ScaledMaskedSoftmaxDropout.apply(x, mask, 0.5, 0.15)
+    out.backward(g.clone())
+    y = masked_ext.forward(x.detach(), mask, 0.5)
+    keep = rng.keep_mask(y.numel(), 0.15, 31, off, device).view(shape)
+    assert torch.equal(out, R.dropout_with_mask(y, keep, 0.15))
+    ref = R.softmax_dropout_backward_fp32(g, y, keep, 0.15, 0.5)
+    assert max_err(x.grad, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+
+    x3 = scores((6, 128, 128), dtype, device, 23).requires_grad_(True)
+    torch.manual_seed(32)
+    off = torch.cuda.default_generators[device.index].get_offset()
+    out = ScaledUpperTriangMaskedSoftmaxDropout.apply(x3, 0.5, 0.15)
+    out.backward(g.view(8, 128, 128)[:6].clone())
+    y = causal_ext.forward(x3.detach(), 0.5)
+    keep = rng.keep_mask(y.numel(), 0.15, 32, off, device).view(y.shape)
+    ref = R.softmax_dropout_backward_fp32(g.view(8, 128, 128)[:6], y, keep, 0.15, 0.5)
+    assert max_err(x3.grad, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+
+
+def test_module_dropout_argument(device):
+    b, np_, s = 2, 4, 256
+    x = scores((b, np_, s, s), torch.bfloat16, device, 24)
+    causal = R.get_attn_mask(s, device)
+    m = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func, True, 0.5)
+    plain = m(x, causal)
+    assert torch.equal(m(x, causal, dropout_p=0.0), plain)
+    torch.manual_seed(41)
+    off = torch.cuda.default_generators[device.index].get_offset()
+    out = m(x, causal, dropout_p=0.1)
+    keep = rng.keep_mask(x.numel(), 0.1, 41, off, device).view(x.shape)
+    assert torch.equal(out, R.dropout_with_mask(plain, keep, 0.1))
+    # a sliding-window mask goes to the mask-tensor kernel, same pattern assignment
+    window = R.get_attn_mask(s, device, sliding_window_width=32)
+    torch.manual_seed(41)
+    out = m(x, window, dropout_p=0.1)
+    assert torch.equal(out, R.dropout_with_mask(m(x, window), keep, 0.1))
+    # general fusion with a padding mask
+    mg = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, None)
+    pad = R.padding_mask(torch.tensor([200, 256]), s, s, device)
+    torch.manual_seed(41)
+    out = mg(x, pad, dropout_p=0.1)
+    assert torch.equal(out, R.dropout_with_mask(mg(x, pad), keep, 0.1))
+    # with an ALiBi bias the softmax kernel is followed by torch's dropout: same law, torch's pattern
+    slopes = torch.tensor(R.alibi_slopes(np_), device=device)
+    out = m(x, causal, alibi_slopes=slopes, dropout_p=0.5)
+    base = m(x, causal, alibi_slopes=slopes)
+    kept = out != 0
+    assert torch.equal(out, R.dropout_with_mask(base, kept, 0.5))
+    lower = ~torch.triu(torch.ones(s, s, dtype=torch.bool, device=device), 1)
+    frac = kept[..., lower].float().mean().item()
+    assert 0.45 < frac < 0.55
+    # the unfused module (fusion off) takes torch's dropout as well
+    mt = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
+    out = mt(x, causal, dropout_p=0.5)
+    assert torch.equal(out, R.dropout_with_mask(mt(x, causal), out != 0, 0.5))
+
+
+def test_statistics_of_the_fused_output(device):
+    # E[dropout(y)] = y: averaged over many patterns the dropped output returns the probabilities
+    x = scores((1, 64, 64), torch.float16, device, 25)
+    y = causal_ext.forward(x, 0.25).float()
+    acc = torch.zeros_like(y)
+    n = 400
+    for i in range(n):
+        _, d = causal_ext.forward_dropout(x, 0.25, 0.3, 1000, 4 * i)
+        acc += d.float()
+    err = (acc / n - y).abs()
+    bound = 5 * y * (0.3 / 0.7 / n) ** 0.5 + 1e-3
+    assert (err <= bound).all()
