@@ -503,6 +503,25 @@ def main():
                 extras.append(drop_extras(r, z, 1, cm, sc, False))
                 del s_, z, cm
             result["fused_dropout"] = extras
+        # relative-position bias [1, np, sq, sk] read inside the causal softmax (125M shape)
+        if want("bias"):
+            Bb, H, n, dt, sc = 4, 12, 2048, torch.bfloat16, 0.125
+            s_ = causal_sets(Bb * H, n, dt, 1242, nsets=2, need_bwd=False)
+            rpe = (torch.randn(1, H, n, n, device=dev, generator=gen(1243)) * 2).to(dt)
+
+            def cb_fwd(t):
+                ok(lib.neox_causal_softmax_bias_fwd(t["y"].data_ptr(), t["x"].data_ptr(), rpe.data_ptr(), sc,
+                                                    Bb, H, n, n, 1, code[dt], stream))
+
+            r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
+                    Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
+            z = s_[0]
+            cm = R.get_attn_mask(n, dev)
+            ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
+            r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
+            r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
+            result["fused_bias"] = [r]
+            del s_, z, rpe
         result["all_configs"] = table
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
         if pcts:

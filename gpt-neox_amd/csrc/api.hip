@@ -216,6 +216,72 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     return check_launch(launch_softmax_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
 }
 
+// bias [bias_b, np, sq, sk]: shared by all samples (bias_b == 1) or one per sample
+static int set_bias(SoftmaxArgs& a, const void* bias, int b, int np, int sq, int sk, int bias_b,
+                    const char* what) {
+    if (bias_b != 1 && bias_b != b)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: bias batch dim %d must be 1 or b=%d", what, bias_b, b);
+    a.bias = bias;
+    a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * sq) : 0u;
+    const uint64_t bytes = (uint64_t)bias_b * (uint64_t)np * (uint64_t)sq * (uint64_t)sk * 2u;
+    a.bias_bytes = bytes < 0xFFFFFFFFull ? (uint32_t)bytes : 0u;
+    return NEOX_OK;
+}
+
+int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
+                                 int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
+                                 void* stream) {
+    static const char* what = "neox_causal_softmax_bias_fwd";
+    if (!y || !x || !bias) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(bias, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = set_bias(a, bias, b, np, sq, sk, bias_b, what)) return e;
+    a.out = y;
+    a.in0 = x;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)((int64_t)b * np * sq);
+    a.sq = sq;
+    a.sk = sk;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(bias, 16);
+    return check_launch(launch_softmax_bias_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
+int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
+                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
+                                 int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream) {
+    static const char* what = "neox_masked_softmax_bias_fwd";
+    if (!y || !x || !mask || !bias) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+    if (int e = check_dtype(dtype, what)) return e;
+    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+    if (mask_b != 1 && mask_b != b)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
+    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
+    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(bias, 2))
+        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+
+    SoftmaxArgs a{};
+    if (int e = set_bias(a, bias, b, np, sq, sk, bias_b, what)) return e;
+    a.out = y;
+    a.in0 = x;
+    a.mask = mask;
+    a.scale = scale * kLog2e;
+    a.rows = (uint32_t)((int64_t)b * np * sq);
+    a.sq = sq;
+    a.sk = sk;
+    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
+    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
+    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
+    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(bias, 16) &&
+                        aligned(mask, 8);
+    return check_launch(launch_softmax_bias_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+}
+
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
                                     uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream) {

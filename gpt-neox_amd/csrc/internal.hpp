@@ -24,6 +24,9 @@ hipError_t launch_softmax_dropout_fwd(const SoftmaxArgs& a, Mask mask, int dtype
                                       hipStream_t stream);
 hipError_t launch_softmax_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                       hipStream_t stream);
+// Forward with an additive bias tensor (a.bias, a.bias_rows, a.bias_bytes).
+hipError_t launch_softmax_bias_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                   hipStream_t stream);
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream);
 

@@ -101,8 +101,10 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
     if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD, EXTRA>(a, st);
     if (chunks == 1) {
         // the forward mask kernel addresses the mask through one 32-bit-sized buffer
-        const bool mask_ok = BWD || M != Mask::Bytes || a.mask_bytes != 0;
-        if (mask_ok) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
+        // and the bias kernel the bias tensor
+        const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
+                             ((EXTRA & kBias) == 0 || a.bias_bytes != 0);
+        if (fits32) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
         return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
     }
     if constexpr (BWD && M == Mask::None) {

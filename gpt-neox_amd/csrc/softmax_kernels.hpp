@@ -38,6 +38,9 @@ struct SoftmaxArgs {
     uint32_t np;                   // heads per sample (kAlibi kernels)
     void* out2;                    // kDropout forward: the probabilities after dropout
     DropoutArgs drop;              // kDropout kernels
+    const void* bias;              // kBias forward: additive bias [1 or b, np, sq, sk], dtype of x
+    uint32_t bias_rows;            // np*sq if the bias is shared by all samples, else 0
+    uint32_t bias_bytes;           // size of the bias tensor, 0 if it does not fit 32 bits
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -51,7 +54,15 @@ constexpr int kAlibi = 4;    // causal forward adds the ALiBi bias -slope[head]*
 // the gradient of dropout(y); the kernel regenerates the keep pattern and uses
 // dy*keep/(1-p) in fp32 where the plain kernel uses dy.
 constexpr int kDropout = 8;
+// Forward adds a bias tensor to the scores before the scale: softmax(scale * (x + bias)), the sum
+// taken in fp32 (the unfused path rounds x + bias to half precision first).
+constexpr int kBias = 16;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
+
+// Row of the bias tensor that belongs to score row `row`
+__device__ __forceinline__ uint32_t bias_row(uint32_t row, const SoftmaxArgs& a) {
+    return a.bias_rows ? row % a.bias_rows : row;
+}
 
 // Philox group (8 consecutive elements) of column `col` (a multiple of 8) of row `row`
 __device__ __forceinline__ uint64_t drop_group(uint32_t row, int sk, int col) {
@@ -125,13 +136,20 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     float slope2 = 0.f;
     if constexpr ((FLAGS & kAlibi) != 0) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
     u32x4 raw[NCH];
+    u32x4 rawb[NCH];  // kBias
     u32x2 mk[NCH];
     {
         // ---- issue every load of the row before the first use
         const char* x = static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2;
-        const rsrc_t rx = make_rsrc(x, (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u);
+        const uint32_t row_bytes = (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
+        const rsrc_t rx = make_rsrc(x, row_bytes);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) raw[c] = buf_ld128<kLdNt>(rx, voff + c * WPR * kChunk * 2, 0);
+        if constexpr ((FLAGS & kBias) != 0) {
+            const rsrc_t rb = make_rsrc(static_cast<const char*>(a.bias) + (size_t)bias_row(pos.row, a) * sk * 2, row_bytes);
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) rawb[c] = buf_ld128<false>(rb, voff + c * WPR * kChunk * 2, 0);
+        }
         if constexpr (MASK == Mask::Bytes) {
             const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
             const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)pos.len);
@@ -150,6 +168,12 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
             const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
             if (c0 < len) {
                 unpack8<T>(raw[c], v[c]);
+                if constexpr ((FLAGS & kBias) != 0) {
+                    float bv[8];
+                    unpack8<T>(rawb[c], bv);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) v[c][k] += bv[k];
+                }
                 const int col = c0 + lane * kVec;
                 bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
                 if constexpr (MASK == Mask::Bytes) {
@@ -391,8 +415,10 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     if constexpr ((FLAGS & kDropout) != 0) {
         ry2 = make_rsrc(static_cast<char*>(a.out2) + (size_t)row0 * sk * 2, rows_here * sk * 2);
     }
+    const rsrc_t rb = make_rsrc(a.bias, a.bias_bytes);  // kBias: the whole bias tensor
 
     u32x4 raw[R][C];
+    u32x4 rawb[R][C];
     u32x2 mk[R][C];
     int len[R];
     int ipos[R];       // row position inside its matrix (ALiBi)
@@ -415,6 +441,10 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
             raw[p][c] = buf_ld128<kLdNt>(rx, col < len[p] ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            if constexpr ((FLAGS & kBias) != 0) {
+                const uint32_t boff = (bias_row(row, a) * (uint32_t)sk + col) * 2u;
+                rawb[p][c] = buf_ld128<false>(rb, col < len[p] ? boff : kOutOfRange, 0);
+            }
             if constexpr (MASK == Mask::Bytes) {
                 const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
                 const uint32_t moff = (mb * (uint32_t)a.sq + i) * sk + col;
@@ -431,6 +461,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
             unpack8<T>(raw[p][c], v[c]);
+            if constexpr ((FLAGS & kBias) != 0) {
+                float bv[8];
+                unpack8<T>(rawb[p][c], bv);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) v[c][k] += bv[k];
+            }
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 bool keep = (col + k) < len[p];
@@ -607,8 +643,12 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
     // ALiBi (causal only): slopes given -> scores get slope*(j - i) before the scale
     const float slope2 = (MASK == Mask::Causal && a.slopes != nullptr)
                              ? a.slopes[(row / (uint32_t)a.sq) % a.np] * a.scale : 0.f;
+    const char* brow = nullptr;
+    if constexpr ((FLAGS & kBias) != 0) brow = static_cast<const char*>(a.bias) + (size_t)bias_row(row, a) * sk * 2;
     auto score = [&](int j) {
-        return fmaf(Elem<T>::load1(x + (size_t)j * 2), a.scale, slope2 * (float)(j - (int)i));
+        float xj = Elem<T>::load1(x + (size_t)j * 2);
+        if constexpr ((FLAGS & kBias) != 0) xj += Elem<T>::load1(brow + (size_t)j * 2);
+        return fmaf(xj, a.scale, slope2 * (float)(j - (int)i));
     };
 
     float mx = ninf;

@@ -52,6 +52,30 @@ def forward(input, mask, scale_factor):
     return softmax_results
 
 
+def forward_bias(input, mask, bias, scale_factor):
+    """Mask-tensor softmax of ``scale * (input + bias)`` with the bias read inside the kernel;
+    ``bias``: ``[1 or b, np, sq, sk]`` (megatron/model/transformer.py:526-528).  No counterpart
+    in the reference's extension: it adds the bias in a separate pass."""
+    from .scaled_upper_triang_masked_softmax_cuda import check_bias
+
+    input, mask = _check_forward(input, mask)
+    _lib.require_gpu(bias)
+    bias = check_bias(input, bias)
+    b, np_, sq, sk = input.shape
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_masked_softmax_bias_fwd(
+                softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), bias.data_ptr(),
+                float(scale_factor), b, np_, sq, sk, mask.size(0), bias.size(0),
+                _lib.dtype_code(input.dtype), _lib.current_stream(input),
+            )
+        )
+    return softmax_results
+
+
 def _check_backward(output_grads, softmax_results):
     if output_grads.dim() != 4 or softmax_results.dim() != 4:
         raise RuntimeError("expected 4D tensor")

@@ -66,6 +66,43 @@ def forward_alibi(input, slopes, scale_factor):
     return softmax_results
 
 
+def check_bias(input, bias):
+    """``bias`` broadcastable to ``input`` ``[b, np, sq, sk]`` over the batch dimension only;
+    returns it contiguous and in ``input``'s dtype."""
+    b, np_, sq, sk = input.shape
+    if bias.dim() != 4 or tuple(bias.shape[1:]) != (np_, sq, sk) or bias.size(0) not in (1, b):
+        raise RuntimeError(f"bias must have shape [1 or {b}, {np_}, {sq}, {sk}], got {tuple(bias.shape)}")
+    return bias.detach().to(dtype=input.dtype).contiguous()
+
+
+def forward_bias(input, bias, scale_factor):
+    """Causal softmax of ``scale * (input + bias)`` with the bias read inside the kernel.
+
+    ``input``: ``[b, np, sq, sk]`` fp16/bf16; ``bias``: ``[1 or b, np, sq, sk]``, e.g. the
+    relative-position bias ``[1, np, sq, sk]`` (megatron/model/transformer.py:526-528).  No
+    counterpart in the reference's extension: it adds the bias in a separate pass.
+    """
+    if input.dim() != 4:
+        raise RuntimeError("expected 4D tensor")
+    if input.dtype not in _HALF:
+        raise RuntimeError("Only fp16 and bf16 are supported")
+    _lib.require_gpu(input, bias)
+    input = input.contiguous()
+    bias = check_bias(input, bias)
+    b, np_, sq, sk = input.shape
+    softmax_results = torch.empty_like(input, requires_grad=False)
+    if input.numel() == 0:
+        return softmax_results
+    with torch.cuda.device(input.device):
+        _lib.check(
+            _lib.lib().neox_causal_softmax_bias_fwd(
+                softmax_results.data_ptr(), input.data_ptr(), bias.data_ptr(), float(scale_factor),
+                b, np_, sq, sk, bias.size(0), _lib.dtype_code(input.dtype), _lib.current_stream(input),
+            )
+        )
+    return softmax_results
+
+
 def backward(output_grads, softmax_results, scale_factor):
     """Returns d(input); like the reference, the result is written into
     ``output_grads`` itself when that tensor is contiguous."""

@@ -150,6 +150,52 @@ class ScaledUpperTriangMaskedSoftmaxAlibi(torch.autograd.Function):
         return grads.view(b, np, sq, sk), None, None
 
 
+def _bias_gradient(grads, bias_shape):
+    """Gradient of an additive bias from the gradient of the scores: the bias is broadcast
+    over the batch dimension when its first dimension is 1."""
+    if bias_shape[0] == 1 and grads.shape[0] != 1:
+        return grads.sum(dim=0, keepdim=True)
+    return grads
+
+
+class ScaledUpperTriangMaskedSoftmaxBias(torch.autograd.Function):
+    """Causal softmax of ``scale * (inputs + bias)`` in one kernel, the bias being a tensor
+    ``[1 or b, np, sq, sk]`` such as the relative-position bias that the reference adds to the
+    scores in a pass of its own (megatron/model/transformer.py:526-534).  Differentiable with
+    respect to ``inputs`` and ``bias``."""
+
+    @staticmethod
+    def forward(ctx, inputs, bias, scale):
+        scale_t = _scale_tensor(scale)
+        ctx.bias_shape = bias.shape
+        return _remember(ctx, _causal_ext.forward_bias(inputs, bias, scale_t[0].item()), scale_t)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        b, np, sq, sk = probs.shape
+        grads = _causal_ext.backward(output_grads.reshape(-1, sq, sk), probs.view(-1, sq, sk), scale)
+        grads = grads.view(b, np, sq, sk)
+        return grads, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[1] else None), None
+
+
+class ScaledMaskedSoftmaxBias(torch.autograd.Function):
+    """Mask-tensor softmax of ``scale * (inputs + bias)`` in one kernel; see
+    ``ScaledUpperTriangMaskedSoftmaxBias``."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, bias, scale):
+        scale_t = _scale_tensor(scale)
+        ctx.bias_shape = bias.shape
+        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale_t[0].item()), scale_t)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        grads = _masked_ext.backward(output_grads, probs, scale)
+        return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None
+
+
 class ScaledMaskedSoftmax(torch.autograd.Function):
     """scale -> mask tensor -> softmax, in one kernel.
 
@@ -248,7 +294,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         if self.fusion:
             load_fused_kernels()  # ImportError here, not at the first forward
 
-    def forward(self, input, mask, alibi_slopes=None, dropout_p=0.0):
+    def forward(self, input, mask, alibi_slopes=None, dropout_p=0.0, bias=None):
         """``alibi_slopes`` (optional, ``[np]``) is an addition to the reference signature:
         ``forward(scores, mask, alibi_slopes=alibi.slopes)`` equals
         ``forward(alibi(scores), mask)`` (megatron/model/transformer.py:529-534) with the bias
@@ -257,11 +303,20 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         ``dropout_p`` (optional, training only) is the second addition:
         ``forward(scores, mask, dropout_p=p)`` equals ``dropout(forward(scores, mask), p)``
         (megatron/model/transformer.py:533-539) and is to be called where the reference calls
-        the dropout, inside the RNG tracker's ``fork()``."""
+        the dropout, inside the RNG tracker's ``fork()``.
+
+        ``bias`` (optional, ``[1 or b, np, sq, sk]``) is the third:
+        ``forward(scores, mask, bias=rpe)`` equals ``forward(scores + rpe, mask)``
+        (megatron/model/transformer.py:526-534) with the bias read inside the softmax kernel and
+        the sum taken in fp32."""
         assert input.dim() == 4  # [b, np, sq, sk]
         if dropout_p:
-            return self.forward_with_dropout(input, mask, alibi_slopes, dropout_p)
+            return self.forward_with_dropout(input, mask, alibi_slopes, dropout_p, bias)
         fused = self.is_kernel_available(mask, *input.size())
+        if bias is not None:
+            if fused and alibi_slopes is None:
+                return self.forward_fused_softmax(input, mask, bias)
+            input = input + bias
         if alibi_slopes is not None:
             b, np, sq, sk = input.size()
             if fused and self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
@@ -270,18 +325,19 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
             input = input + alibi_bias(alibi_slopes, sq, sk, input.device, input.dtype)
         return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
 
-    def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p):
+    def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p, bias=None):
         """Softmax and dropout in one kernel when the fused softmax serves the call, there is
-        no ALiBi bias and no HIP graph is being captured (the generator state would be frozen
+        no additive bias and no HIP graph is being captured (the generator state would be frozen
         into the graph); otherwise the softmax above followed by torch's dropout."""
         b, np, sq, sk = input.size()
         fusable = (
             alibi_slopes is None
+            and bias is None
             and self.is_kernel_available(mask, b, np, sq, sk)
-            and not torch.cuda.is_current_stream_capturing()
+            and not (input.is_cuda and torch.cuda.is_current_stream_capturing())
         )
         if not fusable:
-            return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes), dropout_p, True)
+            return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes, 0.0, bias), dropout_p, True)
         scale = 1.0 if self.scale is None else self.scale
         if self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
             probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(-1, sq, sk), scale, dropout_p)
@@ -314,15 +370,19 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         per_block = FusedScaleMaskSoftmax.get_batch_per_block(sq, sk, b, np)
         return ((b * np) if upper_triang else sq) % per_block == 0
 
-    def forward_fused_softmax(self, input, mask):
+    def forward_fused_softmax(self, input, mask, bias=None):
         b, np, sq, sk = input.size()
         scale = 1.0 if self.scale is None else self.scale
-        if not self.upper_triang_mask_fusion:
+        if self.upper_triang_mask_fusion:
+            assert sq == sk, "causal mask is only for self attention"
+        if not (self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask)):
+            # general fusion, or a causal-fusion call whose mask is not the plain triangle (e.g. a
+            # sliding-window mask): what the torch path computes, from the mask itself
+            if bias is not None:
+                return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale)
             return ScaledMaskedSoftmax.apply(input, mask, scale)
-        assert sq == sk, "causal mask is only for self attention"
-        if not self.mask_is_plain_causal(mask):
-            # e.g. a sliding-window mask: what the torch path computes, from the mask itself
-            return ScaledMaskedSoftmax.apply(input, mask, scale)
+        if bias is not None:
+            return ScaledUpperTriangMaskedSoftmaxBias.apply(input, bias, scale)
         # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
         probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
         return probs.view(b, np, sq, sk)

@@ -107,6 +107,23 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
                             int32_t sk, int32_t dtype, void* stream);
 
 /*
+ * Softmax of scale * (x + bias) with the bias tensor read inside the kernel (no separate
+ * "scores += bias" pass); the sum is taken in fp32.  bias: [bias_b, np, sq, sk] contiguous,
+ * dtype of x, bias_b in {1, b} (1 = shared by all samples).  Causal / mask-tensor variants as
+ * neox_causal_softmax_fwd / neox_masked_softmax_fwd.  The gradient with respect to x is
+ * neox_*_softmax_bwd; the gradient with respect to the bias is that same tensor (summed over
+ * the samples that share it).
+ * Replaces "attention_scores += rpe" followed by the softmax extension call
+ *   megatron/model/transformer.py:526-534, megatron/mpu/layers.py:353-380 (the bias)
+ */
+int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
+                                 int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
+                                 void* stream);
+int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
+                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
+                                 int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream);
+
+/*
  * Softmax with the attention dropout that follows it folded in (training only).
  * Forward stores two tensors: y, the probabilities exactly as neox_*_softmax_fwd gives
  * them (the backward pass needs them), and y_drop = keep ? round(float(y) / (1-p)) : 0,

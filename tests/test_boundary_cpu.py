@@ -279,8 +279,9 @@ def test_public_names_and_signatures_match_the_reference_modules():
 
     assert params(FusedScaleMaskSoftmax.__init__) == [
         "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale"]
-    # the reference's positional parameters, plus two optional additions that default to "off"
-    assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask", "alibi_slopes", "dropout_p"]
+    # the reference's positional parameters, plus three optional additions that default to "off"
+    assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask", "alibi_slopes", "dropout_p", "bias"]
+    assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["bias"].default is None
     assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["alibi_slopes"].default is None
     assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["dropout_p"].default == 0.0
     assert params(FusedScaleMaskSoftmax.is_kernel_available) == ["self", "mask", "b", "np", "sq", "sk"]

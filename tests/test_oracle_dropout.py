@@ -122,7 +122,7 @@ def _call(name, *args):
     return status, handle.neox_fused_last_error().decode()
 
 
-def test_dropout_entry_points_validate_before_touching_the_gpu():
+def test_dropout_and_bias_entry_points_validate_before_touching_the_gpu():
     buf = (ctypes.c_uint16 * 64)()
     other = (ctypes.c_uint16 * 64)()
     third = (ctypes.c_uint16 * 64)()
@@ -142,6 +142,14 @@ def test_dropout_entry_points_validate_before_touching_the_gpu():
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, 0, 8, 0, None)
     assert status == -3
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, 4, 8, 2, None)
+    assert status == -2
+    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, c, 1.0, 2, 1, 8, 8, 3, 0, None)
+    assert status == -3 and "bias batch" in msg
+    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, None, 1.0, 2, 1, 8, 8, 1, 0, None)
+    assert status == -1
+    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 1, 4, 0, None)
+    assert status == -3 and "bias batch" in msg
+    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 1, 1, 7, None)
     assert status == -2
     status, msg = _call("neox_dropout_keep_mask", None, 0.1, 0, 0, 8, None)
     assert status == -1

@@ -762,3 +762,115 @@ def test_config5_long_context(device):
     del y
     torch.cuda.empty_cache()
     check_rotary(device, 8192, 1, 32, 32, 128, 128, torch.bfloat16, seed=1239)
+
+
+# ---------------------------------------------------------------------------------
+# additive bias tensor (relative-position bias) read inside the softmax kernels
+# ---------------------------------------------------------------------------------
+from gpt_neox_amd.fused_softmax import ScaledMaskedSoftmaxBias, ScaledUpperTriangMaskedSoftmaxBias  # noqa: E402
+
+BIAS_SHAPES = [(2, 3, 8, 8), (3, 2, 40, 40), (2, 2, 136, 136), (2, 3, 512, 512), (2, 2, 1024, 1024),
+               (2, 1, 2048, 2048), (1, 2, 4096, 4096), (2, 2, 37, 37), (1, 2, 1001, 1001)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("shape", BIAS_SHAPES)
+def test_causal_softmax_with_bias_tensor(device, shape, shared, dtype):
+    b, np_, s, _ = shape
+    x = scores(shape, dtype, device, 70)
+    bias = scores((1 if shared else b, np_, s, s), dtype, device, 71) * 0.25
+    y = causal_ext.forward_bias(x, bias, 0.125)
+    mask = R.get_attn_mask(s, device)
+    ref = R.softmax_fp32(x.float() + bias.float(), mask, 0.125)
+    assert max_err(y, ref) <= TOL[dtype]
+    assert (y[mask.expand(shape)] == 0).all()
+    # a zero bias is the plain kernel, bit for bit
+    assert torch.equal(causal_ext.forward_bias(x, torch.zeros_like(bias), 0.125),
+                       causal_ext.forward(x.view(-1, s, s), 0.125).view(shape))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("shape", [(2, 3, 5, 8), (2, 2, 9, 40), (1, 3, 16, 136), (2, 2, 8, 512), (2, 2, 16, 1024),
+                                   (1, 2, 8, 2048), (2, 1, 4, 4096), (2, 2, 5, 37), (1, 2, 3, 1001)])
+def test_masked_softmax_with_bias_tensor(device, shape, shared, dtype):
+    b, np_, sq, sk = shape
+    x = scores(shape, dtype, device, 72)
+    bias = scores((1 if shared else b, np_, sq, sk), dtype, device, 73) * 0.25
+    lengths = torch.randint(1, sk + 1, (b,), generator=gen(device, 74), device=device)
+    mask = R.padding_mask(lengths, sq, sk, device)
+    y = masked_ext.forward_bias(x, mask, bias, 0.5)
+    ref = R.softmax_fp32(x.float() + bias.float(), mask, 0.5)
+    assert max_err(y, ref) <= TOL[dtype]
+    assert (y[mask.expand(shape)] == 0).all()
+    assert torch.equal(masked_ext.forward_bias(x, mask, torch.zeros_like(bias), 0.5),
+                       masked_ext.forward(x, mask, 0.5))
+
+
+def test_bias_argument_checks(device):
+    x = scores((2, 3, 16, 16), torch.float16, device, 75)
+    with pytest.raises(RuntimeError, match="bias must have shape"):
+        causal_ext.forward_bias(x, x[:, :2], 1.0)
+    with pytest.raises(RuntimeError, match="bias must have shape"):
+        causal_ext.forward_bias(x, x[0], 1.0)
+    # other dtypes and layouts are converted: the result is that of the converted bias
+    bias = scores((1, 3, 16, 16), torch.float32, device, 76)
+    permuted = bias.permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)  # the layout movedim(2, 0) leaves
+    assert not permuted.is_contiguous()
+    assert torch.equal(causal_ext.forward_bias(x, permuted, 1.0), causal_ext.forward_bias(x, bias.half(), 1.0))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shared", [True, False])
+def test_bias_functions_gradients(device, shared, dtype):
+    b, np_, s = 3, 2, 64
+    shape = (b, np_, s, s)
+    x = scores(shape, dtype, device, 77).requires_grad_(True)
+    bias = (scores((1 if shared else b, np_, s, s), dtype, device, 78) * 0.25).requires_grad_(True)
+    g = normal(shape, dtype, device, 79)
+    causal = R.get_attn_mask(s, device)
+    pad = R.padding_mask(torch.tensor([40, 64, 9]), s, s, device)
+    for fn, mask in ((lambda: ScaledUpperTriangMaskedSoftmaxBias.apply(x, bias, 0.5), causal),
+                     (lambda: ScaledMaskedSoftmaxBias.apply(x, pad, bias, 0.5), pad)):
+        x.grad = bias.grad = None
+        y = fn()
+        y.backward(g.clone())
+        xr = x.detach().float().requires_grad_(True)
+        br = bias.detach().float().requires_grad_(True)
+        R.softmax_fp32(xr + br, mask, 0.5).backward(g.float())
+        scale = max(1.0, xr.grad.abs().max().item())
+        assert max_err(x.grad, xr.grad) <= 4 * TOL[dtype] * scale
+        assert bias.grad.shape == bias.shape
+        assert max_err(bias.grad, br.grad) <= 4 * TOL[dtype] * max(1.0, br.grad.abs().max().item()) * (b if shared else 1)
+    # no bias gradient is formed when the bias does not ask for one
+    x.grad = None
+    fixed = bias.detach()
+    ScaledUpperTriangMaskedSoftmaxBias.apply(x, fixed, 0.5).backward(g.clone())
+    assert fixed.grad is None and x.grad is not None
+
+
+def test_module_bias_argument(device):
+    b, np_, s = 2, 4, 128
+    x = scores((b, np_, s, s), torch.bfloat16, device, 80)
+    rpe = (scores((s, s, np_), torch.bfloat16, device, 81) * 0.25).movedim(2, 0).unsqueeze(0)  # [1, np, s, s] view
+    causal = R.get_attn_mask(s, device)
+    m = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func, True, 0.5)
+    y = m(x, causal, bias=rpe)
+    ref = R.softmax_fp32(x.float() + rpe.float(), causal, 0.5)
+    assert max_err(y, ref) <= TOL[torch.bfloat16]
+    # the reference's two passes round x + rpe to bf16 first: close, not identical
+    two_pass = m(x + rpe, causal)
+    assert max_err(y, two_pass) <= 0.1
+    assert max_err(two_pass, ref) >= max_err(y, ref)
+    # sliding-window mask, general fusion and the unfused module give the same function
+    window = R.get_attn_mask(s, device, sliding_window_width=16)
+    assert max_err(m(x, window, bias=rpe), R.softmax_fp32(x.float() + rpe.float(), window, 0.5)) <= TOL[torch.bfloat16]
+    mg = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.5)
+    pad = R.padding_mask(torch.tensor([100, 128]), s, s, device)
+    assert max_err(mg(x, pad, bias=rpe), R.softmax_fp32(x.float() + rpe.float(), pad, 0.5)) <= TOL[torch.bfloat16]
+    mt = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
+    assert torch.equal(mt(x, causal, bias=rpe), mt(x + rpe, causal))
+    # bias and dropout together: the bias kernel followed by torch's dropout
+    out = m(x, causal, bias=rpe, dropout_p=0.5)
+    assert torch.equal(out, R.dropout_with_mask(y, out != 0, 0.5))
