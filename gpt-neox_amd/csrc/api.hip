@@ -4,6 +4,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <initializer_list>
+
 #include "internal.hpp"
 
 namespace neox {
@@ -57,6 +59,121 @@ static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset,
     return NEOX_OK;
 }
 
+// One softmax call under validation.  The checks run in a fixed order -- null pointers,
+// dtype, shape, alignment, then the optional parts -- and the first failure sticks in
+// `status`; nothing here touches the GPU.  The 16-bit tensors given to the constructor
+// also decide whether 128-bit accesses are legal (`vec_ok`).
+struct SoftmaxCall {
+    typedef hipError_t (*Launcher)(const SoftmaxArgs&, Mask, int, bool, hipStream_t);
+
+    const char* what;
+    int dtype;
+    int status = NEOX_OK;
+    bool vec_ok = true;
+    SoftmaxArgs a{};
+
+    SoftmaxCall(const char* name, int dtype_code, std::initializer_list<const void*> tensors,
+                const void* extra = reinterpret_cast<const void*>(1))
+        : what(name), dtype(dtype_code) {
+        bool null = (extra == nullptr), odd = false;
+        for (const void* t : tensors) {
+            null = null || t == nullptr;
+            odd = odd || !aligned(t, 2);
+            vec_ok = vec_ok && aligned(t, 16);
+        }
+        if (null) {
+            status = fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
+        } else if ((status = check_dtype(dtype, what)) == NEOX_OK && odd) {
+            misaligned_ = true;  // reported after the shape checks
+        }
+    }
+
+    // [batches, sq, sk]
+    void causal_rows(int64_t batches, int sq, int sk) {
+        if (status) return;
+        if (batches < 1) {
+            status = fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
+            return;
+        }
+        rows(sq < 1 ? 0 : batches * sq, sq, sk);
+    }
+    // [b, np, sq, sk]
+    void head_rows(int b, int np, int sq, int sk) {
+        if (status) return;
+        if (b < 1 || np < 1) {
+            status = fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
+            return;
+        }
+        rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk);
+    }
+    // [rows, sk]
+    void plain_rows(int64_t n, int sk) { if (!status) rows(n, 1, sk); }
+
+    // mask bytes [mask_b, 1, sq, sk]
+    void mask(const uint8_t* m, int b, int np, int mask_b) {
+        if (status) return;
+        if (mask_b != 1 && mask_b != b) {
+            status = fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
+            return;
+        }
+        a.mask = m;
+        a.rows_per_mask_batch = (uint32_t)((int64_t)np * a.sq);
+        a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+        a.mask_bytes = fits32((uint64_t)mask_b * (uint64_t)a.sq * (uint64_t)a.sk);
+        vec_ok = vec_ok && aligned(m, 8);
+    }
+    // bias [bias_b, np, sq, sk] in the dtype of the scores (one of the constructor's tensors)
+    void bias(const void* t, int b, int np, int bias_b) {
+        if (status) return;
+        if (bias_b != 1 && bias_b != b) {
+            status = fail(NEOX_ERR_BAD_SHAPE, "%s: bias batch dim %d must be 1 or b=%d", what, bias_b, b);
+            return;
+        }
+        a.bias = t;
+        a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * a.sq) : 0u;
+        a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
+    }
+    void dropout(float p, uint64_t seed, uint64_t offset) {
+        if (!status) status = make_dropout(a.drop, p, seed, offset, what);
+    }
+    void second_output(void* y_drop, const void* y) {
+        if (status) return;
+        if (y_drop == y) status = fail(NEOX_ERR_BAD_STRIDE, "%s: y_drop must not alias y", what);
+        a.out2 = y_drop;
+    }
+
+    void forward(void* y, const void* x, float scale) {
+        a.out = y;
+        a.in0 = x;
+        a.scale = scale * kLog2e;
+    }
+    void backward(void* dx, const void* dy, const void* y, float scale) {
+        a.out = dx;
+        a.in0 = dy;
+        a.in1 = y;
+        a.scale = scale;
+    }
+    int launch(Launcher fn, Mask m, void* stream) const {
+        return check_launch(fn(a, m, dtype, vec_ok && a.sk % kVec == 0, (hipStream_t)stream), what);
+    }
+
+  private:
+    bool misaligned_ = false;
+
+    void rows(int64_t n, int sq, int sk) {
+        if ((status = check_rows(n, sq, sk, what)) != NEOX_OK) return;
+        if (misaligned_) {
+            status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+            return;
+        }
+        a.rows = (uint32_t)n;
+        a.sq = sq;
+        a.sk = sk;
+    }
+    // size of a tensor the packed kernels address through one buffer, 0 if it needs more than 32 bits
+    static uint32_t fits32(uint64_t bytes) { return bytes < 0xFFFFFFFFull ? (uint32_t)bytes : 0u; }
+};
+
 // The keep pattern of the dropout kernels, one byte per element (1 = kept).
 __global__ __launch_bounds__(256) void keep_mask_kernel(uint8_t* keep, DropoutArgs d, uint64_t n) {
     const uint64_t group = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -104,288 +221,123 @@ const char* neox_fused_last_error(void) { return g_last_error; }
 
 int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int32_t sq,
                             int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_causal_softmax_fwd";
-    if (!y || !x) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
-    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    a.out = y;
-    a.in0 = x;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)(batches * sq);
-    a.sq = sq;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_fwd", dtype, {y, x});
+    c.causal_rows(batches, sq, sk);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_fwd, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, float scale, int32_t b,
                                   int32_t np, int32_t sq, int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_causal_softmax_alibi_fwd";
-    if (!y || !x || !slopes) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
-    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(slopes, 4))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    a.out = y;
-    a.in0 = x;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)((int64_t)b * np * sq);
-    a.sq = sq;
-    a.sk = sk;
-    a.slopes = slopes;
-    a.np = (uint32_t)np;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_alibi_fwd", dtype, {y, x}, slopes);
+    c.head_rows(b, np, sq, sk);
+    if (!c.status && !aligned(slopes, 4)) c.status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", c.what);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    c.a.slopes = slopes;
+    c.a.np = (uint32_t)np;
+    return c.launch(launch_softmax_fwd, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
                             int32_t sq, int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_causal_softmax_bwd";
-    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
-    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
-    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    a.out = dx;
-    a.in0 = dy;
-    a.in1 = y;
-    a.scale = scale;
-    a.rows = (uint32_t)(batches * sq);
-    a.sq = sq;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_bwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_bwd", dtype, {dx, dy, y});
+    c.causal_rows(batches, sq, sk);
+    if (c.status) return c.status;
+    c.backward(dx, dy, y, scale);
+    return c.launch(launch_softmax_bwd, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
                             int32_t np, int32_t sq, int32_t sk, int32_t mask_b, int32_t dtype,
                             void* stream) {
-    static const char* what = "neox_masked_softmax_fwd";
-    if (!y || !x || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
-    if (mask_b != 1 && mask_b != b)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
-    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    a.out = y;
-    a.in0 = x;
-    a.mask = mask;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)((int64_t)b * np * sq);
-    a.sq = sq;
-    a.sk = sk;
-    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
-    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
-    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
-    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(mask, 8);
-    return check_launch(launch_softmax_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_masked_softmax_fwd", dtype, {y, x}, mask);
+    c.head_rows(b, np, sq, sk);
+    c.mask(mask, b, np, mask_b);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_fwd, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows,
                             int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_masked_softmax_bwd";
-    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (int e = check_rows(rows, 1, sk, what)) return e;
-    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    a.out = dx;
-    a.in0 = dy;
-    a.in1 = y;
-    a.scale = scale;
-    a.rows = (uint32_t)rows;
-    a.sq = 1;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
-}
-
-// bias [bias_b, np, sq, sk]: shared by all samples (bias_b == 1) or one per sample
-static int set_bias(SoftmaxArgs& a, const void* bias, int b, int np, int sq, int sk, int bias_b,
-                    const char* what) {
-    if (bias_b != 1 && bias_b != b)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: bias batch dim %d must be 1 or b=%d", what, bias_b, b);
-    a.bias = bias;
-    a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * sq) : 0u;
-    const uint64_t bytes = (uint64_t)bias_b * (uint64_t)np * (uint64_t)sq * (uint64_t)sk * 2u;
-    a.bias_bytes = bytes < 0xFFFFFFFFull ? (uint32_t)bytes : 0u;
-    return NEOX_OK;
+    SoftmaxCall c("neox_masked_softmax_bwd", dtype, {dx, dy, y});
+    c.plain_rows(rows, sk);
+    if (c.status) return c.status;
+    c.backward(dx, dy, y, scale);
+    return c.launch(launch_softmax_bwd, Mask::None, stream);
 }
 
 int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
                                  int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
                                  void* stream) {
-    static const char* what = "neox_causal_softmax_bias_fwd";
-    if (!y || !x || !bias) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
-    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(bias, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = set_bias(a, bias, b, np, sq, sk, bias_b, what)) return e;
-    a.out = y;
-    a.in0 = x;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)((int64_t)b * np * sq);
-    a.sq = sq;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(bias, 16);
-    return check_launch(launch_softmax_bias_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_bias_fwd", dtype, {y, x, bias});
+    c.head_rows(b, np, sq, sk);
+    c.bias(bias, b, np, bias_b);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_bias_fwd, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
                                  float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
                                  int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream) {
-    static const char* what = "neox_masked_softmax_bias_fwd";
-    if (!y || !x || !mask || !bias) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
-    if (mask_b != 1 && mask_b != b)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
-    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(bias, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = set_bias(a, bias, b, np, sq, sk, bias_b, what)) return e;
-    a.out = y;
-    a.in0 = x;
-    a.mask = mask;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)((int64_t)b * np * sq);
-    a.sq = sq;
-    a.sk = sk;
-    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
-    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
-    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
-    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(bias, 16) &&
-                        aligned(mask, 8);
-    return check_launch(launch_softmax_bias_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_masked_softmax_bias_fwd", dtype, {y, x, bias}, mask);
+    c.head_rows(b, np, sq, sk);
+    c.mask(mask, b, np, mask_b);
+    c.bias(bias, b, np, bias_b);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_bias_fwd, Mask::Bytes, stream);
 }
 
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
                                     uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_causal_softmax_dropout_fwd";
-    if (!y_drop || !y || !x) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (y_drop == y) return fail(NEOX_ERR_BAD_STRIDE, "%s: y_drop must not alias y", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
-    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(y_drop, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
-    a.out = y;
-    a.out2 = y_drop;
-    a.in0 = x;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)(batches * sq);
-    a.sq = sq;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(y_drop, 16);
-    return check_launch(launch_softmax_dropout_fwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_dropout_fwd", dtype, {y_drop, y, x});
+    c.second_output(y_drop, y);
+    c.causal_rows(batches, sq, sk);
+    c.dropout(p, seed, offset);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_dropout_fwd, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
                                     uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream) {
-    static const char* what = "neox_causal_softmax_dropout_bwd";
-    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (batches < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: batches=%lld must be >= 1", what, (long long)batches);
-    if (int e = check_rows(sq < 1 ? 0 : batches * sq, sq, sk, what)) return e;
-    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
-    a.out = dx;
-    a.in0 = dy;
-    a.in1 = y;
-    a.scale = scale;
-    a.rows = (uint32_t)(batches * sq);
-    a.sq = sq;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_dropout_bwd(a, Mask::Causal, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_causal_softmax_dropout_bwd", dtype, {dx, dy, y});
+    c.causal_rows(batches, sq, sk);
+    c.dropout(p, seed, offset);
+    if (c.status) return c.status;
+    c.backward(dx, dy, y, scale);
+    return c.launch(launch_softmax_dropout_bwd, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
                                     float scale, float p, uint64_t seed, uint64_t offset, int32_t b,
                                     int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream) {
-    static const char* what = "neox_masked_softmax_dropout_fwd";
-    if (!y_drop || !y || !x || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (y_drop == y) return fail(NEOX_ERR_BAD_STRIDE, "%s: y_drop must not alias y", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (b < 1 || np < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d np=%d must be >= 1", what, b, np);
-    if (mask_b != 1 && mask_b != b)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
-    if (int e = check_rows(sq < 1 ? 0 : (int64_t)b * np * sq, sq, sk, what)) return e;
-    if (!aligned(x, 2) || !aligned(y, 2) || !aligned(y_drop, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
-    a.out = y;
-    a.out2 = y_drop;
-    a.in0 = x;
-    a.mask = mask;
-    a.scale = scale * kLog2e;
-    a.rows = (uint32_t)((int64_t)b * np * sq);
-    a.sq = sq;
-    a.sk = sk;
-    a.rows_per_mask_batch = (uint32_t)((int64_t)np * sq);
-    a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
-    const uint64_t mask_bytes = (uint64_t)mask_b * (uint64_t)sq * (uint64_t)sk;
-    a.mask_bytes = mask_bytes < 0xFFFFFFFFull ? (uint32_t)mask_bytes : 0u;
-    const bool vec_ok = (sk % kVec == 0) && aligned(x, 16) && aligned(y, 16) && aligned(y_drop, 16) &&
-                        aligned(mask, 8);
-    return check_launch(launch_softmax_dropout_fwd(a, Mask::Bytes, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_masked_softmax_dropout_fwd", dtype, {y_drop, y, x}, mask);
+    c.second_output(y_drop, y);
+    c.head_rows(b, np, sq, sk);
+    c.mask(mask, b, np, mask_b);
+    c.dropout(p, seed, offset);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(launch_softmax_dropout_fwd, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
                                     uint64_t seed, uint64_t offset, int64_t rows, int32_t sk,
                                     int32_t dtype, void* stream) {
-    static const char* what = "neox_masked_softmax_dropout_bwd";
-    if (!dx || !dy || !y) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
-    if (int e = check_dtype(dtype, what)) return e;
-    if (int e = check_rows(rows, 1, sk, what)) return e;
-    if (!aligned(dx, 2) || !aligned(dy, 2) || !aligned(y, 2))
-        return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-
-    SoftmaxArgs a{};
-    if (int e = make_dropout(a.drop, p, seed, offset, what)) return e;
-    a.out = dx;
-    a.in0 = dy;
-    a.in1 = y;
-    a.scale = scale;
-    a.rows = (uint32_t)rows;
-    a.sq = 1;
-    a.sk = sk;
-    const bool vec_ok = (sk % kVec == 0) && aligned(dx, 16) && aligned(dy, 16) && aligned(y, 16);
-    return check_launch(launch_softmax_dropout_bwd(a, Mask::None, dtype, vec_ok, (hipStream_t)stream), what);
+    SoftmaxCall c("neox_masked_softmax_dropout_bwd", dtype, {dx, dy, y});
+    c.plain_rows(rows, sk);
+    c.dropout(p, seed, offset);
+    if (c.status) return c.status;
+    c.backward(dx, dy, y, scale);
+    return c.launch(launch_softmax_dropout_bwd, Mask::None, stream);
 }
 
 int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset, int64_t n,
