@@ -81,3 +81,34 @@ def rotary_vec_backward(g, pos, base=10000.0):
         out[j] = g[j] * c + g[j + h] * s
         out[j + h] = g[j + h] * c - g[j] * s
     return out
+
+
+# --- attention dropout: Philox4x32-10 on Python integers -----------------------------------
+
+
+def philox4x32_10(counter, key):
+    """One Philox4x32-10 block (Salmon et al., SC'11) on Python integers: ``counter`` four and
+    ``key`` two 32-bit words; ten rounds of two 32x32->64 bit multiplications, the key bumped
+    by the Weyl constants between rounds."""
+    c = [int(v) for v in counter]
+    k = [int(v) for v in key]
+    for _ in range(10):
+        p0 = 0xD2511F53 * c[0]
+        p1 = 0xCD9E8D57 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & 0xFFFFFFFF, (p0 >> 32) ^ c[3] ^ k[1], p0 & 0xFFFFFFFF]
+        k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
+    return c
+
+
+def keep_element(e, p, seed, offset):
+    """Whether the element with row-major index ``e`` survives a dropout of probability ``p``
+    drawn from Philox state ``(seed, offset)``: its group of 8 shares the block with counter
+    ``(offset, e // 8)``; the element owns 16 bits of it and is kept iff they are not below
+    ``round(p * 65536)``."""
+    group = e // 8
+    words = philox4x32_10(
+        [offset & 0xFFFFFFFF, offset >> 32, group & 0xFFFFFFFF, group >> 32],
+        [seed & 0xFFFFFFFF, seed >> 32],
+    )
+    field = (words[(e % 8) // 2] >> (16 * (e % 2))) & 0xFFFF
+    return field >= int(round(p * 65536))

@@ -67,6 +67,20 @@ def rotary_case(rng, name, s, b, heads, dim, offset, base=10000.0):
              offset=np.int64(offset), base=np.float64(base))
 
 
+def dropout_case(rng, name, batches, s, scale, p, seed, offset):
+    """Causal softmax followed by dropout: the keep pattern from the integer Philox of
+    oracle/brute.py, everything else in float64 (no rounding of the probabilities)."""
+    x = grid_values(rng, (batches, s, s))
+    g = grid_values(rng, (batches, s, s), span=16)
+    hidden = brute.causal_hidden(s, s)
+    keep = np.array([brute.keep_element(e, p, seed, offset) for e in range(x.size)]).reshape(x.shape)
+    y = np.stack([brute.softmax_rows(x[b], scale, hidden) for b in range(batches)])
+    y_drop = y * keep / (1.0 - p)
+    dx = np.stack([brute.softmax_rows_backward(g[b] * keep[b] / (1.0 - p), y[b], scale) for b in range(batches)])
+    np.savez(os.path.join(HERE, name), x=x, g=g, y=y, keep=keep.astype(np.uint8), y_drop=y_drop, dx=dx,
+             scale=np.float64(scale), p=np.float64(p), seed=np.uint64(seed), offset=np.uint64(offset))
+
+
 def main():
     rng = np.random.default_rng(20240521)
     causal_case(rng, "causal_8", batches=2, s=8, scale=0.125)
@@ -76,6 +90,9 @@ def main():
     rotary_case(rng, "rotary_d8", s=5, b=2, heads=2, dim=8, offset=3)
     rotary_case(rng, "rotary_d32", s=6, b=1, heads=3, dim=32, offset=0)
     rotary_case(rng, "rotary_d24", s=4, b=2, heads=1, dim=24, offset=1)
+    # drawn after all earlier cases, so their files do not change
+    dropout_case(rng, "dropout_causal_16", batches=2, s=16, scale=0.25, p=0.25, seed=2**40 + 77, offset=2**33 + 8)
+    dropout_case(rng, "dropout_causal_37", batches=1, s=37, scale=0.125, p=0.1, seed=1234, offset=0)
 
 
 if __name__ == "__main__":

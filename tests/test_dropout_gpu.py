@@ -85,6 +85,27 @@ def test_dropout_scale_is_the_device_library_s(device):
 
 
 # ---------------------------------------------------------------------------------
+# golden vectors
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["dropout_causal_16", "dropout_causal_37"])
+def test_golden_dropout(device, golden, name, dtype):
+    f = golden[name]
+    p, seed, offset, scale = float(f["p"]), int(f["seed"]), int(f["offset"]), float(f["scale"])
+    x = torch.tensor(f["x"], device=device).to(dtype)
+    assert torch.equal(x.float().cpu(), torch.tensor(f["x"]))  # inputs are exact in both types
+    y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset)
+    keep = torch.tensor(f["keep"], device=device).bool()
+    assert torch.equal(rng.keep_mask(x.numel(), p, seed, offset, device).view(x.shape), keep)
+    assert torch.equal(dropped != 0, keep & (y != 0))
+    assert max_err(y, torch.tensor(f["y"], device=device)) <= TOL[dtype]
+    assert max_err(dropped, torch.tensor(f["y_drop"], device=device)) <= TOL[dtype] / (1 - p)
+    g = torch.tensor(f["g"], device=device).to(dtype)
+    dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+    assert max_err(dx, torch.tensor(f["dx"], device=device)) <= 4 * TOL[dtype] * max(1.0, np.abs(f["dx"]).max())
+
+
+# ---------------------------------------------------------------------------------
 # forward
 # ---------------------------------------------------------------------------------
 def check_forward(y, dropped, y_plain, p, seed, offset, device):

@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import philox, torch_ref
+from oracle import brute, philox, torch_ref
 
 gpt_neox_amd = pytest.importorskip("gpt_neox_amd")
 from gpt_neox_amd import _lib  # noqa: E402
@@ -34,26 +34,9 @@ def test_philox_known_answers(counter, key, expected):
     assert tuple(int(v) for v in out) == expected
 
 
-def _philox_scalar(counter, key):
-    """Philox4x32-10 on Python integers, written from the paper's round description."""
-    c = list(counter)
-    k = list(key)
-    for _ in range(10):
-        p0 = 0xD2511F53 * c[0]
-        p1 = 0xCD9E8D57 * c[2]
-        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & 0xFFFFFFFF, (p0 >> 32) ^ c[3] ^ k[1], p0 & 0xFFFFFFFF]
-        k = [(k[0] + 0x9E3779B9) & 0xFFFFFFFF, (k[1] + 0xBB67AE85) & 0xFFFFFFFF]
-    return c
-
-
-def _keep_scalar(e, p, seed, offset):
-    group = e // 8
-    words = _philox_scalar(
-        [offset & 0xFFFFFFFF, offset >> 32, group & 0xFFFFFFFF, group >> 32],
-        [seed & 0xFFFFFFFF, seed >> 32],
-    )
-    field = (words[(e % 8) // 2] >> (16 * (e % 2))) & 0xFFFF
-    return field >= int(round(p * 65536))
+@pytest.mark.parametrize("counter,key,expected", KAT)
+def test_integer_philox_known_answers(counter, key, expected):
+    assert tuple(brute.philox4x32_10(counter, key)) == expected
 
 
 @pytest.mark.parametrize("seed,offset", [(0, 0), (1234, 8), (2**63 + 12345, 2**40 + 4)])
@@ -61,7 +44,7 @@ def test_keep_mask_matches_the_per_element_restatement(seed, offset):
     n = 203
     mask = philox.keep_mask(n, 0.3, seed, offset)
     assert mask.dtype == np.bool_ and mask.shape == (n,)
-    assert [bool(v) for v in mask] == [_keep_scalar(e, 0.3, seed, offset) for e in range(n)]
+    assert [bool(v) for v in mask] == [brute.keep_element(e, 0.3, seed, offset) for e in range(n)]
 
 
 def test_keep_mask_statistics_and_structure():
@@ -114,6 +97,22 @@ def test_softmax_dropout_backward_matches_autograd_of_the_unfused_expression():
     (dx,) = torch.autograd.grad(dropped, x, grad_out)
     got = torch_ref.softmax_dropout_backward_fp32(grad_out.float(), probs.detach().float(), keep, p, scale)
     assert torch.allclose(got.double(), dx, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("name", ["dropout_causal_16", "dropout_causal_37"])
+def test_golden_dropout_vectors(golden, name):
+    f = golden[name]
+    p, seed, offset, scale = float(f["p"]), int(f["seed"]), int(f["offset"]), float(f["scale"])
+    keep = philox.keep_mask(f["x"].size, p, seed, offset).reshape(f["x"].shape)
+    assert np.array_equal(keep, f["keep"].astype(bool))
+    x = torch.tensor(f["x"])
+    s = x.shape[-1]
+    probs = torch_ref.softmax_fp32(x.unsqueeze(1), torch_ref.get_attn_mask(s), scale).squeeze(1)
+    assert np.abs(probs.numpy() - f["y"]).max() < 1e-6
+    dropped = torch_ref.dropout_with_mask(probs, torch.from_numpy(keep), p)
+    assert np.abs(dropped.numpy() - f["y_drop"]).max() < 1e-6
+    dx = torch_ref.softmax_dropout_backward_fp32(torch.tensor(f["g"]), probs, torch.from_numpy(keep), p, scale)
+    assert np.abs(dx.numpy() - f["dx"]).max() < 1e-5 * max(1.0, np.abs(f["dx"]).max())
 
 
 def _call(name, *args):
