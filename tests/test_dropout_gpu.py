@@ -99,7 +99,9 @@ def test_golden_dropout(device, golden, name, dtype):
     assert torch.equal(rng.keep_mask(x.numel(), p, seed, offset, device).view(x.shape), keep)
     assert torch.equal(dropped != 0, keep & (y != 0))
     assert max_err(y, torch.tensor(f["y"], device=device)) <= TOL[dtype]
-    assert max_err(dropped, torch.tensor(f["y_drop"], device=device)) <= TOL[dtype] / (1 - p)
+    # values up to 1/(1-p) > 1: the error of y scaled up, plus half an ulp of the second rounding
+    half_ulp = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    assert max_err(dropped, torch.tensor(f["y_drop"], device=device)) <= (TOL[dtype] + half_ulp) / (1 - p)
     g = torch.tensor(f["g"], device=device).to(dtype)
     dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
     assert max_err(dx, torch.tensor(f["dx"], device=device)) <= 4 * TOL[dtype] * max(1.0, np.abs(f["dx"]).max())
