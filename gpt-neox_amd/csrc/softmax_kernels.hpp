@@ -45,7 +45,7 @@ struct SoftmaxArgs {
 
 enum class Mask { Causal, Bytes, None };
 
-// Compile-time tuning switches of the row kernels.
+// Compile-time switches of the kernels (FLAGS): two memory hints and three optional features.
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
 constexpr int kNtStore = 2;  // non-temporal hint on the streaming stores
 constexpr int kAlibi = 4;    // causal forward adds the ALiBi bias -slope[head]*(i - j) to the scores

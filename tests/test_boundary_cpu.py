@@ -213,7 +213,7 @@ def test_is_kernel_available_table():
     mask = torch.zeros(1, 1, 4, 4, dtype=torch.bool)
     causal, general, none = (make(t) for t in (SoftmaxFusionTypes.upper_triang,
                                                 SoftmaxFusionTypes.general, SoftmaxFusionTypes.none))
-    # every BASELINE shape takes the fused branch, including the 8192 one
+    # every benchmark shape takes the fused branch, including the 8192 one
     for b, np_, sq, sk in [(4, 12, 2048, 2048), (1, 64, 2048, 2048), (1, 32, 8192, 8192), (3, 5, 7, 7)]:
         assert causal.is_kernel_available(mask, b, np_, sq, sk)
     assert general.is_kernel_available(mask, 8, 16, 1024, 1024)

@@ -220,7 +220,7 @@ def test_backward_against_fp64_autograd_of_the_unfused_expression(device):
 
 
 # ---------------------------------------------------------------------------------
-# BASELINE shapes at full size
+# the benchmark shapes at full size
 # ---------------------------------------------------------------------------------
 def test_full_size_padded_config(device):
     shape = (8, 16, 1024, 1024)

@@ -1,6 +1,6 @@
 """Parity of the gfx950 kernels (called through the C-ABI) with the oracle.
 
-Bars (BASELINE.json north_star): softmax |err| <= 2e-3 (bf16) / 1e-3 (fp16)
+Bars: softmax |err| <= 2e-3 (bf16) / 1e-3 (fp16)
 against the fp32 computation of the reference's unfused path, masked positions
 exactly 0; rotary is bit-equal to the fp32 expression rounded once to the storage
 type.  The backward pass is compared with the fp32 closed form evaluated on the
@@ -732,7 +732,7 @@ def test_rotary_round_trip_property(device):
 
 
 # ---------------------------------------------------------------------------------
-# BASELINE.json shapes at full size
+# the benchmark shapes at full size
 # ---------------------------------------------------------------------------------
 def test_config1_causal_fwd_125m(device):
     x, y, g, dx = check_causal(device, 48, 2048, torch.bfloat16, 0.125, seed=1234)
