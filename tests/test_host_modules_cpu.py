@@ -127,3 +127,35 @@ def test_alibi_slopes_argument_on_the_unfused_branch():
     mask = R.get_attn_mask(8)
     sm = FusedScaleMaskSoftmax(False, False, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
     assert torch.equal(sm(x.clone(), mask, alibi_slopes=mod.slopes), sm(mod(x.clone()), mask))
+
+
+def test_get_fusion_type_prefers_the_causal_kernel():
+    from types import SimpleNamespace
+
+    from gpt_neox_amd.utils import get_fusion_type
+
+    def args(causal, general):
+        return SimpleNamespace(scaled_upper_triang_masked_softmax_fusion=causal,
+                               scaled_masked_softmax_fusion=general)
+
+    assert get_fusion_type(args(False, False)) is SoftmaxFusionTypes.none
+    assert get_fusion_type(args(False, True)) is SoftmaxFusionTypes.general
+    assert get_fusion_type(args(True, False)) is SoftmaxFusionTypes.upper_triang
+    assert get_fusion_type(args(True, True)) is SoftmaxFusionTypes.upper_triang
+
+
+def test_dropout_and_bias_arguments_on_the_unfused_branch():
+    # fusion off: softmax of (scores + bias) by the torch expression, then torch's dropout
+    m = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(2, 2, 16, 16, generator=g) * 4).bfloat16()
+    bias = torch.randn(1, 2, 16, 16, generator=g).bfloat16()
+    mask = R.get_attn_mask(16)
+    assert torch.equal(m(x, mask, bias=bias), m(x + bias, mask))
+    torch.manual_seed(5)
+    out = m(x, mask, dropout_p=0.5)
+    base = m(x, mask)
+    kept = out != 0
+    assert 0.2 < kept[..., ~mask[0, 0]].float().mean() < 0.8
+    assert torch.allclose(out[kept].float(), 2 * base[kept].float(), rtol=1e-2)
+    assert torch.equal(m(x, mask, dropout_p=0.0), base)
