@@ -6,7 +6,8 @@ extensions with torch's cpp_extension (hipifying the CUDA sources on ROCm) and
 Here the three extension APIs are thin Python modules over ONE prebuilt C-ABI
 library of hand-written gfx950 kernels, so
 
-* ``load()`` compiles that library with hipcc if it is not built yet;
+* ``load()`` compiles that library with hipcc if it is not built yet and registers the
+  extension-named modules, as the reference's JIT load leaves them importable;
 * ``load_fused_kernels()`` loads it, raises ``ImportError`` if that fails (no
   ``exit()``), and registers the modules under the reference's top-level names
   so that code doing ``import scaled_masked_softmax_cuda`` finds them.
@@ -33,6 +34,9 @@ def load(neox_args=None):
         rank = getattr(neox_args, "rank", 0) if neox_args is not None else 0
         if rank == 0:
             _lib.build()
+    if os.path.exists(_lib.LIB_PATH):
+        # the reference's JIT load leaves the three extensions importable by name; so does this
+        load_fused_kernels()
     return _lib.LIB_PATH
 
 
