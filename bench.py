@@ -461,11 +461,11 @@ def main():
             def md_fwd(t):
                 ok(lib.neox_masked_softmax_dropout_fwd(
                     t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), scale,
-                    p_drop, seed, 0, b, heads, sq, sk, b, code[dtype], stream))
+                    p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
 
             def md_bwd(t):
                 ok(lib.neox_masked_softmax_dropout_bwd(
-                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0,
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0, None,
                     b * heads * sq, sk, code[dtype], stream))
 
             z = s_[0]
@@ -485,12 +485,12 @@ def main():
 
                 def cd_fwd(t):
                     ok(lib.neox_causal_softmax_dropout_fwd(
-                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), sc, p_drop, seed, 0, B, n, n,
+                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
                         code[dt], stream))
 
                 def cd_bwd(t):
                     ok(lib.neox_causal_softmax_dropout_bwd(
-                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, B, n, n,
+                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
                         code[dt], stream))
 
                 z = s_[0]

@@ -46,19 +46,19 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_causal_softmax_dropout_fwd": (
-        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _i32, _vp]
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _i32, _vp]
     ),
     "neox_causal_softmax_dropout_bwd": (
-        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _i32, _vp]
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _i32, _vp]
     ),
     "neox_masked_softmax_dropout_fwd": (
         ctypes.c_int,
-        [_vp, _vp, _vp, _vp, _f32, _f32, _u64, _u64, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+        [_vp, _vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_masked_softmax_dropout_bwd": (
-        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _i64, _i32, _i32, _vp]
+        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _vp]
     ),
-    "neox_dropout_keep_mask": (ctypes.c_int, [_vp, _f32, _u64, _u64, _i64, _vp]),
+    "neox_dropout_keep_mask": (ctypes.c_int, [_vp, _f32, _u64, _u64, _vp, _i64, _vp]),
     "neox_get_batch_per_block": (ctypes.c_int, [_i32, _i32, _i32, _i32]),
     "neox_rope_apply": (
         ctypes.c_int,

@@ -46,9 +46,13 @@ static int check_rows(int64_t rows, int sq, int sk, const char* what) {
 
 // Dropout parameters of a call: threshold in 16-bit units and the fp32 factor 1/(1-p)
 // formed as torch's dropout kernel forms it (fp32 keep probability, then the quotient).
-static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset, const char* what) {
+static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset,
+                        const uint64_t* device_state, const char* what) {
     if (!(p >= 0.f && p <= 1.f))
         return fail(NEOX_ERR_BAD_SHAPE, "%s: dropout probability has to be between 0 and 1, but got %g", what, (double)p);
+    if (!aligned(device_state, 8))
+        return fail(NEOX_ERR_MISALIGNED, "%s: device_state must be 8-byte aligned", what);
+    d.state = device_state;
     d.seed_lo = (uint32_t)seed;
     d.seed_hi = (uint32_t)(seed >> 32);
     d.off_lo = (uint32_t)offset;
@@ -133,8 +137,8 @@ struct SoftmaxCall {
         a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * a.sq) : 0u;
         a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
     }
-    void dropout(float p, uint64_t seed, uint64_t offset) {
-        if (!status) status = make_dropout(a.drop, p, seed, offset, what);
+    void dropout(float p, uint64_t seed, uint64_t offset, const uint64_t* device_state) {
+        if (!status) status = make_dropout(a.drop, p, seed, offset, device_state, what);
     }
     void second_output(void* y_drop, const void* y) {
         if (status) return;
@@ -178,7 +182,7 @@ struct SoftmaxCall {
 __global__ __launch_bounds__(256) void keep_mask_kernel(uint8_t* keep, DropoutArgs d, uint64_t n) {
     const uint64_t group = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (group * 8 >= n) return;
-    const uint32_t bits = keep_bits8(d, group);
+    const uint32_t bits = keep_bits8(resolve(d), group);
     for (int k = 0; k < 8; ++k)
         if (group * 8 + k < n) keep[group * 8 + k] = (bits >> k) & 1u;
 }
@@ -293,60 +297,64 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
 }
 
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream) {
     SoftmaxCall c("neox_causal_softmax_dropout_fwd", dtype, {y_drop, y, x});
     c.second_output(y_drop, y);
     c.causal_rows(batches, sq, sk);
-    c.dropout(p, seed, offset);
+    c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
     return c.launch(launch_softmax_dropout_fwd, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream) {
     SoftmaxCall c("neox_causal_softmax_dropout_bwd", dtype, {dx, dy, y});
     c.causal_rows(batches, sq, sk);
-    c.dropout(p, seed, offset);
+    c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
     return c.launch(launch_softmax_dropout_bwd, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    float scale, float p, uint64_t seed, uint64_t offset, int32_t b,
+                                    float scale, float p, uint64_t seed, uint64_t offset,
+                                    const uint64_t* device_state, int32_t b,
                                     int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream) {
     SoftmaxCall c("neox_masked_softmax_dropout_fwd", dtype, {y_drop, y, x}, mask);
     c.second_output(y_drop, y);
     c.head_rows(b, np, sq, sk);
     c.mask(mask, b, np, mask_b);
-    c.dropout(p, seed, offset);
+    c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
     return c.launch(launch_softmax_dropout_fwd, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t rows, int32_t sk,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t rows, int32_t sk,
                                     int32_t dtype, void* stream) {
     SoftmaxCall c("neox_masked_softmax_dropout_bwd", dtype, {dx, dy, y});
     c.plain_rows(rows, sk);
-    c.dropout(p, seed, offset);
+    c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
     return c.launch(launch_softmax_dropout_bwd, Mask::None, stream);
 }
 
-int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset, int64_t n,
-                           void* stream) {
+int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset,
+                           const uint64_t* device_state, int64_t n, void* stream) {
     static const char* what = "neox_dropout_keep_mask";
     if (!keep) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
     if (n < 1 || n > (int64_t)1 << 40) return fail(NEOX_ERR_BAD_SHAPE, "%s: n=%lld outside [1, 2^40]", what, (long long)n);
     DropoutArgs d{};
-    if (int e = make_dropout(d, p, seed, offset, what)) return e;
+    if (int e = make_dropout(d, p, seed, offset, device_state, what)) return e;
     const uint64_t groups = ((uint64_t)n + 7) / 8;
     hipLaunchKernelGGL(keep_mask_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, keep, d, (uint64_t)n);

@@ -20,7 +20,23 @@ struct DropoutArgs {
     uint32_t off_lo, off_hi;    // low half of the counter
     uint32_t threshold;         // 0 .. 65536
     float scale;                // 1/(1-p), 0 for p = 1
+    // If not null: {seed, offset} in device memory, read when the kernel runs instead of the
+    // four words above.  A launch recorded into a HIP graph then draws a fresh pattern on
+    // every replay, provided the graph itself advances the offset stored there.
+    const uint64_t* state;
 };
+
+// The parameters a kernel works with: the by-value ones, or those in device memory.
+__device__ __forceinline__ DropoutArgs resolve(DropoutArgs d) {
+    if (d.state != nullptr) {
+        const uint64_t seed = d.state[0], offset = d.state[1];  // wave-uniform loads
+        d.seed_lo = (uint32_t)seed;
+        d.seed_hi = (uint32_t)(seed >> 32);
+        d.off_lo = (uint32_t)offset;
+        d.off_hi = (uint32_t)(offset >> 32);
+    }
+    return d;
+}
 
 __device__ __forceinline__ u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
 #pragma unroll

@@ -132,6 +132,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     const int voff = lane * 16 + wir * kChunk * 2;
 
     const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     // ALiBi: scale*(x + slope*(j - i)) = x*scale + slope2*(j - i), slope2 wave-uniform
     float slope2 = 0.f;
     if constexpr ((FLAGS & kAlibi) != 0) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
@@ -267,8 +269,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 const int c0 = (wir + WPR * c) * kChunk;
                 u32x4 o2 = u32x4{0, 0, 0, 0};
                 if (c0 < len) {
-                    const uint32_t bits = keep_bits8(a.drop, drop_group(pos.row, sk, c0) + lane);
-                    o2 = dropout8<T>(o[c], bits, a.drop.scale);
+                    const uint32_t bits = keep_bits8(drop, drop_group(pos.row, sk, c0) + lane);
+                    o2 = dropout8<T>(o[c], bits, drop.scale);
                 }
                 buf_st128<kStNt>(ry2, o2, voff + c * WPR * kChunk * 2, 0);
             }
@@ -292,6 +294,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     const int voff = lane * 16 + wir * kChunk * 2;  // the range check ignores a scalar offset
 
     const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     u32x4 rg[NCH], rp[NCH];
     {
         const uint32_t bytes = (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
@@ -320,9 +324,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                 unpack8<T>(rp[c], pv);
                 const int col = c0 + lane * kVec;
                 if constexpr ((FLAGS & kDropout) != 0) {
-                    kb[c] = keep_bits8(a.drop, drop_group(pos.row, sk, c0) + lane);
+                    kb[c] = keep_bits8(drop, drop_group(pos.row, sk, c0) + lane);
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
+                    for (int k = 0; k < 8; ++k) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 }
                 if (c0 + kChunk > len) {
                     // the lane holding the diagonal may have loaded columns past it
@@ -350,7 +354,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                 const int col = c0 + lane * kVec;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
+                    if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                     gv[k] = a.scale * (pv[k] * (gv[k] - dot));
                     if ((c0 + kChunk > len) && (col + k) >= len) gv[k] = 0.f;
                 }
@@ -406,6 +410,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     const int sk = a.sk;
     const int grp = lane / G;
     const int col0 = (lane % G) * kVec;
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     const float ninf = -__builtin_inff();
 
     const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)row0 * sk * 2, rows_here * sk * 2);
@@ -517,8 +523,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
             const u32x4 o = pack8<T>(v[c]);
             buf_st128<kStNt>(ry, o, st ? (lr * sk + col) * 2u : kOutOfRange, 0);
             if constexpr ((FLAGS & kDropout) != 0) {
-                const uint32_t bits = keep_bits8(a.drop, drop_group(row0 + lr, sk, col));
-                buf_st128<kStNt>(ry2, dropout8<T>(o, bits, a.drop.scale), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+                const uint32_t bits = keep_bits8(drop, drop_group(row0 + lr, sk, col));
+                buf_st128<kStNt>(ry2, dropout8<T>(o, bits, drop.scale), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
             }
         }
     }
@@ -537,6 +543,8 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     const int sk = a.sk;
     const int grp = lane / G;
     const int col0 = (lane % G) * kVec;
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
 
     const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)row0 * sk * 2, rows_here * sk * 2);
     const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)row0 * sk * 2, rows_here * sk * 2);
@@ -571,10 +579,10 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             unpack8<T>(rg[p][c], gv);
             unpack8<T>(rp[p][c], pv);
             kb[c] = 0xffu;
-            if constexpr ((FLAGS & kDropout) != 0) kb[c] = keep_bits8(a.drop, drop_group(row0 + lr, sk, col0 + c * kChunk));
+            if constexpr ((FLAGS & kDropout) != 0) kb[c] = keep_bits8(drop, drop_group(row0 + lr, sk, col0 + c * kChunk));
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
+                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 if ((col0 + c * kChunk + k) >= len[p]) pv[k] = 0.f;  // past the diagonal / row end
                 dot = fmaf(gv[k], pv[k], dot);
             }
@@ -588,7 +596,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             unpack8<T>(rp[p][c], pv);
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
-                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * a.drop.scale : 0.f;
+                if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 gv[k] = a.scale * (pv[k] * (gv[k] - dot));
                 if ((col + k) >= len[p]) gv[k] = 0.f;
             }
@@ -631,6 +639,8 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
     const uint32_t row = blockIdx.x;
     const int sk = a.sk;
     const uint32_t i = row % (uint32_t)a.sq;
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
     const char* x = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
     char* y = static_cast<char*>(a.out) + (size_t)row * sk * 2;
@@ -685,8 +695,8 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
         if constexpr ((FLAGS & kDropout) != 0) {
             float rounded, unused;
             Elem<T>::unpack(Elem<T>::pack(o, 0.f), rounded, unused);
-            const bool keep = j < len && keep_element(a.drop, row, sk, j);
-            Elem<T>::store1(static_cast<char*>(a.out2) + ((size_t)row * sk + j) * 2, keep ? rounded * a.drop.scale : 0.f);
+            const bool keep = j < len && keep_element(drop, row, sk, j);
+            Elem<T>::store1(static_cast<char*>(a.out2) + ((size_t)row * sk + j) * 2, keep ? rounded * drop.scale : 0.f);
         }
     }
 }
@@ -697,6 +707,8 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_bwd_generic_kernel(So
     const uint32_t row = blockIdx.x;
     const int sk = a.sk;
     const uint32_t i = row % (uint32_t)a.sq;
+    DropoutArgs drop = a.drop;
+    if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     const int len = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
     const char* g = static_cast<const char*>(a.in0) + (size_t)row * sk * 2;
     const char* p = static_cast<const char*>(a.in1) + (size_t)row * sk * 2;
@@ -704,7 +716,7 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_bwd_generic_kernel(So
 
     auto grad = [&](int j) {
         float gj = Elem<T>::load1(g + (size_t)j * 2);
-        if constexpr ((FLAGS & kDropout) != 0) gj = keep_element(a.drop, row, sk, j) ? gj * a.drop.scale : 0.f;
+        if constexpr ((FLAGS & kDropout) != 0) gj = keep_element(drop, row, sk, j) ? gj * drop.scale : 0.f;
         return gj;
     };
     float dot = 0.f;

@@ -12,6 +12,8 @@ import torch
 
 from .. import _lib
 
+from .attention_dropout import state_pointer as _state_ptr
+
 _HALF = (torch.float16, torch.bfloat16)
 
 
@@ -104,13 +106,15 @@ def backward(output_grads, softmax_results, scale_factor):
     return output_grads
 
 
-def forward_dropout(input, mask, scale_factor, p, seed, offset):
+def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None):
     """Mask-tensor softmax and the attention dropout that follows it, in one kernel.
 
     Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
     and ``dropout(softmax_results, p)`` as ``torch.nn.Dropout`` computes it from them, with
     the keep pattern drawn from Philox state ``(seed, offset)``
-    (megatron/model/transformer.py:533-539).  No counterpart in the reference's extension.
+    (megatron/model/transformer.py:533-539).  ``state``, if given, is an int64 device tensor
+    ``[seed, offset]`` read by the kernel when it runs (for launches recorded into a HIP graph)
+    and replaces the two numbers.  No counterpart in the reference's extension.
     """
     input, mask = _check_forward(input, mask)
     b, np_, sq, sk = input.shape
@@ -122,14 +126,15 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset):
         _lib.check(
             _lib.lib().neox_masked_softmax_dropout_fwd(
                 dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
-                float(scale_factor), float(p), int(seed), int(offset), b, np_, sq, sk, mask.size(0),
+                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
+                mask.size(0),
                 _lib.dtype_code(input.dtype), _lib.current_stream(input),
             )
         )
     return softmax_results, dropped
 
 
-def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset):
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset, state=None):
     """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
     that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
     output_grads, softmax_results = _check_backward(output_grads, softmax_results)
@@ -140,7 +145,7 @@ def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offse
         _lib.check(
             _lib.lib().neox_masked_softmax_dropout_bwd(
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
-                float(scale_factor), float(p), int(seed), int(offset), b * np_ * sq, sk,
+                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b * np_ * sq, sk,
                 _lib.dtype_code(output_grads.dtype), _lib.current_stream(output_grads),
             )
         )

@@ -228,10 +228,10 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inputs, scale, p):
         scale_t = _scale_tensor(scale)
-        seed, offset = _rng.take_philox_state(inputs.device)
-        probs, dropped = _causal_ext.forward_dropout(inputs, scale_t[0].item(), p, seed, offset)
+        seed, offset, state = _rng.take_philox_state(inputs.device)
+        probs, dropped = _causal_ext.forward_dropout(inputs, scale_t[0].item(), p, seed, offset, state)
         ctx.save_for_backward(probs, scale_t)
-        ctx.dropout = (p, seed, offset)
+        ctx.dropout = (p, seed, offset, state)
         return dropped
 
     @staticmethod
@@ -247,10 +247,10 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inputs, mask, scale, p):
         scale_t = _scale_tensor(scale)
-        seed, offset = _rng.take_philox_state(inputs.device)
-        probs, dropped = _masked_ext.forward_dropout(inputs, mask, scale_t[0].item(), p, seed, offset)
+        seed, offset, state = _rng.take_philox_state(inputs.device)
+        probs, dropped = _masked_ext.forward_dropout(inputs, mask, scale_t[0].item(), p, seed, offset, state)
         ctx.save_for_backward(probs, scale_t)
-        ctx.dropout = (p, seed, offset)
+        ctx.dropout = (p, seed, offset, state)
         return dropped
 
     @staticmethod
@@ -326,15 +326,15 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
 
     def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p, bias=None):
-        """Softmax and dropout in one kernel when the fused softmax serves the call, there is
-        no additive bias and no HIP graph is being captured (the generator state would be frozen
-        into the graph); otherwise the softmax above followed by torch's dropout."""
+        """Softmax and dropout in one kernel when the fused softmax serves the call and there is
+        no additive bias; otherwise the softmax above followed by torch's dropout.  Under HIP
+        graph capture the fused kernels follow ``attention_dropout.graph_state(device)``, which
+        has to exist before the capture starts."""
         b, np, sq, sk = input.size()
         fusable = (
             alibi_slopes is None
             and bias is None
             and self.is_kernel_available(mask, b, np, sq, sk)
-            and not (input.is_cuda and torch.cuda.is_current_stream_capturing())
         )
         if not fusable:
             return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes, 0.0, bias), dropout_p, True)

@@ -136,25 +136,32 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
  * pattern as bytes (1 = kept) for n elements.  (seed, offset) are the device generator's
  * Philox state; a call consumes one counter value per group, so the caller advances the
  * generator's offset by 4 (torch's granularity) per call.  0 <= p <= 1.
+ * device_state, if not NULL, points to {seed, offset} (two uint64) in device memory that the
+ * kernel reads when it runs, instead of the seed and offset arguments: a launch recorded into
+ * a HIP graph then follows a state that the graph itself advances between replays.
  * Replaces scaled_*_softmax_cuda.forward/backward followed by the attention dropout
  *   megatron/model/transformer.py:533-539 (softmax, then dropout under the RNG tracker)
  *   megatron/mpu/random.py:20-37 (the tracker that selects the generator state)
  */
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream);
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t batches, int32_t sq,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream);
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    float scale, float p, uint64_t seed, uint64_t offset, int32_t b,
+                                    float scale, float p, uint64_t seed, uint64_t offset,
+                                    const uint64_t* device_state, int32_t b,
                                     int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream);
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
-                                    uint64_t seed, uint64_t offset, int64_t rows, int32_t sk,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int64_t rows, int32_t sk,
                                     int32_t dtype, void* stream);
-int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset, int64_t n,
-                           void* stream);
+int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset,
+                           const uint64_t* device_state, int64_t n, void* stream);
 
 /*
  * Rows-per-block figure the reference's dispatcher predicate consumes; kept for

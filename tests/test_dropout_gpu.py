@@ -372,3 +372,83 @@ def test_statistics_of_the_fused_output(device):
     err = (acc / n - y).abs()
     bound = 5 * y * (0.3 / 0.7 / n) ** 0.5 + 1e-3
     assert (err <= bound).all()
+
+
+# ---------------------------------------------------------------------------------
+# HIP graphs: the pattern follows a device-resident state that the graph advances
+# ---------------------------------------------------------------------------------
+def test_device_state_argument_equals_the_numbers_it_holds(device):
+    x = scores((3, 264, 264), torch.bfloat16, device, 30)
+    g = normal((3, 264, 264), torch.bfloat16, device, 31)
+    seed, offset = 2**45 + 17, rng.GRAPH_OFFSET_BASE + 40
+    state = torch.tensor([seed, offset], dtype=torch.int64, device=device)
+    y0, d0 = causal_ext.forward_dropout(x, 0.25, 0.2, seed, offset)
+    y1, d1 = causal_ext.forward_dropout(x, 0.25, 0.2, 0, 0, state)
+    assert torch.equal(y0, y1) and torch.equal(d0, d1)
+    assert torch.equal(causal_ext.backward_dropout(g.clone(), y0, 0.25, 0.2, seed, offset),
+                       causal_ext.backward_dropout(g.clone(), y0, 0.25, 0.2, 0, 0, state))
+    assert torch.equal(rng.keep_mask(1000, 0.2, seed, offset, device), rng.keep_mask(1000, 0.2, 0, 0, device, state))
+    with pytest.raises(RuntimeError, match="int64 device tensor"):
+        causal_ext.forward_dropout(x, 0.25, 0.2, 0, 0, state.int())
+
+
+def test_fused_dropout_in_a_hip_graph_draws_a_fresh_pattern_per_replay(device):
+    shape = (2, 4, 256, 256)
+    x = scores(shape, torch.float16, device, 32).requires_grad_(True)
+    g = normal(shape, torch.float16, device, 33)
+    pad = R.padding_mask(torch.tensor([256, 100]), 256, 256, device)
+    causal = R.get_attn_mask(256, device)
+    mc = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func, True, 0.5)
+    mg = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.5)
+    assert mc.mask_is_plain_causal(causal)  # decided (with a host sync) before the capture
+    torch.manual_seed(99)
+    live = rng.graph_state(device, reseed=True)
+    first = live.tolist()
+    assert first == [99, rng.GRAPH_OFFSET_BASE + torch.cuda.default_generators[device.index].get_offset()]
+
+    out = {}
+
+    def step():
+        a = ScaledUpperTriangMaskedSoftmaxDropout.apply(x.view(-1, 256, 256), 0.5, 0.1)
+        b = mg(x, pad, dropout_p=0.1)
+        # the backward kernels write into the gradient they are given: hand them copies
+        (ga,) = torch.autograd.grad(a, x, g.view(-1, 256, 256).clone(), retain_graph=False)
+        (gb,) = torch.autograd.grad(b, x, g.clone(), retain_graph=False)
+        out.update(a=a, b=b, ga=ga, gb=gb)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # eager warm-up on the capture stream: takes the host generator, not the device state
+        side.synchronize()
+        assert live.tolist() == first
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    assert live.tolist() == first  # capturing executes nothing
+
+    seen = []
+    for rep in range(3):
+        for t in out.values():
+            t.fill_(float("nan"))  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        seed, off_a = first[0], first[1] + 2 * rep * rng.OFFSET_STEP
+        off_b = off_a + rng.OFFSET_STEP
+        assert live.tolist() == [seed, first[1] + 2 * (rep + 1) * rng.OFFSET_STEP]
+        xd = x.detach()
+        ya, want_a = causal_ext.forward_dropout(xd.view(-1, 256, 256), 0.5, 0.1, seed, off_a)
+        yb, want_b = masked_ext.forward_dropout(xd, pad, 0.5, 0.1, seed, off_b)
+        assert torch.equal(out["a"], want_a) and torch.equal(out["b"], want_b)
+        assert torch.equal(out["ga"].view(-1, 256, 256),
+                           causal_ext.backward_dropout(g.view(-1, 256, 256).clone(), ya, 0.5, 0.1, seed, off_a))
+        assert torch.equal(out["gb"], masked_ext.backward_dropout(g.clone(), yb, 0.5, 0.1, seed, off_b))
+        seen.append(out["a"].clone())
+    assert not torch.equal(seen[0], seen[1]) and not torch.equal(seen[1], seen[2])
+    # capture without the state prepared is refused with a clear message
+    rng._graph_states.pop(device.index)
+    with pytest.raises(RuntimeError, match="graph_state"):
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                mg(x.detach(), pad, dropout_p=0.1)

@@ -126,21 +126,21 @@ def test_dropout_and_bias_entry_points_validate_before_touching_the_gpu():
     other = (ctypes.c_uint16 * 64)()
     third = (ctypes.c_uint16 * 64)()
     a, b, c = (ctypes.addressof(v) for v in (buf, other, third))
-    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, 1.0, 1.5, 0, 0, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, 1.0, 1.5, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -3 and "between 0 and 1" in msg
-    status, msg = _call("neox_causal_softmax_dropout_fwd", a, a, c, 1.0, 0.1, 0, 0, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, a, c, 1.0, 0.1, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -4 and "alias" in msg
-    status, msg = _call("neox_causal_softmax_dropout_fwd", None, b, c, 1.0, 0.1, 0, 0, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", None, b, c, 1.0, 0.1, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -1
-    status, msg = _call("neox_causal_softmax_dropout_bwd", a, b, c, 1.0, -0.1, 0, 0, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_bwd", a, b, c, 1.0, -0.1, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -3
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, 1.0, 0.1, 0, 0, 1, 1, 8, 8, 1, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
     assert status == -1
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, 1.0, 0.1, 0, 0, 2, 1, 8, 8, 3, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "mask batch" in msg
-    status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, 0, 8, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 0, 8, 0, None)
     assert status == -3
-    status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, 4, 8, 2, None)
+    status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 4, 8, 2, None)
     assert status == -2
     status, msg = _call("neox_causal_softmax_bias_fwd", a, b, c, 1.0, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "bias batch" in msg
@@ -150,9 +150,11 @@ def test_dropout_and_bias_entry_points_validate_before_touching_the_gpu():
     assert status == -3 and "bias batch" in msg
     status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 1, 1, 7, None)
     assert status == -2
-    status, msg = _call("neox_dropout_keep_mask", None, 0.1, 0, 0, 8, None)
+    status, msg = _call("neox_dropout_keep_mask", None, 0.1, 0, 0, None, 8, None)
     assert status == -1
-    status, msg = _call("neox_dropout_keep_mask", a, float("nan"), 0, 0, 8, None)
+    status, msg = _call("neox_dropout_keep_mask", a, float("nan"), 0, 0, None, 8, None)
     assert status == -3
-    status, msg = _call("neox_dropout_keep_mask", a, 0.1, 0, 0, 0, None)
+    status, msg = _call("neox_dropout_keep_mask", a, 0.1, 0, 0, None, 0, None)
     assert status == -3
+    status, msg = _call("neox_dropout_keep_mask", a, 0.1, 0, 0, a + 4, 8, None)  # state not 8-byte aligned
+    assert status == -5 and "device_state" in msg
