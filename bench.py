@@ -460,7 +460,7 @@ def main():
 
             def md_fwd(t):
                 ok(lib.neox_masked_softmax_dropout_fwd(
-                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), scale,
+                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), None, 0, scale,
                     p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
 
             def md_bwd(t):
@@ -485,8 +485,8 @@ def main():
 
                 def cd_fwd(t):
                     ok(lib.neox_causal_softmax_dropout_fwd(
-                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
-                        code[dt], stream))
+                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), None, None, 0, sc, p_drop, seed, 0, None,
+                        B, 1, n, n, code[dt], stream))
 
                 def cd_bwd(t):
                     ok(lib.neox_causal_softmax_dropout_bwd(

@@ -46,14 +46,16 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_causal_softmax_dropout_fwd": (
-        ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _i32, _vp]
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_causal_softmax_dropout_bwd": (
         ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _i32, _vp]
     ),
     "neox_masked_softmax_dropout_fwd": (
         ctypes.c_int,
-        [_vp, _vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+        [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
+         _vp],
     ),
     "neox_masked_softmax_dropout_bwd": (
         ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _vp]

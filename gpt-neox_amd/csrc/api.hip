@@ -126,16 +126,31 @@ struct SoftmaxCall {
         a.mask_bytes = fits32((uint64_t)mask_b * (uint64_t)a.sq * (uint64_t)a.sk);
         vec_ok = vec_ok && aligned(m, 8);
     }
-    // bias [bias_b, np, sq, sk] in the dtype of the scores (one of the constructor's tensors)
+    // bias [bias_b, np, sq, sk] in the dtype of the scores
     void bias(const void* t, int b, int np, int bias_b) {
         if (status) return;
         if (bias_b != 1 && bias_b != b) {
             status = fail(NEOX_ERR_BAD_SHAPE, "%s: bias batch dim %d must be 1 or b=%d", what, bias_b, b);
             return;
         }
+        if (!aligned(t, 2)) {
+            status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+            return;
+        }
+        vec_ok = vec_ok && aligned(t, 16);
         a.bias = t;
         a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * a.sq) : 0u;
         a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
+    }
+    // ALiBi slopes, fp32 [np]
+    void alibi(const float* slopes, int np) {
+        if (status) return;
+        if (!aligned(slopes, 4)) {
+            status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+            return;
+        }
+        a.slopes = slopes;
+        a.np = (uint32_t)np;
     }
     void dropout(float p, uint64_t seed, uint64_t offset, const uint64_t* device_state) {
         if (!status) status = make_dropout(a.drop, p, seed, offset, device_state, what);
@@ -236,11 +251,9 @@ int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, f
                                   int32_t np, int32_t sq, int32_t sk, int32_t dtype, void* stream) {
     SoftmaxCall c("neox_causal_softmax_alibi_fwd", dtype, {y, x}, slopes);
     c.head_rows(b, np, sq, sk);
-    if (!c.status && !aligned(slopes, 4)) c.status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", c.what);
+    c.alibi(slopes, np);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    c.a.slopes = slopes;
-    c.a.np = (uint32_t)np;
     return c.launch(launch_softmax_fwd, Mask::Causal, stream);
 }
 
@@ -276,7 +289,7 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
 int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
                                  int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
                                  void* stream) {
-    SoftmaxCall c("neox_causal_softmax_bias_fwd", dtype, {y, x, bias});
+    SoftmaxCall c("neox_causal_softmax_bias_fwd", dtype, {y, x}, bias);
     c.head_rows(b, np, sq, sk);
     c.bias(bias, b, np, bias_b);
     if (c.status) return c.status;
@@ -287,7 +300,8 @@ int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float
 int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
                                  float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
                                  int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream) {
-    SoftmaxCall c("neox_masked_softmax_bias_fwd", dtype, {y, x, bias}, mask);
+    if (!bias) return fail(NEOX_ERR_NULL_POINTER, "neox_masked_softmax_bias_fwd: null tensor pointer");
+    SoftmaxCall c("neox_masked_softmax_bias_fwd", dtype, {y, x}, mask);
     c.head_rows(b, np, sq, sk);
     c.mask(mask, b, np, mask_b);
     c.bias(bias, b, np, bias_b);
@@ -296,13 +310,19 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
     return c.launch(launch_softmax_bias_fwd, Mask::Bytes, stream);
 }
 
-int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
+int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const float* alibi_slopes,
+                                    const void* bias, int32_t bias_b, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
-                                    int64_t batches, int32_t sq,
-                                    int32_t sk, int32_t dtype, void* stream) {
-    SoftmaxCall c("neox_causal_softmax_dropout_fwd", dtype, {y_drop, y, x});
+                                    int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t dtype,
+                                    void* stream) {
+    static const char* what = "neox_causal_softmax_dropout_fwd";
+    if (alibi_slopes && bias)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: give ALiBi slopes or a bias tensor, not both", what);
+    SoftmaxCall c(what, dtype, {y_drop, y, x});
     c.second_output(y_drop, y);
-    c.causal_rows(batches, sq, sk);
+    c.head_rows(b, np, sq, sk);
+    if (alibi_slopes) c.alibi(alibi_slopes, np);
+    if (bias) c.bias(bias, b, np, bias_b);
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
@@ -322,14 +342,15 @@ int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
 }
 
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    float scale, float p, uint64_t seed, uint64_t offset,
-                                    const uint64_t* device_state, int32_t b,
-                                    int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                    const void* bias, int32_t bias_b, float scale, float p,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream) {
     SoftmaxCall c("neox_masked_softmax_dropout_fwd", dtype, {y_drop, y, x}, mask);
     c.second_output(y_drop, y);
     c.head_rows(b, np, sq, sk);
     c.mask(mask, b, np, mask_b);
+    if (bias) c.bias(bias, b, np, bias_b);
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);

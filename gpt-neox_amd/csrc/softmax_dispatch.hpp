@@ -14,33 +14,41 @@
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 #pragma once
 
+#include <type_traits>
+
 #include "internal.hpp"
 
 namespace neox {
 
-// kernel flags: the causal forward has a second instantiation that adds the ALiBi bias
-template <Mask M, bool BWD>
-static bool wants_alibi(const SoftmaxArgs& a) {
-    return !BWD && M == Mask::Causal && a.slopes != nullptr;
+// Forward features selected at run time on top of a translation unit's EXTRA flags: the
+// ALiBi slopes (causal kernels) and, in the dropout unit, a bias tensor.  `launch` is called
+// with the resulting flag set as a compile-time constant.
+template <Mask M, bool BWD, int EXTRA, typename Launch>
+static hipError_t with_runtime_flags(const SoftmaxArgs& a, Launch&& launch) {
+    if constexpr (!BWD && (EXTRA & kBias) == 0) {
+        if constexpr (M == Mask::Causal) {
+            if (a.slopes != nullptr) return launch(std::integral_constant<int, EXTRA | kAlibi>{});
+        }
+        if constexpr ((EXTRA & kDropout) != 0) {
+            if (a.bias != nullptr) return launch(std::integral_constant<int, EXTRA | kBias>{});
+        }
+    }
+    return launch(std::integral_constant<int, EXTRA>{});
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA, int NCH, int WPR, int RPB>
 static hipError_t launch_shape(const SoftmaxArgs& a, hipStream_t st) {
     const dim3 grid((a.rows + RPB - 1) / RPB);
     const dim3 block(kWave * WPR * RPB);
-    constexpr int FLAGS = kDefaultFlags | EXTRA;
-    if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
-    } else {
-        if constexpr (M == Mask::Causal && EXTRA == 0) {
-            if (wants_alibi<M, BWD>(a)) {
-                hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS | kAlibi>), grid, block, 0, st, a);
-                return hipGetLastError();
-            }
+    return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
+        constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
+        if constexpr (BWD) {
+            hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
+        } else {
+            hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
         }
-        hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
-    }
-    return hipGetLastError();
+        return hipGetLastError();
+    });
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA>
@@ -59,19 +67,15 @@ template <typename T, Mask M, bool BWD, int EXTRA, int G, int R, int C>
 static hipError_t launch_packed_shape(const SoftmaxArgs& a, hipStream_t st) {
     const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
     const dim3 grid((a.rows + per_block - 1) / per_block);
-    constexpr int FLAGS = kDefaultFlags | EXTRA;
-    if constexpr (BWD) {
-        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
-    } else {
-        if constexpr (M == Mask::Causal && EXTRA == 0) {
-            if (wants_alibi<M, BWD>(a)) {
-                hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS | kAlibi, R, C>), grid, dim3(256), 0, st, a);
-                return hipGetLastError();
-            }
+    return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
+        constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
+        if constexpr (BWD) {
+            hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
+        } else {
+            hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
         }
-        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
-    }
-    return hipGetLastError();
+        return hipGetLastError();
+    });
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA, int G>
@@ -103,7 +107,7 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         // the forward mask kernel addresses the mask through one 32-bit-sized buffer
         // and the bias kernel the bias tensor
         const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
-                             ((EXTRA & kBias) == 0 || a.bias_bytes != 0);
+                            (a.bias == nullptr || a.bias_bytes != 0);
         if (fits32) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
         return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
     }

@@ -653,11 +653,12 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
     // ALiBi (causal only): slopes given -> scores get slope*(j - i) before the scale
     const float slope2 = (MASK == Mask::Causal && a.slopes != nullptr)
                              ? a.slopes[(row / (uint32_t)a.sq) % a.np] * a.scale : 0.f;
+    // bias tensor given -> added to the scores before the scale (decided at run time here)
     const char* brow = nullptr;
-    if constexpr ((FLAGS & kBias) != 0) brow = static_cast<const char*>(a.bias) + (size_t)bias_row(row, a) * sk * 2;
+    if (a.bias != nullptr) brow = static_cast<const char*>(a.bias) + (size_t)bias_row(row, a) * sk * 2;
     auto score = [&](int j) {
         float xj = Elem<T>::load1(x + (size_t)j * 2);
-        if constexpr ((FLAGS & kBias) != 0) xj += Elem<T>::load1(brow + (size_t)j * 2);
+        if (brow != nullptr) xj += Elem<T>::load1(brow + (size_t)j * 2);
         return fmaf(xj, a.scale, slope2 * (float)(j - (int)i));
     };
 

@@ -106,7 +106,7 @@ def backward(output_grads, softmax_results, scale_factor):
     return output_grads
 
 
-def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None):
+def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias=None):
     """Mask-tensor softmax and the attention dropout that follows it, in one kernel.
 
     Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
@@ -114,9 +114,15 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None):
     the keep pattern drawn from Philox state ``(seed, offset)``
     (megatron/model/transformer.py:533-539).  ``state``, if given, is an int64 device tensor
     ``[seed, offset]`` read by the kernel when it runs (for launches recorded into a HIP graph)
-    and replaces the two numbers.  No counterpart in the reference's extension.
+    and replaces the two numbers.  ``bias`` (optional) is added to the scores as in
+    :func:`forward_bias`.  No counterpart in the reference's extension.
     """
     input, mask = _check_forward(input, mask)
+    if bias is not None:
+        from .scaled_upper_triang_masked_softmax_cuda import check_bias
+
+        _lib.require_gpu(bias)
+        bias = check_bias(input, bias)
     b, np_, sq, sk = input.shape
     softmax_results = torch.empty_like(input, requires_grad=False)
     dropped = torch.empty_like(input, requires_grad=False)
@@ -126,6 +132,7 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None):
         _lib.check(
             _lib.lib().neox_masked_softmax_dropout_fwd(
                 dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
+                bias.data_ptr() if bias is not None else None, bias.size(0) if bias is not None else 0,
                 float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
                 mask.size(0),
                 _lib.dtype_code(input.dtype), _lib.current_stream(input),

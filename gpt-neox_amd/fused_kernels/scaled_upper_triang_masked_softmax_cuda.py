@@ -131,7 +131,7 @@ def backward(output_grads, softmax_results, scale_factor):
     return output_grads
 
 
-def forward_dropout(input, scale_factor, p, seed, offset, state=None):
+def forward_dropout(input, scale_factor, p, seed, offset, state=None, slopes=None, bias=None):
     """Causal softmax and the attention dropout that follows it, in one kernel.
 
     Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
@@ -139,15 +139,29 @@ def forward_dropout(input, scale_factor, p, seed, offset, state=None):
     the keep pattern drawn from Philox state ``(seed, offset)``
     (megatron/model/transformer.py:533-539).  ``state``, if given, is an int64 device tensor
     ``[seed, offset]`` read by the kernel when it runs (for launches recorded into a HIP graph)
-    and replaces the two numbers.  No counterpart in the reference's extension.
+    and replaces the two numbers.  ``input`` is ``[attn_batches, sq, sk]``, or ``[b, np, sq, sk]``
+    -- required with ``slopes`` (ALiBi, as :func:`forward_alibi`) or ``bias`` (as
+    :func:`forward_bias`), of which at most one may be given.  No counterpart in the
+    reference's extension.
     """
-    if input.dim() != 3:
-        raise RuntimeError("expected 3D tensor")
+    if input.dim() not in (3, 4):
+        raise RuntimeError("expected 3D or 4D tensor")
+    if input.dim() == 3 and (slopes is not None or bias is not None):
+        raise RuntimeError("expected 4D tensor")
+    if slopes is not None and bias is not None:
+        raise RuntimeError("give ALiBi slopes or a bias tensor, not both")
     if input.dtype not in _HALF:
         raise RuntimeError("Only fp16 and bf16 are supported")
-    _lib.require_gpu(input)
+    _lib.require_gpu(input, slopes, bias)
     input = input.contiguous()
-    attn_batches, sq, sk = input.shape
+    b, np_ = (input.shape[0], 1) if input.dim() == 3 else input.shape[:2]
+    sq, sk = input.shape[-2:]
+    if slopes is not None:
+        if slopes.numel() != np_:
+            raise RuntimeError(f"expected {np_} ALiBi slopes (one per head), got {slopes.numel()}")
+        slopes = slopes.detach().to(dtype=torch.float32).contiguous()
+    if bias is not None:
+        bias = check_bias(input, bias)
     softmax_results = torch.empty_like(input, requires_grad=False)
     dropped = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
@@ -155,9 +169,11 @@ def forward_dropout(input, scale_factor, p, seed, offset, state=None):
     with torch.cuda.device(input.device):
         _lib.check(
             _lib.lib().neox_causal_softmax_dropout_fwd(
-                dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), float(scale_factor),
-                float(p), int(seed), int(offset), _state_ptr(state), attn_batches, sq, sk, _lib.dtype_code(input.dtype),
-                _lib.current_stream(input),
+                dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(),
+                slopes.data_ptr() if slopes is not None else None,
+                bias.data_ptr() if bias is not None else None, bias.size(0) if bias is not None else 0,
+                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
+                _lib.dtype_code(input.dtype), _lib.current_stream(input),
             )
         )
     return softmax_results, dropped
@@ -165,9 +181,9 @@ def forward_dropout(input, scale_factor, p, seed, offset, state=None):
 
 def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset, state=None):
     """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
-    that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
-    if output_grads.dim() != 3 or softmax_results.dim() != 3:
-        raise RuntimeError("expected 3D tensor")
+    that tensor is contiguous.  ``(p, seed, offset, state)`` are those of the forward call."""
+    if output_grads.dim() not in (3, 4) or softmax_results.dim() != output_grads.dim():
+        raise RuntimeError("expected 3D or 4D tensor")
     if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
         raise RuntimeError("Only fp16 and bf16 are supported")
     if output_grads.dtype != softmax_results.dtype or output_grads.shape != softmax_results.shape:
@@ -175,7 +191,8 @@ def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offse
     _lib.require_gpu(output_grads, softmax_results)
     output_grads = output_grads.contiguous()
     softmax_results = softmax_results.contiguous()
-    attn_batches, sq, sk = output_grads.shape
+    sq, sk = output_grads.shape[-2:]
+    attn_batches = output_grads.numel() // max(1, sq * sk)
     if output_grads.numel() == 0:
         return output_grads
     with torch.cuda.device(output_grads.device):

@@ -223,40 +223,53 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
     pattern comes from the device's default generator (see ``fused_kernels.attention_dropout``),
     so call it where the reference calls the dropout: inside the RNG tracker's ``fork()``.
     The undropped probabilities are kept for the backward pass; the pattern is regenerated
-    there from the saved generator state instead of being stored."""
+    there from the saved generator state instead of being stored.
+
+    ``inputs``: ``[attn_batches, sq, sk]``, or ``[b, np, sq, sk]`` -- required with ``slopes``
+    (ALiBi slopes ``[np]``) or ``bias`` (``[1 or b, np, sq, sk]``, differentiable), which add to
+    the scores as in ``ScaledUpperTriangMaskedSoftmaxAlibi`` / ``...Bias``; at most one of them."""
 
     @staticmethod
-    def forward(ctx, inputs, scale, p):
+    def forward(ctx, inputs, scale, p, slopes=None, bias=None):
         scale_t = _scale_tensor(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
-        probs, dropped = _causal_ext.forward_dropout(inputs, scale_t[0].item(), p, seed, offset, state)
+        probs, dropped = _causal_ext.forward_dropout(
+            inputs, scale_t[0].item(), p, seed, offset, state, slopes=slopes, bias=bias)
         ctx.save_for_backward(probs, scale_t)
         ctx.dropout = (p, seed, offset, state)
+        ctx.bias_shape = None if bias is None else bias.shape
         return dropped
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _causal_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout), None, None
+        grads = _causal_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout)
+        wants_bias = ctx.bias_shape is not None and ctx.needs_input_grad[4]
+        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None)
 
 
 class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     """Mask-tensor softmax followed by dropout with probability ``p``, in one kernel per
-    pass; see ``ScaledUpperTriangMaskedSoftmaxDropout``."""
+    pass; see ``ScaledUpperTriangMaskedSoftmaxDropout``.  ``bias`` (optional,
+    ``[1 or b, np, sq, sk]``, differentiable) adds to the scores."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, p):
+    def forward(ctx, inputs, mask, scale, p, bias=None):
         scale_t = _scale_tensor(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
-        probs, dropped = _masked_ext.forward_dropout(inputs, mask, scale_t[0].item(), p, seed, offset, state)
+        probs, dropped = _masked_ext.forward_dropout(
+            inputs, mask, scale_t[0].item(), p, seed, offset, state, bias=bias)
         ctx.save_for_backward(probs, scale_t)
         ctx.dropout = (p, seed, offset, state)
+        ctx.bias_shape = None if bias is None else bias.shape
         return dropped
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout), None, None, None
+        grads = _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout)
+        wants_bias = ctx.bias_shape is not None and ctx.needs_input_grad[4]
+        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None)
 
 
 class SoftmaxFusionTypes(enum.Enum):
@@ -326,23 +339,22 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
 
     def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p, bias=None):
-        """Softmax and dropout in one kernel when the fused softmax serves the call and there is
-        no additive bias; otherwise the softmax above followed by torch's dropout.  Under HIP
+        """Softmax and dropout in one kernel per pass when the fused softmax serves the call --
+        with the ALiBi slopes (plain causal mask only) or a bias tensor folded in as well, though
+        not both at once; otherwise the softmax above followed by torch's dropout.  Under HIP
         graph capture the fused kernels follow ``attention_dropout.graph_state(device)``, which
         has to exist before the capture starts."""
         b, np, sq, sk = input.size()
-        fusable = (
-            alibi_slopes is None
-            and bias is None
-            and self.is_kernel_available(mask, b, np, sq, sk)
-        )
+        fusable = self.is_kernel_available(mask, b, np, sq, sk) and (alibi_slopes is None or bias is None)
+        causal = fusable and self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask)
+        if fusable and alibi_slopes is not None and not causal:
+            fusable = False  # the mask-tensor kernels have no ALiBi variant
         if not fusable:
             return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes, 0.0, bias), dropout_p, True)
         scale = 1.0 if self.scale is None else self.scale
-        if self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
-            probs = ScaledUpperTriangMaskedSoftmaxDropout.apply(input.view(-1, sq, sk), scale, dropout_p)
-            return probs.view(b, np, sq, sk)
-        return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p)
+        if causal:
+            return ScaledUpperTriangMaskedSoftmaxDropout.apply(input, scale, dropout_p, alibi_slopes, bias)
+        return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p, bias)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """Whether the fused branch serves this call.

@@ -136,6 +136,9 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
  * pattern as bytes (1 = kept) for n elements.  (seed, offset) are the device generator's
  * Philox state; a call consumes one counter value per group, so the caller advances the
  * generator's offset by 4 (torch's granularity) per call.  0 <= p <= 1.
+ * The forward entry points take x as [b, np, sq, sk] and two optional additions to the scores,
+ * NULL when absent: alibi_slopes (causal only, as neox_causal_softmax_alibi_fwd) or a bias tensor
+ * [bias_b, np, sq, sk] (as neox_*_softmax_bias_fwd), not both.
  * device_state, if not NULL, points to {seed, offset} (two uint64) in device memory that the
  * kernel reads when it runs, instead of the seed and offset arguments: a launch recorded into
  * a HIP graph then follows a state that the graph itself advances between replays.
@@ -143,18 +146,19 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
  *   megatron/model/transformer.py:533-539 (softmax, then dropout under the RNG tracker)
  *   megatron/mpu/random.py:20-37 (the tracker that selects the generator state)
  */
-int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, float scale, float p,
+int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const float* alibi_slopes,
+                                    const void* bias, int32_t bias_b, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
-                                    int64_t batches, int32_t sq,
-                                    int32_t sk, int32_t dtype, void* stream);
+                                    int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t dtype,
+                                    void* stream);
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
                                     int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream);
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    float scale, float p, uint64_t seed, uint64_t offset,
-                                    const uint64_t* device_state, int32_t b,
-                                    int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                    const void* bias, int32_t bias_b, float scale, float p,
+                                    uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                    int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream);
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,

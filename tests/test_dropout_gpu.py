@@ -345,15 +345,27 @@ def test_module_dropout_argument(device):
     torch.manual_seed(41)
     out = mg(x, pad, dropout_p=0.1)
     assert torch.equal(out, R.dropout_with_mask(mg(x, pad), keep, 0.1))
-    # with an ALiBi bias the softmax kernel is followed by torch's dropout: same law, torch's pattern
+    # ALiBi slopes or a bias tensor are folded into the same kernel: the pattern is still ours
     slopes = torch.tensor(R.alibi_slopes(np_), device=device)
-    out = m(x, causal, alibi_slopes=slopes, dropout_p=0.5)
-    base = m(x, causal, alibi_slopes=slopes)
-    kept = out != 0
-    assert torch.equal(out, R.dropout_with_mask(base, kept, 0.5))
-    lower = ~torch.triu(torch.ones(s, s, dtype=torch.bool, device=device), 1)
-    frac = kept[..., lower].float().mean().item()
-    assert 0.45 < frac < 0.55
+    torch.manual_seed(41)
+    out = m(x, causal, alibi_slopes=slopes, dropout_p=0.1)
+    assert torch.equal(out, R.dropout_with_mask(m(x, causal, alibi_slopes=slopes), keep, 0.1))
+    rpe = scores((1, np_, s, s), torch.bfloat16, device, 26) * 0.25
+    torch.manual_seed(41)
+    out = m(x, causal, bias=rpe, dropout_p=0.1)
+    assert torch.equal(out, R.dropout_with_mask(m(x, causal, bias=rpe), keep, 0.1))
+    torch.manual_seed(41)
+    out = mg(x, pad, bias=rpe, dropout_p=0.1)
+    assert torch.equal(out, R.dropout_with_mask(mg(x, pad, bias=rpe), keep, 0.1))
+    # both at once, or ALiBi with a mask that is not the plain triangle: the softmax kernel
+    # followed by torch's dropout -- same law, torch's pattern
+    for kwargs, mask in ((dict(alibi_slopes=slopes, bias=rpe), causal), (dict(alibi_slopes=slopes), window)):
+        out = m(x, mask, dropout_p=0.5, **kwargs)
+        base = m(x, mask, **kwargs)
+        kept = out != 0
+        assert torch.equal(out, R.dropout_with_mask(base, kept, 0.5))
+        frac = (kept & (base != 0)).float().sum().item() / (base != 0).float().sum().item()
+        assert 0.45 < frac < 0.55
     # the unfused module (fusion off) takes torch's dropout as well
     mt = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.none, R.gpt2_attention_mask_func, True, 0.5)
     out = mt(x, causal, dropout_p=0.5)
@@ -452,3 +464,75 @@ def test_fused_dropout_in_a_hip_graph_draws_a_fresh_pattern_per_replay(device):
         with torch.cuda.stream(side):
             with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
                 mg(x.detach(), pad, dropout_p=0.1)
+
+
+# ---------------------------------------------------------------------------------
+# ALiBi slopes / bias tensor together with dropout
+# ---------------------------------------------------------------------------------
+COMBO_SHAPES = [(2, 3, 8, 8), (2, 2, 136, 136), (1, 4, 512, 512), (2, 2, 1024, 1024), (1, 2, 2048, 2048),
+                (1, 2, 4096, 4096), (2, 2, 37, 37)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", COMBO_SHAPES)
+def test_causal_dropout_with_alibi_or_bias(device, shape, dtype):
+    b, np_, s, _ = shape
+    x = scores(shape, dtype, device, 40)
+    g = normal(shape, dtype, device, 41)
+    slopes = torch.tensor(R.alibi_slopes(np_), device=device)
+    bias = scores((1, np_, s, s), dtype, device, 42) * 0.25
+    p, seed, offset, scale = 0.2, 77, 16, 0.125
+    keep = rng.keep_mask(x.numel(), p, seed, offset, device).view(shape)
+    for kwargs, plain in ((dict(slopes=slopes), causal_ext.forward_alibi(x, slopes, scale)),
+                          (dict(bias=bias), causal_ext.forward_bias(x, bias, scale))):
+        y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, **kwargs)
+        assert torch.equal(y, plain)
+        assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
+        dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+        ref = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
+        assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    with pytest.raises(RuntimeError, match="not both"):
+        causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
+    with pytest.raises(RuntimeError, match="4D"):
+        causal_ext.forward_dropout(x.view(-1, s, s), scale, p, seed, offset, slopes=slopes)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 3, 5, 8), (1, 3, 16, 136), (2, 2, 8, 512), (2, 2, 16, 1024), (1, 2, 8, 2048),
+                                   (2, 2, 5, 37)])
+def test_masked_dropout_with_bias(device, shape, dtype):
+    b, np_, sq, sk = shape
+    x = scores(shape, dtype, device, 43)
+    bias = scores((b, np_, sq, sk), dtype, device, 44) * 0.25
+    mask = R.padding_mask(torch.randint(1, sk + 1, (b,), generator=gen(device, 45), device=device), sq, sk, device)
+    p, seed, offset = 0.3, 5, 2**34
+    y, dropped = masked_ext.forward_dropout(x, mask, 0.5, p, seed, offset, bias=bias)
+    assert torch.equal(y, masked_ext.forward_bias(x, mask, bias, 0.5))
+    keep = rng.keep_mask(x.numel(), p, seed, offset, device).view(shape)
+    assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
+
+
+@pytest.mark.parametrize("shared", [True, False])
+def test_dropout_function_gradient_reaches_the_bias(device, shared):
+    b, np_, s = 3, 2, 64
+    shape = (b, np_, s, s)
+    x = scores(shape, torch.bfloat16, device, 46).requires_grad_(True)
+    bias = (scores((1 if shared else b, np_, s, s), torch.bfloat16, device, 47) * 0.25).requires_grad_(True)
+    g = normal(shape, torch.bfloat16, device, 48)
+    causal = R.get_attn_mask(s, device)
+    pad = R.padding_mask(torch.tensor([40, 64, 9]), s, s, device)
+    for fn, mask in ((lambda: ScaledUpperTriangMaskedSoftmaxDropout.apply(x, 0.5, 0.2, None, bias), causal),
+                     (lambda: ScaledMaskedSoftmaxDropout.apply(x, pad, 0.5, 0.2, bias), pad)):
+        x.grad = bias.grad = None
+        torch.manual_seed(61)
+        off = torch.cuda.default_generators[device.index].get_offset()
+        fn().backward(g.clone())
+        keep = rng.keep_mask(x.numel(), 0.2, 61, off, device).view(shape)
+        xr = x.detach().float().requires_grad_(True)
+        br = bias.detach().float().requires_grad_(True)
+        probs = R.softmax_fp32(xr + br, mask, 0.5)
+        (probs * keep * R.dropout_scale(0.2)).backward(g.float())
+        tol = 4 * TOL[torch.bfloat16]
+        assert max_err(x.grad, xr.grad) <= tol * max(1.0, xr.grad.abs().max().item())
+        assert bias.grad.shape == bias.shape
+        assert max_err(bias.grad, br.grad) <= tol * max(1.0, br.grad.abs().max().item()) * (b if shared else 1)

@@ -126,22 +126,28 @@ def test_dropout_and_bias_entry_points_validate_before_touching_the_gpu():
     other = (ctypes.c_uint16 * 64)()
     third = (ctypes.c_uint16 * 64)()
     a, b, c = (ctypes.addressof(v) for v in (buf, other, third))
-    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, 1.0, 1.5, 0, 0, None, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, None, None, 0, 1.0, 1.5, 0, 0, None, 1, 1, 8, 8, 0, None)
     assert status == -3 and "between 0 and 1" in msg
-    status, msg = _call("neox_causal_softmax_dropout_fwd", a, a, c, 1.0, 0.1, 0, 0, None, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, a, c, None, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 0, None)
     assert status == -4 and "alias" in msg
-    status, msg = _call("neox_causal_softmax_dropout_fwd", None, b, c, 1.0, 0.1, 0, 0, None, 1, 8, 8, 0, None)
+    status, msg = _call("neox_causal_softmax_dropout_fwd", None, b, c, None, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 0, None)
     assert status == -1
     status, msg = _call("neox_causal_softmax_dropout_bwd", a, b, c, 1.0, -0.1, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -3
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
     assert status == -1
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 3, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, None, 0, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "mask batch" in msg
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 0, 8, 0, None)
     assert status == -3
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 4, 8, 2, None)
     assert status == -2
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, a, b, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 0, None)
+    assert status == -3 and "not both" in msg
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, None, a, 3, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 0, None)
+    assert status == -3 and "bias batch" in msg
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, a + 1, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
+    assert status == -5
     status, msg = _call("neox_causal_softmax_bias_fwd", a, b, c, 1.0, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "bias batch" in msg
     status, msg = _call("neox_causal_softmax_bias_fwd", a, b, None, 1.0, 2, 1, 8, 8, 1, 0, None)
