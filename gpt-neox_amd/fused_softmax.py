@@ -30,6 +30,13 @@ Deliberate differences from the reference:
   uniform ``1/sk`` as in the torch path;
 * ``scale`` is applied in fp32 (the reference's forward narrows it to fp16/bf16);
 * a missing kernel library raises ``ImportError`` instead of calling ``exit()``.
+
+Additions (all optional, off by default): ``FusedScaleMaskSoftmax.forward`` also takes
+``alibi_slopes``, ``bias`` and ``dropout_p``, which fold the ALiBi bias, an additive bias
+tensor (relative-position bias) and the attention dropout that follows the softmax
+(megatron/model/transformer.py:526-539) into the softmax kernels; the autograd Functions
+``ScaledUpperTriangMaskedSoftmaxAlibi``, ``Scaled*SoftmaxBias`` and ``Scaled*SoftmaxDropout``
+are their building blocks.
 """
 import enum
 import weakref
