@@ -302,3 +302,38 @@ def test_public_names_and_signatures_match_the_reference_modules():
     for name in ("FusedScaleMaskSoftmax", "RotaryEmbedding", "apply_rotary_pos_emb_torch",
                  "apply_rotary_pos_emb", "AliBi", "SoftmaxFusionTypes", "SinusoidalPositionalEmbedding"):
         assert hasattr(gpt_neox_amd, name)
+
+
+def test_header_is_plain_c_and_links_from_a_c_program(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 on its own, and a C program that
+    includes it links against the library and gets status codes back (argument errors are
+    reported without a GPU)."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = os.path.join(root, "include", "neox_fused.h")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-x", "c", header],
+                   check=True)
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "neox_fused.h"\n'
+        "int main(void) {\n"
+        "    unsigned short buf[64];\n"
+        "    if (neox_fused_abi_version() != NEOX_FUSED_ABI_VERSION) return 1;\n"
+        "    if (neox_causal_softmax_fwd(NULL, buf, 1.0f, 1, 8, 8, NEOX_F16, NULL) != NEOX_ERR_NULL_POINTER) return 2;\n"
+        "    if (neox_masked_softmax_bwd(buf, buf, buf, 1.0f, 4, 8, 7, NULL) != NEOX_ERR_BAD_DTYPE) return 3;\n"
+        '    if (strstr(neox_fused_last_error(), "fp16 and bf16") == NULL) return 4;\n'
+        "    if (neox_get_batch_per_block(1024, 1024, 8, 16) != 2) return 5;\n"
+        '    puts("c abi ok");\n'
+        "    return 0;\n}\n"
+    )
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-I", os.path.dirname(header), str(src), "-o", str(exe),
+                    "-L", libdir, "-lneox_fused", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    res = subprocess.run([str(exe)], stdout=subprocess.PIPE, text=True)
+    assert res.returncode == 0 and "c abi ok" in res.stdout, (res.returncode, res.stdout)
