@@ -11,8 +11,8 @@ steps between device synchronisations; the JSON line carries
 
 * value       -- algorithmic GB/s of the step (forward + backward bytes / step time);
 * roofline    -- the dominant kernel (the backward) alone: algorithmic bytes per
-                 launch / mean launch duration from HIP events recorded on the launch
-                 stream inside the timed region, against the 8 TB/s HBM peak;
+                 launch / mean launch duration of K back-to-back launches between two HIP
+                 events on the launch stream, against the 8 TB/s HBM peak;
 * cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
                  this host's cores on a slice of the same batch;
 * all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak, the error
@@ -187,21 +187,28 @@ def main():
     for i in range(args.warmup):
         step(sets[i % len(sets)])
     torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # the timed region: exactly K steps between two device synchronisations
     t0 = time.perf_counter()
     for i in range(args.steps):
-        s = sets[i % len(sets)]
-        ev[i][0].record()
-        masked_fwd(s, b, heads, sq, sk, dtype, scale)
-        ev[i][1].record()
-        masked_bwd(s, b, heads, sq, sk, dtype, scale)
-        ev[i][2].record()
+        step(sets[i % len(sets)])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    fwd_us = statistics.mean(e[0].elapsed_time(e[1]) for e in ev) * 1e3
-    bwd_us = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) * 1e3
     value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    # each kernel alone: K launches between two HIP events on the launch stream (an event
+    # between consecutive launches would add about 2 us of idle time to every launch)
+    def launches_us(fn):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(args.steps):
+            fn(sets[i % len(sets)], b, heads, sq, sk, dtype, scale)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / args.steps
+
+    fwd_us = launches_us(masked_fwd)
+    bwd_us = launches_us(masked_bwd)
     bwd_gbps = bwd_bytes / bwd_us / 1e3
 
     result = {
@@ -238,7 +245,7 @@ def main():
             "avg_launch_us": round(bwd_us, 2),
         },
     }
-    del sets, ev
+    del sets
     torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline
