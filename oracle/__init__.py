@@ -16,5 +16,9 @@ Pins (tests/test_oracle_*.py): the reference ships no golden vectors, fixtures o
 asserting tests for this path, so every function here is pinned by closed forms,
 invariants, brute force on tiny inputs, fp64 gradcheck and -- for the rotary
 pairing convention -- the installed ``transformers`` GPT-NeoX implementation.
+The dropout expressions of ``torch_ref`` (``dropout_scale``, ``dropout_with_mask``,
+``softmax_dropout_backward_fp32``) are pinned by fp64 autograd of the unfused expression, by
+the float64 vectors ``tests/golden/dropout_*.npz`` (written from ``brute``) and, on the GPU,
+by the kept entries of ``torch.nn.functional.dropout`` itself.
 No function of this package is "parity unpinned".
 """
