@@ -486,6 +486,24 @@ int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, cons
     a.half = half;
     a.lpv = lpv;
     a.nt = has_k ? 2 : 1;
+    // In place, a rotated span that ends inside a 64-byte block is written back together with the
+    // rest of that block (unchanged pass-through dims the loads fetch anyway): the memory system
+    // then sees whole 64-byte writes instead of partial ones.
+    {
+        const int slot_bytes = w * 2, span_bytes = d_rot * 2;
+        const int pad_bytes = (64 - span_bytes % 64) % 64;
+        auto in_place_64 = [&](const void* in, const void* out, const int64_t* is, const int64_t* os) {
+            if (in != out) return false;
+            for (int i = 0; i < 3; ++i)
+                if (is[i] != os[i] || (is[i] * 2) % 64 != 0) return false;
+            return aligned(in, 64) && is[2] * 2 >= span_bytes + pad_bytes;
+        };
+        bool ok = w >= 2 && pad_bytes > 0 && pad_bytes % slot_bytes == 0 &&
+                  lpv * 2 + pad_bytes / slot_bytes <= kWave &&
+                  in_place_64(q, out_q, q_strides, out_q_strides);
+        if (ok && has_k) ok = in_place_64(k, out_k, k_strides, out_k_strides);
+        a.pad_slots = ok ? pad_bytes / slot_bytes : 0;
+    }
     return check_launch(launch_rope(a, s, collapse ? 1 : b, w, dtype, cs_dtype, backward != 0,
                                     (hipStream_t)stream),
                         what);

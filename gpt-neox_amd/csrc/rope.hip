@@ -25,9 +25,10 @@ static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipSt
     return hipGetLastError();
 }
 
-template <typename T, typename CS, bool BWD>
+template <typename T, typename CS, int W, bool BWD>
 static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStream_t st) {
-    const int vpb = 256 / (a.lpv * 2) * kSpanIters;  // vectors per block iteration
+    const int spans_per_wave = kWave / (a.lpv * 2 + a.pad_slots);
+    const int vpb = (256 / kWave) * spans_per_wave * kSpanIters;  // vectors per block iteration
     int nmax = a.t[0].n_inner;
     if (a.nt > 1 && a.t[1].n_inner > nmax) nmax = a.t[1].n_inner;
     const int iters = (nmax + vpb - 1) / vpb;
@@ -39,19 +40,22 @@ static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStr
         if (zsplit > 65535) zsplit = 65535;
         if (zsplit < 1) zsplit = 1;
     }
-    hipLaunchKernelGGL((rope_span_kernel<T, CS, BWD>), dim3(s, n_outer, zsplit), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((rope_span_kernel<T, CS, W, BWD>), dim3(s, n_outer, zsplit), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 
-// d_rot/8 slots form a power of two that fits a wave: the contiguous-span kernel applies
-static bool span_shape(const RopeArgs& a, int w) {
-    const int lps = a.lpv * 2;
-    return w == 8 && lps <= 64 && (lps & (lps - 1)) == 0;
-}
+// the rotated span is at most 64 slots of w >= 2 dims: the contiguous-span kernel applies
+static bool span_shape(const RopeArgs& a, int w) { return w >= 2 && a.lpv * 2 <= kWave; }
 
 template <typename T, typename CS, bool BWD>
 static hipError_t launch_rope_w(const RopeArgs& a, int s, int n_outer, int w, hipStream_t st) {
-    if (span_shape(a, w)) return launch_rope_span<T, CS, BWD>(a, s, n_outer, st);
+    if (span_shape(a, w)) {
+        switch (w) {
+            case 8: return launch_rope_span<T, CS, 8, BWD>(a, s, n_outer, st);
+            case 4: return launch_rope_span<T, CS, 4, BWD>(a, s, n_outer, st);
+            default: return launch_rope_span<T, CS, 2, BWD>(a, s, n_outer, st);
+        }
+    }
     switch (w) {
         case 8: return launch_rope_shape<T, CS, 8, BWD>(a, s, n_outer, st);
         case 4: return launch_rope_shape<T, CS, 4, BWD>(a, s, n_outer, st);

@@ -5,15 +5,16 @@
 // One block serves one sequence position: the position's cos/sin values are loaded
 // once into registers and reused for every head of q and k.  Two kernels:
 //
-// * rope_span_kernel -- d_rot/8 a power of two (d_rot = 16 ... 512) and 16-byte aligned
-//   layouts.  Each lane owns ONE 16-byte slot (8 dims) of a head's rotated span and
-//   consecutive lanes own consecutive slots, so a wave access covers whole contiguous
-//   spans (64 B for d_rot = 32, 256 B for d_rot = 128).  The partner dims (j +- d_rot/2)
-//   live d_rot/16 lanes away and are fetched with a wave shuffle.  q and k of one
-//   block iteration are loaded together before any arithmetic.
-// * rope_kernel -- every other head size / alignment.  threadIdx.x selects a slot of W
-//   consecutive dims in the first half of the rotated span; the thread also owns the
-//   matching W dims of the second half, so no data crosses lanes (W = 8, 4, 2, 1).
+// * rope_span_kernel -- the rotated span splits into at most 64 slots of W = 8, 4 or 2 dims
+//   (the widest the alignment of the layouts and of d_rot/2 allows).  Each lane owns ONE
+//   slot and consecutive lanes own consecutive slots, so a wave access covers whole
+//   contiguous spans (64 B for d_rot = 32, 256 B for d_rot = 128, 48 B for d_rot = 24).  The
+//   partner dims (j +- d_rot/2) live d_rot/(2W) lanes away and are fetched with a wave
+//   shuffle.  q and k of one block iteration are loaded together before any arithmetic.
+// * rope_kernel -- the rest (odd d_rot/2, 2-byte aligned layouts, spans of more than 64
+//   slots).  threadIdx.x selects a slot of W consecutive dims in the first half of the
+//   rotated span; the thread also owns the matching W dims of the second half, so no data
+//   crosses lanes (W = 8, 4, 2, 1).
 //
 // In both, a lane reads everything it needs before it writes, and a pair
 // (j, j + d_rot/2) is written by the lane(s) that read it, so in-place operation is
@@ -46,6 +47,7 @@ struct RopeArgs {
     int32_t half;        // d_rot / 2
     int32_t lpv;         // slots per vector = half / W
     int32_t nt;          // 1: q only, 2: q and k
+    int32_t pad_slots;   // span kernel, in place: slots after the rotated span that are rewritten unchanged
 };
 
 template <int W>
@@ -186,35 +188,66 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
 // ---- contiguous-span kernel -----------------------------------------------------------
 constexpr int kSpanIters = 2;  // head vectors per thread and tensor whose loads are in flight together
 
-template <typename T, typename CS, bool BWD>
+template <int W, bool NT>
+__device__ __forceinline__ void load_words(const char* p, uint32_t (&w)[W / 2]) {
+    typedef typename Pack<W>::type P;
+    const P v = NT ? __builtin_nontemporal_load(reinterpret_cast<const P*>(p)) : *reinterpret_cast<const P*>(p);
+    const uint32_t* u = reinterpret_cast<const uint32_t*>(&v);
+#pragma unroll
+    for (int k = 0; k < W / 2; ++k) w[k] = u[k];
+}
+
+template <int W, bool NT>
+__device__ __forceinline__ void store_words(char* p, const uint32_t (&w)[W / 2]) {
+    typedef typename Pack<W>::type P;
+    P v;
+    uint32_t* u = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+    for (int k = 0; k < W / 2; ++k) u[k] = w[k];
+    if constexpr (NT) __builtin_nontemporal_store(v, reinterpret_cast<P*>(p));
+    else *reinterpret_cast<P*>(p) = v;
+}
+
+// Each lane owns ONE slot of W dims (16, 8 or 4 bytes) of a head's rotated span; the
+// d_rot/W lanes of a span are consecutive, a wave holds floor(64 / lanes-per-span) spans and
+// leaves its last few lanes idle when that does not divide 64 (d_rot = 24, 48, 80, 96 ...).
+template <typename T, typename CS, int W, bool BWD>
 __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
-    const int lps = a.lpv * 2;  // 16-byte slots per rotated span: a power of two <= 64
-    const int hl = a.lpv;       // lane distance to the partner slot
-    const int tid = threadIdx.x;
-    const int slot = tid & (lps - 1);
-    const int vib = tid / lps;   // vector handled in a block iteration
-    const int vpb = 256 / lps;   // vectors per block iteration
+    const int hl = a.lpv;         // slots per half span = lane distance to the partner slot
+    const int lps = hl * 2;       // slots (lanes) per rotated span
+    const int lph = lps + a.pad_slots;  // lanes per head: the span plus the copied slots, <= 64
+    const int spw = kWave / lph;  // heads per wave
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sw = lane / lph;    // head of this lane inside its wave
+    const int slot = lane - sw * lph;
+    const bool active = sw < spw;
+    const bool rotated = slot < lps;  // else: a slot that is stored back as loaded
+    const int vib = (threadIdx.x >> 6) * spw + sw;  // vector handled in a block iteration
+    const int vpb = (256 / kWave) * spw;            // vectors per block iteration
     const int pos = blockIdx.x;
     const int outer = blockIdx.y;
     const bool second = slot >= hl;
-    const int j = slot * 8;            // first dim this lane owns
-    const int jp = (slot ^ hl) * 8;    // first dim of the partner lane
+    const int partner = (second ? lane - hl : lane + hl) & (kWave - 1);  // idle lanes: any valid lane
+    const int j = slot * W;                                                 // first dim this lane owns
+    const int jt = rotated ? j : 0;                                         // its table column
+    const int jp = rotated ? (second ? slot - hl : slot + hl) * W : 0;      // the partner lane's
 
     // out = x*cos[own] + sign * partner * sin[.]: the forward pass takes sin at the lane's own
     // dims with sign -,+ for the first/second half; the backward pass takes sin at the
     // partner's dims with sign +,-.  Folding the sign into sin is exact.
-    float c[8], sn[8];
+    float c[W], sn[W];
     const int64_t crow = (int64_t)(pos + a.pos_offset) * a.cs_stride;
-    load_table<CS, 8>(a.cos, crow + j, c);
-    load_table<CS, 8>(a.sin, crow + (BWD ? jp : j), sn);
+    load_table<CS, W>(a.cos, crow + jt, c);
+    load_table<CS, W>(a.sin, crow + (BWD ? jp : jt), sn);
     if (second == BWD) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) sn[k] = -sn[k];
+        for (int k = 0; k < W; ++k) sn[k] = -sn[k];
     }
 
-    const int nq = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
-    const int nk = (a.nt > 1 && outer < a.t[1].n_outer) ? a.t[1].n_inner : 0;
-    const int nmax = max(nq, nk);
+    const int nq = (active && outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
+    const int nk = (active && a.nt > 1 && outer < a.t[1].n_outer) ? a.t[1].n_inner : 0;
+    int nmax = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;  // block-uniform loop bound
+    if (a.nt > 1 && outer < a.t[1].n_outer) nmax = max(nmax, a.t[1].n_inner);
     const int64_t qi = (int64_t)pos * a.t[0].in_stride[0] + (int64_t)outer * a.t[0].in_stride[1] + j;
     const int64_t qo = (int64_t)pos * a.t[0].out_stride[0] + (int64_t)outer * a.t[0].out_stride[1] + j;
     const int64_t ki = (int64_t)pos * a.t[1].in_stride[0] + (int64_t)outer * a.t[1].in_stride[1] + j;
@@ -223,37 +256,38 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
     const int step = vpb * kSpanIters;
     // every lane of a wave runs the same number of iterations (the shuffles need all lanes)
     for (int v0 = blockIdx.z * step; v0 < nmax; v0 += step * gridDim.z) {
-        u32x4 xq[kSpanIters], xk[kSpanIters];
+        uint32_t xq[kSpanIters][W / 2], xk[kSpanIters][W / 2];
 #pragma unroll
         for (int u = 0; u < kSpanIters; ++u) {
             const int v = v0 + u * vpb + vib;
-            xq[u] = u32x4{0, 0, 0, 0};
-            xk[u] = u32x4{0, 0, 0, 0};
-            if (v < nq) xq[u] = ld128(a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2);
-            if (v < nk) xk[u] = ld128(a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2);
+#pragma unroll
+            for (int k = 0; k < W / 2; ++k) xq[u][k] = xk[u][k] = 0u;
+            if (v < nq) load_words<W, true>(a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2, xq[u]);
+            if (v < nk) load_words<W, true>(a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2, xk[u]);
         }
 #pragma unroll
         for (int u = 0; u < kSpanIters; ++u) {
             const int v = v0 + u * vpb + vib;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const u32x4 x = t ? xk[u] : xq[u];
-                u32x4 p;
-                p.x = __shfl_xor((int)x.x, hl);
-                p.y = __shfl_xor((int)x.y, hl);
-                p.z = __shfl_xor((int)x.z, hl);
-                p.w = __shfl_xor((int)x.w, hl);
-                float xf[8], pf[8], o[8];
-                unpack8<T>(x, xf);
-                unpack8<T>(p, pf);
+                const uint32_t(&x)[W / 2] = t ? xk[u] : xq[u];
+                float xf[W], pf[W], o[W];
+#pragma unroll
+                for (int k = 0; k < W / 2; ++k) {
+                    const uint32_t p = (uint32_t)__shfl((int)x[k], partner);
+                    Elem<T>::unpack(x[k], xf[2 * k], xf[2 * k + 1]);
+                    Elem<T>::unpack(p, pf[2 * k], pf[2 * k + 1]);
+                }
                 {
 #pragma clang fp contract(off)
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) o[k] = xf[k] * c[k] + pf[k] * sn[k];
+                    for (int k = 0; k < W; ++k) o[k] = xf[k] * c[k] + pf[k] * sn[k];
                 }
                 if (v < (t ? nk : nq)) {
-                    char* op = a.t[t].out + ((t ? ko : qo) + (int64_t)v * a.t[t].out_stride[2]) * 2;
-                    st128(op, pack8<T>(o));
+                    uint32_t ow[W / 2];
+#pragma unroll
+                    for (int k = 0; k < W / 2; ++k) ow[k] = rotated ? Elem<T>::pack(o[2 * k], o[2 * k + 1]) : x[k];
+                    store_words<W, true>(a.t[t].out + ((t ? ko : qo) + (int64_t)v * a.t[t].out_stride[2]) * 2, ow);
                 }
             }
         }

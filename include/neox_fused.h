@@ -186,8 +186,11 @@ int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np);
  * cos/sin: [>= pos_offset + s, d_rot] rows of stride cs_stride elements, dtype
  * cs_dtype (NEOX_F32 or the same as dtype).  Arithmetic is fp32 with separately
  * rounded products (bit-equal to torch's fp32 q*cos + rotate_half(q)*sin), one
- * rounding to dtype on store.  out_* may alias the inputs (in place); dims
- * >= d_rot are never read or written.  k / out_k may both be NULL.
+ * rounding to dtype on store.  out_* may alias the inputs (in place).  Dims >= d_rot
+ * keep their values; out of place they are never read or written, in place those that
+ * share a 64-byte block with the end of the rotated span may be written back unchanged
+ * (whole 64-byte writes are much cheaper for the memory system than partial ones).
+ * k / out_k may both be NULL.
  * Replaces apply_rotary_pos_emb / apply_rotary_pos_emb_torch
  *   megatron/model/positional_embeddings.py:103-126
  * and fused_rotary_positional_embedding.forward_cached / backward_cached

@@ -874,3 +874,37 @@ def test_module_bias_argument(device):
     # bias and dropout together: the bias kernel followed by torch's dropout
     out = m(x, causal, bias=rpe, dropout_p=0.5)
     assert torch.equal(out, R.dropout_with_mask(y, out != 0, 0.5))
+
+
+# ---------------------------------------------------------------------------------
+# in-place partial rotary whose span ends inside a 64-byte block (head sizes of real models)
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hn,d_rot,qkv", [(96, 24, False), (96, 24, True), (64, 16, False), (64, 16, True),
+                                          (80, 20, False), (256, 64, False), (48, 24, False), (24, 24, False),
+                                          (96, 48, True), (160, 40, False)])
+def test_in_place_partial_rotary_keeps_pass_through_bits(device, hn, d_rot, qkv, dtype):
+    s, b, h = 33, 2, 5
+    width = 3 * hn if qkv else hn
+    base = normal((s, b, h, width), dtype, device, 90)
+    # pass-through dims hold every kind of bit pattern: they must come back bit for bit
+    special = torch.tensor([float("nan"), float("inf"), -float("inf"), -0.0, 65504.0, 6e-8], device=device).to(dtype)
+    bits = base.view(torch.int16).clone()
+    fill = special.view(torch.int16).repeat((width + 5) // 6)[:width]
+    passthrough = torch.ones(width, dtype=torch.bool, device=device)
+    for start in ((0, hn) if qkv else (0,)):
+        passthrough[start:start + d_rot] = False
+    bits[..., passthrough] = fill[passthrough]
+    x = bits.view(dtype)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + 3))
+    q_ref, k_ref = x[..., :d_rot].float(), (x[..., hn:hn + d_rot] if qkv else x[..., :d_rot]).float()
+    want_q, want_k = R.rotary_fp32(q_ref, k_ref, cos, sin, offset=3)
+    work = x.clone()
+    if qkv:
+        q, k, v = apply_rotary_pos_emb_qkv_(work, cos, sin, offset=3, rotary_ndims=d_rot)
+    else:
+        other = x.clone()
+        q, k = apply_rotary_pos_emb_(work, other, cos, sin, offset=3, rotary_ndims=d_rot)
+        assert torch.equal(other.view(torch.int16)[..., d_rot:], bits[..., d_rot:])
+    assert torch.equal(q[..., :d_rot], want_q.to(dtype)) and torch.equal(k[..., :d_rot], want_k.to(dtype))
+    assert torch.equal(work.view(torch.int16)[..., passthrough], bits[..., passthrough])
