@@ -430,6 +430,21 @@ def main():
                     *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
             table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
             del s_
+        # rotary at head sizes of other shipped model configurations (in place over whole heads,
+        # q and k in one launch): 20B (96-dim heads, rotary_pct 0.25), a 64-dim-head model at
+        # rotary_pct 0.25, 256-dim heads at 0.25, and full rotary on 96- and 128-dim heads
+        if want("models"):
+            extra = []
+            for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
+                                     (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
+                s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
+                nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+                for bwd in (0, 1):
+                    r = row(f"rotary {'bwd' if bwd else 'fwd'} q+k [{S},{Bb},{H},{HN}] bf16 d_rot={DR}", nb,
+                            *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, bwd), s_, 200))
+                    extra.append(rope_extras(r, S, Bb, H, HN, DR, bwd))
+                del s_
+            result["rotary_other_head_sizes"] = extra
         # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
         if want("copy"):
             nbytes = 1 << 30

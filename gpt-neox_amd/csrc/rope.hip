@@ -27,20 +27,23 @@ static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipSt
 
 template <typename T, typename CS, int W, bool BWD>
 static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStream_t st) {
-    const int spans_per_wave = kWave / (a.lpv * 2 + a.pad_slots);
-    const int vpb = (256 / kWave) * spans_per_wave * kSpanIters;  // vectors per block iteration
+    RopeArgs b = a;
+    b.lph = a.lpv * 2 + a.pad_slots;
+    b.lph_magic = (65536 + b.lph - 1) / b.lph;
+    b.spw = kWave / b.lph;
+    const int vpb = (256 / kWave) * b.spw * kSpanIters;  // vectors per block iteration
     int nmax = a.t[0].n_inner;
     if (a.nt > 1 && a.t[1].n_inner > nmax) nmax = a.t[1].n_inner;
-    const int iters = (nmax + vpb - 1) / vpb;
-    long long blocks = (long long)s * n_outer;
-    int zsplit = 1;
-    if (blocks < 4096) {
-        zsplit = (int)((4096 + blocks - 1) / blocks);
-        if (zsplit > iters) zsplit = iters;
-        if (zsplit > 65535) zsplit = 65535;
-        if (zsplit < 1) zsplit = 1;
-    }
-    hipLaunchKernelGGL((rope_span_kernel<T, CS, W, BWD>), dim3(s, n_outer, zsplit), dim3(256), 0, st, a);
+    // one loop iteration per block: many short-lived blocks measured faster than fewer blocks
+    // that loop (the cos/sin values a block reloads come from L2)
+    long long zsplit = (nmax + vpb - 1) / vpb;
+    const long long pairs = (long long)s * n_outer;
+    if (pairs * zsplit > 0x7fffffffLL) zsplit = 0x7fffffffLL / pairs;  // grid.x limit: blocks loop instead
+    if (zsplit < 1) return hipErrorInvalidValue;
+    b.zsplit = (int)zsplit;
+    b.outer_grid = n_outer;
+    b.share = (int)((nmax + zsplit - 1) / zsplit);
+    hipLaunchKernelGGL((rope_span_kernel<T, CS, W, BWD>), dim3((unsigned)(pairs * zsplit)), dim3(256), 0, st, b);
     return hipGetLastError();
 }
 

@@ -48,6 +48,13 @@ struct RopeArgs {
     int32_t lpv;         // slots per vector = half / W
     int32_t nt;          // 1: q only, 2: q and k
     int32_t pad_slots;   // span kernel, in place: slots after the rotated span that are rewritten unchanged
+    // span kernel, filled in by its launcher
+    int32_t zsplit;      // blocks sharing the vectors of one (position, outer) pair
+    int32_t outer_grid;  // extent of the outer loop in the block index
+    int32_t share;       // vectors per block: ceil(vectors of a pair / zsplit)
+    int32_t lph;         // lanes per head: slots of the rotated span plus pad_slots, <= 64
+    int32_t lph_magic;   // ceil(2^16 / lph): lane / lph == (lane * lph_magic) >> 16 for lane < 64
+    int32_t spw;         // heads per wave: 64 / lph
 };
 
 template <int W>
@@ -213,19 +220,29 @@ __device__ __forceinline__ void store_words(char* p, const uint32_t (&w)[W / 2])
 // leaves its last few lanes idle when that does not divide 64 (d_rot = 24, 48, 80, 96 ...).
 template <typename T, typename CS, int W, bool BWD>
 __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
-    const int hl = a.lpv;         // slots per half span = lane distance to the partner slot
-    const int lps = hl * 2;       // slots (lanes) per rotated span
-    const int lph = lps + a.pad_slots;  // lanes per head: the span plus the copied slots, <= 64
-    const int spw = kWave / lph;  // heads per wave
+    const int hl = a.lpv;    // slots per half span = lane distance to the partner slot
+    const int lps = hl * 2;  // slots (lanes) per rotated span
+    const int lph = a.lph, spw = a.spw;
     const int lane = threadIdx.x & (kWave - 1);
-    const int sw = lane / lph;    // head of this lane inside its wave
+    const int sw = (lane * a.lph_magic) >> 16;  // head of this lane inside its wave
     const int slot = lane - sw * lph;
     const bool active = sw < spw;
     const bool rotated = slot < lps;  // else: a slot that is stored back as loaded
     const int vib = (threadIdx.x >> 6) * spw + sw;  // vector handled in a block iteration
     const int vpb = (256 / kWave) * spw;            // vectors per block iteration
-    const int pos = blockIdx.x;
-    const int outer = blockIdx.y;
+    // blocks are numbered in memory order -- position, outer, piece of the vector loop -- so that
+    // the blocks running at any moment stream through neighbouring addresses
+    uint32_t po = blockIdx.x;
+    int piece = 0, outer = 0;
+    if (a.zsplit > 1) {  // block-uniform branches: the common shapes skip the divisions
+        piece = po % (uint32_t)a.zsplit;
+        po /= (uint32_t)a.zsplit;
+    }
+    if (a.outer_grid > 1) {
+        outer = po % (uint32_t)a.outer_grid;
+        po /= (uint32_t)a.outer_grid;
+    }
+    const int pos = po;
     const bool second = slot >= hl;
     const int partner = (second ? lane - hl : lane + hl) & (kWave - 1);  // idle lanes: any valid lane
     const int j = slot * W;                                                 // first dim this lane owns
@@ -244,10 +261,12 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
         for (int k = 0; k < W; ++k) sn[k] = -sn[k];
     }
 
-    const int nq = (active && outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
-    const int nk = (active && a.nt > 1 && outer < a.t[1].n_outer) ? a.t[1].n_inner : 0;
-    int nmax = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;  // block-uniform loop bound
-    if (a.nt > 1 && outer < a.t[1].n_outer) nmax = max(nmax, a.t[1].n_inner);
+    // the blocks of one (position, outer) pair share its vectors evenly: equal work per block keeps
+    // the XCDs, which receive consecutive blocks in turn, equally loaded
+    const int lo = piece * a.share;
+    const int hi = lo + a.share;  // block-uniform loop bound; the per-tensor bounds below clip it
+    const int nq_hi = active ? min(a.t[0].n_inner, hi) : 0;
+    const int nk_hi = (active && a.nt > 1) ? min(a.t[1].n_inner, hi) : 0;
     const int64_t qi = (int64_t)pos * a.t[0].in_stride[0] + (int64_t)outer * a.t[0].in_stride[1] + j;
     const int64_t qo = (int64_t)pos * a.t[0].out_stride[0] + (int64_t)outer * a.t[0].out_stride[1] + j;
     const int64_t ki = (int64_t)pos * a.t[1].in_stride[0] + (int64_t)outer * a.t[1].in_stride[1] + j;
@@ -255,15 +274,15 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
 
     const int step = vpb * kSpanIters;
     // every lane of a wave runs the same number of iterations (the shuffles need all lanes)
-    for (int v0 = blockIdx.z * step; v0 < nmax; v0 += step * gridDim.z) {
+    for (int v0 = lo; v0 < hi; v0 += step) {
         uint32_t xq[kSpanIters][W / 2], xk[kSpanIters][W / 2];
 #pragma unroll
         for (int u = 0; u < kSpanIters; ++u) {
             const int v = v0 + u * vpb + vib;
 #pragma unroll
             for (int k = 0; k < W / 2; ++k) xq[u][k] = xk[u][k] = 0u;
-            if (v < nq) load_words<W, true>(a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2, xq[u]);
-            if (v < nk) load_words<W, true>(a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2, xk[u]);
+            if (v < nq_hi) load_words<W, true>(a.t[0].in + (qi + (int64_t)v * a.t[0].in_stride[2]) * 2, xq[u]);
+            if (v < nk_hi) load_words<W, true>(a.t[1].in + (ki + (int64_t)v * a.t[1].in_stride[2]) * 2, xk[u]);
         }
 #pragma unroll
         for (int u = 0; u < kSpanIters; ++u) {
@@ -283,12 +302,14 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
 #pragma unroll
                     for (int k = 0; k < W; ++k) o[k] = xf[k] * c[k] + pf[k] * sn[k];
                 }
-                if (v < (t ? nk : nq)) {
-                    uint32_t ow[W / 2];
+                uint32_t ow[W / 2];
 #pragma unroll
-                    for (int k = 0; k < W / 2; ++k) ow[k] = rotated ? Elem<T>::pack(o[2 * k], o[2 * k + 1]) : x[k];
-                    store_words<W, true>(a.t[t].out + ((t ? ko : qo) + (int64_t)v * a.t[t].out_stride[2]) * 2, ow);
+                for (int k = 0; k < W / 2; ++k) {
+                    const uint32_t packed = Elem<T>::pack(o[2 * k], o[2 * k + 1]);
+                    ow[k] = rotated ? packed : x[k];
                 }
+                if (v < (t ? nk_hi : nq_hi))
+                    store_words<W, true>(a.t[t].out + ((t ? ko : qo) + (int64_t)v * a.t[t].out_stride[2]) * 2, ow);
             }
         }
     }
