@@ -140,6 +140,25 @@ def require_gpu(*tensors):
             )
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_no_guard = _NoGuard()
+
+
+def device_guard(tensor):
+    """Context that makes the tensor's device current for the launch; a no-op object when it
+    already is (the usual case: one process per GPU), which saves a few microseconds per call."""
+    if tensor.device.index == torch.cuda.current_device():
+        return _no_guard
+    return torch.cuda.device(tensor.device)
+
+
 def current_stream(tensor):
     """hipStream_t of torch's current stream on the tensor's device, as an integer."""
     return torch.cuda.current_stream(tensor.device).cuda_stream

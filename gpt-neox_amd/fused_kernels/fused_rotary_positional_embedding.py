@@ -24,7 +24,7 @@ def rope_launch(out_q, out_k, q, k, cos, sin, d_rot, pos_offset, backward):
     s, b, h_q = q.shape[0], q.shape[1], q.shape[2]
     h_k = k.shape[2] if k is not None else 0
     lib = _lib.lib()
-    with torch.cuda.device(q.device):
+    with _lib.device_guard(q):
         _lib.check(
             lib.neox_rope_apply(
                 out_q.data_ptr(), out_k.data_ptr() if k is not None else None,

@@ -43,7 +43,7 @@ def forward(input, mask, scale_factor):
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_masked_softmax_fwd(
                 softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), float(scale_factor),
@@ -67,7 +67,7 @@ def forward_bias(input, mask, bias, scale_factor):
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_masked_softmax_bias_fwd(
                 softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), bias.data_ptr(),
@@ -95,7 +95,7 @@ def backward(output_grads, softmax_results, scale_factor):
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
-    with torch.cuda.device(output_grads.device):
+    with _lib.device_guard(output_grads):
         _lib.check(
             _lib.lib().neox_masked_softmax_bwd(
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
@@ -128,7 +128,7 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias
     dropped = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results, dropped
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_masked_softmax_dropout_fwd(
                 dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
@@ -148,7 +148,7 @@ def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offse
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
-    with torch.cuda.device(output_grads.device):
+    with _lib.device_guard(output_grads):
         _lib.check(
             _lib.lib().neox_masked_softmax_dropout_bwd(
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),

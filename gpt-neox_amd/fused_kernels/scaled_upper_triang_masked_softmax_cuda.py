@@ -27,7 +27,7 @@ def forward(input, scale_factor):
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_causal_softmax_fwd(
                 softmax_results.data_ptr(), input.data_ptr(), float(scale_factor), attn_batches,
@@ -58,7 +58,7 @@ def forward_alibi(input, slopes, scale_factor):
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_causal_softmax_alibi_fwd(
                 softmax_results.data_ptr(), input.data_ptr(), slopes.data_ptr(), float(scale_factor),
@@ -95,7 +95,7 @@ def forward_bias(input, bias, scale_factor):
     softmax_results = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_causal_softmax_bias_fwd(
                 softmax_results.data_ptr(), input.data_ptr(), bias.data_ptr(), float(scale_factor),
@@ -120,7 +120,7 @@ def backward(output_grads, softmax_results, scale_factor):
     attn_batches, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
-    with torch.cuda.device(output_grads.device):
+    with _lib.device_guard(output_grads):
         _lib.check(
             _lib.lib().neox_causal_softmax_bwd(
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
@@ -166,7 +166,7 @@ def forward_dropout(input, scale_factor, p, seed, offset, state=None, slopes=Non
     dropped = torch.empty_like(input, requires_grad=False)
     if input.numel() == 0:
         return softmax_results, dropped
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input):
         _lib.check(
             _lib.lib().neox_causal_softmax_dropout_fwd(
                 dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(),
@@ -195,7 +195,7 @@ def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offse
     attn_batches = output_grads.numel() // max(1, sq * sk)
     if output_grads.numel() == 0:
         return output_grads
-    with torch.cuda.device(output_grads.device):
+    with _lib.device_guard(output_grads):
         _lib.check(
             _lib.lib().neox_causal_softmax_dropout_bwd(
                 output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),

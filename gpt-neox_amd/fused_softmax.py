@@ -38,6 +38,7 @@ tensor (relative-position bias) and the attention dropout that follows the softm
 ``ScaledUpperTriangMaskedSoftmaxAlibi``, ``Scaled*SoftmaxBias`` and ``Scaled*SoftmaxDropout``
 are their building blocks.
 """
+import ctypes
 import enum
 import weakref
 
@@ -63,21 +64,23 @@ def alibi_bias(slopes, sq, sk, device, dtype):
     return bias
 
 
-def _remember(ctx, probs, scale_t):
-    ctx.save_for_backward(probs, scale_t)
+def _fp32(scale):
+    """``scale`` rounded to fp32, as a Python float: the value the kernels receive in both
+    passes.  (The reference keeps it as a one-element fp32 CPU tensor next to the saved
+    probabilities, megatron/model/fused_softmax.py:36-41; a float on ``ctx`` costs the host a
+    few microseconds less per call.)"""
+    return ctypes.c_float(scale).value
+
+
+def _remember(ctx, probs, scale):
+    ctx.save_for_backward(probs)
+    ctx.scale = scale
     return probs
 
 
-def _scale_tensor(scale):
-    # the reference keeps the scale as a one-element fp32 CPU tensor next to the saved
-    # probabilities (fused_softmax.py:36-41); same here, so the kernels see the
-    # fp32-rounded value in both passes
-    return torch.tensor([scale])
-
-
 def _recall(ctx):
-    probs, scale_t = ctx.saved_tensors
-    return probs, scale_t[0].item()
+    (probs,) = ctx.saved_tensors
+    return probs, ctx.scale
 
 
 class _CausalMaskMemo:
@@ -127,8 +130,8 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, scale):
-        scale_t = _scale_tensor(scale)
-        return _remember(ctx, _causal_ext.forward(inputs, scale_t[0].item()), scale_t)
+        scale = _fp32(scale)
+        return _remember(ctx, _causal_ext.forward(inputs, scale), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
@@ -146,8 +149,8 @@ class ScaledUpperTriangMaskedSoftmaxAlibi(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, slopes, scale):
-        scale_t = _scale_tensor(scale)
-        return _remember(ctx, _causal_ext.forward_alibi(inputs, slopes, scale_t[0].item()), scale_t)
+        scale = _fp32(scale)
+        return _remember(ctx, _causal_ext.forward_alibi(inputs, slopes, scale), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
@@ -173,9 +176,9 @@ class ScaledUpperTriangMaskedSoftmaxBias(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, bias, scale):
-        scale_t = _scale_tensor(scale)
+        scale = _fp32(scale)
         ctx.bias_shape = bias.shape
-        return _remember(ctx, _causal_ext.forward_bias(inputs, bias, scale_t[0].item()), scale_t)
+        return _remember(ctx, _causal_ext.forward_bias(inputs, bias, scale), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
@@ -192,9 +195,9 @@ class ScaledMaskedSoftmaxBias(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, mask, bias, scale):
-        scale_t = _scale_tensor(scale)
+        scale = _fp32(scale)
         ctx.bias_shape = bias.shape
-        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale_t[0].item()), scale_t)
+        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
@@ -213,8 +216,8 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, mask, scale):
-        scale_t = _scale_tensor(scale)
-        return _remember(ctx, _masked_ext.forward(inputs, mask, scale_t[0].item()), scale_t)
+        scale = _fp32(scale)
+        return _remember(ctx, _masked_ext.forward(inputs, mask, scale), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
@@ -238,11 +241,11 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, scale, p, slopes=None, bias=None):
-        scale_t = _scale_tensor(scale)
+        scale = _fp32(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
         probs, dropped = _causal_ext.forward_dropout(
-            inputs, scale_t[0].item(), p, seed, offset, state, slopes=slopes, bias=bias)
-        ctx.save_for_backward(probs, scale_t)
+            inputs, scale, p, seed, offset, state, slopes=slopes, bias=bias)
+        _remember(ctx, probs, scale)
         ctx.dropout = (p, seed, offset, state)
         ctx.bias_shape = None if bias is None else bias.shape
         return dropped
@@ -262,11 +265,11 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, inputs, mask, scale, p, bias=None):
-        scale_t = _scale_tensor(scale)
+        scale = _fp32(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
         probs, dropped = _masked_ext.forward_dropout(
-            inputs, mask, scale_t[0].item(), p, seed, offset, state, bias=bias)
-        ctx.save_for_backward(probs, scale_t)
+            inputs, mask, scale, p, seed, offset, state, bias=bias)
+        _remember(ctx, probs, scale)
         ctx.dropout = (p, seed, offset, state)
         ctx.bias_shape = None if bias is None else bias.shape
         return dropped
