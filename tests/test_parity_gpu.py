@@ -908,3 +908,44 @@ def test_in_place_partial_rotary_keeps_pass_through_bits(device, hn, d_rot, qkv,
         assert torch.equal(other.view(torch.int16)[..., d_rot:], bits[..., d_rot:])
     assert torch.equal(q[..., :d_rot], want_q.to(dtype)) and torch.equal(k[..., :d_rot], want_k.to(dtype))
     assert torch.equal(work.view(torch.int16)[..., passthrough], bits[..., passthrough])
+
+
+def test_seeded_random_rotary_layouts(device):
+    """Random head sizes, rotary widths, head counts (q and k differ), batch layouts that can and
+    cannot be collapsed, table dtypes, offsets, in place and out of place: every kernel shape the
+    launcher can pick, each bit-equal to the fp32 expression rounded once."""
+    rs = np.random.RandomState(2024)
+    for case in range(80):
+        dtype = DTYPES[case % 2]
+        d_rot = int(rs.choice([2, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64, 72, 80, 96, 128, 160, 256, 512]))
+        extra = int(rs.choice([0, 0, 8, 16, 24, 2, 96]))
+        hn = d_rot + extra
+        s, b = int(rs.randint(1, 9)), int(rs.randint(1, 4))
+        h_q, h_k = int(rs.randint(1, 9)), int(rs.randint(1, 9))
+        offset = int(rs.randint(0, 5))
+        pad_b = int(rs.choice([0, 0, 8, 3]))  # extra elements between batch entries: (b, h) no longer collapse
+        in_place = bool(rs.randint(0, 2))
+        half_tables = bool(rs.randint(0, 2))
+
+        def make(h, seed):
+            buf = normal((s, b, h * hn + pad_b), dtype, device, seed)
+            return buf[..., : h * hn].view(s, b, h, hn)
+
+        q, k = make(h_q, 1000 + case), make(h_k, 2000 + case)
+        cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + offset))
+        if half_tables:
+            cos, sin = cos.to(dtype), sin.to(dtype)
+        want_q, want_k = R.rotary_fp32(q[..., :d_rot], k[..., :d_rot], cos, sin, offset=offset)
+        tag = (case, dtype, d_rot, hn, s, b, h_q, h_k, offset, pad_b, in_place, half_tables)
+        if in_place:
+            q0, k0 = q.clone(), k.clone()  # clones are dense: a second layout for the same data
+            for qq, kk in ((q, k), (q0, k0)):
+                keep_q, keep_k = qq[..., d_rot:].clone(), kk[..., d_rot:].clone()
+                oq, ok = apply_rotary_pos_emb_(qq, kk, cos, sin, offset=offset, rotary_ndims=d_rot)
+                assert torch.equal(oq[..., :d_rot], want_q.to(dtype)) and torch.equal(ok[..., :d_rot], want_k.to(dtype)), tag
+                assert torch.equal(oq[..., d_rot:], keep_q) and torch.equal(ok[..., d_rot:], keep_k), tag
+                if h_q != h_k:
+                    break  # one layout is enough for the rarer case
+        else:
+            oq, ok = apply_rotary_pos_emb(q[..., :d_rot], k[..., :d_rot], cos, sin, offset=offset)
+            assert torch.equal(oq, want_q.to(dtype)) and torch.equal(ok, want_k.to(dtype)), tag
