@@ -544,6 +544,26 @@ def main():
             r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
             result["fused_bias"] = [r]
             del s_, z, rpe
+        # what the memory pattern of the partial rotary costs by itself: the first 64 of every 256
+        # bytes of a 134 MB buffer loaded and stored back (cfg3's q and k), and the same number of
+        # bytes as one contiguous run
+        if want("pattern"):
+            probes = []
+            bufs = [torch.empty(2 * 2048 * 4 * 32 * 256, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(10)]
+            n_spans = 2 * 2048 * 4 * 32
+
+            def strided(t):
+                ok(lib.neox_touch_strided(t.data_ptr(), n_spans, 64, 256, stream))
+
+            def dense(t):
+                ok(lib.neox_touch_strided(t.data_ptr(), 1, n_spans * 64, n_spans * 64, stream))
+
+            probes.append(row("pattern probe: 64 of every 256 bytes, load + store back (cfg3's accesses)",
+                              2 * n_spans * 64, *time_launches(strided, bufs, 200)))
+            probes.append(row("pattern probe: the same bytes contiguous", 2 * n_spans * 64,
+                              *time_launches(dense, bufs, 200)))
+            result["memory_pattern_probes"] = probes
+            del bufs
         result["all_configs"] = table
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
         if pcts:

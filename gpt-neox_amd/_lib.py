@@ -68,6 +68,7 @@ SIGNATURES = {
          _c_i64p, _i64, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_copy_bytes": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
+    "neox_touch_strided": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp]),
 }
 
 _lock = threading.Lock()

@@ -214,6 +214,28 @@ __global__ __launch_bounds__(256) void copy_kernel(u32x4* dst, const u32x4* src,
         if (idx + k * 256 < n16) st128(dst + idx + k * 256, r[k]);
 }
 
+// Loads the first span_bytes of every stride_bytes and stores them back unchanged, one 16-byte
+// slot per lane, consecutive lanes on consecutive slots (measurement aid: the memory pattern of an
+// in-place partial rotary without its arithmetic, tables or index computations).
+__global__ __launch_bounds__(256) void touch_strided_kernel(char* buf, uint64_t slots, uint32_t slots_per_span,
+                                                            uint64_t stride_bytes, uint32_t flip) {
+    const uint64_t g0 = (uint64_t)blockIdx.x * 1024 + threadIdx.x;
+    char* p[4];
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {  // four accesses in flight per lane, as in the kernels
+        const uint64_t g = g0 + k * 256;
+        const uint64_t span = g / slots_per_span;
+        p[k] = buf + span * stride_bytes + (g - span * slots_per_span) * 16;
+        if (g < slots) v[k] = ld128(p[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        v[k].x ^= flip;  // 0 at run time; keeps the compiler from dropping the store of an unchanged value
+        if (g0 + k * 256 < slots) st128(p[k], v[k]);
+    }
+}
+
 }  // namespace neox
 
 using namespace neox;
@@ -519,6 +541,20 @@ int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
     if (blocks > 0x7fffffffULL) return fail(NEOX_ERR_BAD_SHAPE, "%s: nbytes too large", what);
     hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), n16);
+    return check_launch(hipGetLastError(), what);
+}
+
+int neox_touch_strided(void* buf, int64_t n_spans, int32_t span_bytes, int64_t stride_bytes, void* stream) {
+    static const char* what = "neox_touch_strided";
+    if (!buf) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
+    if (n_spans < 1 || span_bytes < 16 || span_bytes % 16 || stride_bytes < span_bytes || stride_bytes % 16)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: need n_spans >= 1, span_bytes and stride_bytes multiples of 16, span <= stride", what);
+    if (!aligned(buf, 16)) return fail(NEOX_ERR_MISALIGNED, "%s: pointer must be 16-byte aligned", what);
+    const uint64_t slots = (uint64_t)n_spans * (uint32_t)(span_bytes / 16);
+    const uint64_t blocks = (slots + 1023) / 1024;
+    if (blocks > 0x7fffffffULL) return fail(NEOX_ERR_BAD_SHAPE, "%s: too many spans", what);
+    hipLaunchKernelGGL(touch_strided_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<char*>(buf), slots, (uint32_t)(span_bytes / 16), (uint64_t)stride_bytes, 0u);
     return check_launch(hipGetLastError(), what);
 }
 

@@ -210,6 +210,14 @@ int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, cons
  */
 int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
 
+/*
+ * Measurement aid: loads the first span_bytes of every stride_bytes of buf (n_spans times) and
+ * stores them back unchanged -- the memory pattern of an in-place partial rotary (e.g. 64 of
+ * every 256 bytes) without its arithmetic.  Shows what that pattern costs on this memory system
+ * whatever the kernel around it does.  span_bytes, stride_bytes: multiples of 16.
+ */
+int neox_touch_strided(void* buf, int64_t n_spans, int32_t span_bytes, int64_t stride_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
