@@ -67,6 +67,9 @@ def main():
     import torch
 
     from gpt_neox_amd import _lib
+    from gpt_neox_amd.positional_embeddings import RotaryEmbedding
+    # The oracle is used as the checker of the kernels' outputs and as the timed CPU baseline
+    # only; the inputs of the measured launches are built below without it.
     from oracle import torch_ref as R
 
     if not torch.cuda.is_available():
@@ -93,7 +96,8 @@ def main():
             g0 = gen(seed + i)
             x = (torch.randn(b, heads, sq, sk, device=dev, generator=g0) * 8).to(dtype)
             lens = torch.randint(256, sk + 1, (b,), device=dev, generator=g0)
-            mask = R.padding_mask(lens, sq, sk, dev)
+            mask = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None])
+            mask = mask.expand(b, 1, sq, sk).contiguous()  # True: key j >= the sample's length
             dy = torch.randn(b, heads, sq, sk, device=dev, generator=g0).to(dtype)
             sets.append(dict(x=x, mask=mask, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x)))
         return sets
@@ -131,8 +135,8 @@ def main():
                                        scale, batches, n, n, code[dtype], stream))
 
     def rope_sets(s, b, h, hn, d_rot, dtype, seed, nsets):
-        cos, sin = R.rotary_tables(d_rot, s, 10000, torch.float)
-        cos, sin = cos.to(dev).reshape(s, d_rot), sin.to(dev).reshape(s, d_rot)
+        cos, sin = RotaryEmbedding(d_rot, s, base=10000, precision=torch.float)(torch.empty(0, device=dev), seq_len=s)
+        cos, sin = cos.reshape(s, d_rot), sin.reshape(s, d_rot)
         sets = []
         for i in range(nsets):
             g0 = gen(seed + i)

@@ -120,7 +120,12 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
     }
     if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
     if (chunks == 3) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
-    if (chunks == 4) return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
+    if (chunks == 4) {
+        // the causal forward with two output streams (dropout) measured 3 % faster with 2 rows
+        if constexpr (!BWD && M == Mask::Causal && (EXTRA & kDropout) != 0)
+            return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
+        return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
+    }
     if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
     if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);
     if (chunks <= 32) return launch_shape<T, M, BWD, EXTRA, 2, 16, 1>(a, st);
