@@ -356,7 +356,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         has to exist before the capture starts."""
         b, np, sq, sk = input.size()
         fusable = self.is_kernel_available(mask, b, np, sq, sk) and (alibi_slopes is None or bias is None)
-        causal = fusable and self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask)
+        causal = fusable and self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask)
         if fusable and alibi_slopes is not None and not causal:
             fusable = False  # the mask-tensor kernels have no ALiBi variant
         if not fusable:
@@ -372,15 +372,27 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         Kept from the reference predicate (megatron/model/fused_softmax.py:148-168):
         the user asked for fusion, the input is fp16/bf16, a mask tensor is given.
         Dropped: ``16 < sk <= 2048``, ``sq % 4``, ``(b*np) % 4`` and the
-        ``batch_per_block`` rules.  Added: the causal branch needs ``sq == sk`` (the
-        reference asserts it later; a decode step with ``sq == 1`` goes to the torch path
-        with the mask it was given), and the tensor must not be empty.
+        ``batch_per_block`` rules.  Added: the tensor must not be empty, and a causal-fusion call
+        with ``sq != sk`` (a decode or prefill step against a key/value cache; the reference
+        asserts ``sq == sk`` and never gets there) is served by the mask-tensor kernel with the
+        mask it was given, provided that mask has the kernel's layout ``[1 or b, 1, sq, sk]``.
         """
         if not (self.fusion and self.input_in_float16 and mask is not None):
             return False
         if b * np * sq * sk == 0:
             return False
-        return sq == sk if self.upper_triang_mask_fusion else True
+        if self.upper_triang_mask_fusion and sq != sk:
+            return self._mask_fits_the_mask_kernel(mask, b, sq, sk)
+        return True
+
+    @staticmethod
+    def _mask_fits_the_mask_kernel(mask, b, sq, sk):
+        return (
+            mask.dim() == 4
+            and mask.dtype in (torch.bool, torch.uint8)
+            and mask.shape[0] in (1, b)
+            and tuple(mask.shape[1:]) == (1, sq, sk)
+        )
 
     @staticmethod
     def reference_is_kernel_available(fusion, upper_triang, input_in_float16, mask, b, np, sq, sk):
@@ -395,11 +407,10 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     def forward_fused_softmax(self, input, mask, bias=None):
         b, np, sq, sk = input.size()
         scale = 1.0 if self.scale is None else self.scale
-        if self.upper_triang_mask_fusion:
-            assert sq == sk, "causal mask is only for self attention"
-        if not (self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask)):
-            # general fusion, or a causal-fusion call whose mask is not the plain triangle (e.g. a
-            # sliding-window mask): what the torch path computes, from the mask itself
+        if not (self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask)):
+            # general fusion, or a causal-fusion call whose mask is not the plain square triangle (a
+            # sliding-window mask, a step against a key/value cache): what the torch path computes,
+            # from the mask itself
             if bias is not None:
                 return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale)
             return ScaledMaskedSoftmax.apply(input, mask, scale)

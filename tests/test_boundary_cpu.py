@@ -218,7 +218,13 @@ def test_is_kernel_available_table():
         assert causal.is_kernel_available(mask, b, np_, sq, sk)
     assert general.is_kernel_available(mask, 8, 16, 1024, 1024)
     assert general.is_kernel_available(mask, 1, 3, 1, 77)  # decode step, odd sizes
-    assert not causal.is_kernel_available(mask, 1, 4, 1, 77)  # causal kernel needs sq == sk
+    # causal fusion with sq != sk (a step against a key/value cache): fused through the mask-tensor
+    # kernel when the mask has that kernel's layout, otherwise the torch branch
+    assert not causal.is_kernel_available(mask, 1, 4, 1, 77)
+    assert causal.is_kernel_available(torch.zeros(1, 1, 1, 77, dtype=torch.bool), 1, 4, 1, 77)
+    assert causal.is_kernel_available(torch.zeros(2, 1, 5, 77, dtype=torch.uint8), 2, 4, 5, 77)
+    assert not causal.is_kernel_available(torch.zeros(3, 1, 5, 77, dtype=torch.bool), 2, 4, 5, 77)
+    assert not causal.is_kernel_available(torch.zeros(1, 1, 5, 77), 2, 4, 5, 77)  # float mask
     assert not causal.is_kernel_available(None, 4, 12, 64, 64)  # no mask tensor
     assert not general.is_kernel_available(None, 4, 12, 64, 64)
     assert not none.is_kernel_available(mask, 4, 12, 64, 64)  # fusion not requested

@@ -397,12 +397,29 @@ def test_alibi_module_argument_and_gradient(device):
     assert max_err(yw, fused(alibi(x), window)) == 0.0
 
 
-def test_causal_decode_step_takes_the_torch_branch(device):
+def test_causal_fusion_against_a_key_value_cache(device):
+    # sq != sk: the reference's causal branch asserts; here the mask-tensor kernel serves the call
+    # with the mask it is given, and a mask of another layout still goes to the torch branch
     fused = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang,
                                   R.gpt2_attention_mask_func, True, None)
-    x = scores((1, 2, 1, 33), torch.float16, device, 4)
+    x = scores((1, 2, 1, 33), torch.float16, device, 4)  # one new token, 33 keys
     mask = torch.zeros(1, 1, 1, 33, dtype=torch.bool, device=device)
-    assert torch.equal(fused(x, mask), R.forward_torch_softmax(x, mask, None, True, False, True))
+    assert fused.is_kernel_available(mask, *x.shape)
+    assert max_err(fused(x, mask), R.softmax_fp32(x, mask, None)) <= TOL[torch.float16]
+    # prefill of 5 tokens after 28 cached ones: query i sees keys j <= 28 + i
+    x = scores((2, 3, 5, 33), torch.float16, device, 5).requires_grad_(True)
+    mask = (torch.arange(33, device=device)[None, :] > (28 + torch.arange(5, device=device))[:, None]).view(1, 1, 5, 33)
+    y = fused(x, mask)
+    ref = R.softmax_fp32(x.detach(), mask, None)
+    assert max_err(y, ref) <= TOL[torch.float16] and (y[mask.expand_as(y)] == 0).all()
+    g = normal(x.shape, torch.float16, device, 6)
+    y.backward(g.clone())
+    want = R.softmax_backward_fp32(g, y.detach(), None)
+    assert max_err(x.grad, want) <= TOL[torch.float16] * max(1.0, want.abs().max().item())
+    broadcast = torch.zeros(1, 1, 1, 1, dtype=torch.bool, device=device)  # not the kernel's layout
+    assert not fused.is_kernel_available(broadcast, 2, 3, 5, 33)
+    xd = x.detach()
+    assert torch.equal(fused(xd, broadcast), R.forward_torch_softmax(xd, broadcast, None, True, False, True))
 
 
 # ---------------------------------------------------------------------------------
