@@ -24,7 +24,8 @@ Deliberate differences from the reference:
   runs the mask-tensor kernel with the mask it was given -- the reference's causal
   kernel ignores the mask's contents, so above its 2048 limit (torch path) and below
   it (fused kernel) the reference computes two different things for such masks; here
-  both agree with the torch path;
+  both agree with the torch path; a causal-fusion call with ``sq != sk`` (a step against a
+  key/value cache, where the reference asserts) also runs the mask-tensor kernel;
 * masked scores are excluded, so their probability is exactly 0 as in the torch
   path (the reference's padded kernel fills -10000), and a fully masked row is
   uniform ``1/sk`` as in the torch path;
