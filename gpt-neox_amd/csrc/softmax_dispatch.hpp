@@ -13,6 +13,10 @@
 //   chunks <= 16   8 waves per row, 512-thread block                 (sk <= 8192)
 //   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
+//   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
+//                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
+//   anything else  element-wise kernels (sk % 8 != 0, unaligned pointers, longer rows still, and
+//                  rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
 
 #include <type_traits>
@@ -103,7 +107,26 @@ static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
 template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     const int chunks = (a.sk + kChunk - 1) / kChunk;
-    if (!vec_ok || a.sk > kMaxRegisterRow) return launch_generic<T, M, BWD, EXTRA>(a, st);
+    if (!vec_ok) return launch_generic<T, M, BWD, EXTRA>(a, st);
+    if (a.sk > kMaxRegisterRow) {
+        // beyond the register budget: the row is staged in LDS (plain kernels only), in half
+        // of a CU's LDS when it fits there
+        if constexpr (EXTRA == 0) {
+            if (a.sk <= kMaxLdsRow && a.slopes == nullptr) {
+                const bool half = a.sk <= kMaxLdsHalfRow;
+                const dim3 grid(a.rows), block(kLdsThreads);
+                if constexpr (BWD) {
+                    if (half) hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 5, kLdsHalf>), grid, block, 0, st, a);
+                    else hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 10, kLdsBytes>), grid, block, 0, st, a);
+                } else {
+                    if (half) hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsHalf>), grid, block, 0, st, a);
+                    else hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsBytes>), grid, block, 0, st, a);
+                }
+                return hipGetLastError();
+            }
+        }
+        return launch_generic<T, M, BWD, EXTRA>(a, st);
+    }
     if (chunks == 1) {
         // the forward mask kernel addresses the mask through one 32-bit-sized buffer
         // and the bias kernel the bias tensor

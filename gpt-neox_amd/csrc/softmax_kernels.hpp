@@ -17,6 +17,8 @@
 // one reciprocal per row, one rounding to the storage type on store.
 #pragma once
 
+#include <type_traits>
+
 #include "philox.hpp"
 #include "wave.hpp"
 
@@ -332,7 +334,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                     // the lane holding the diagonal may have loaded columns past it
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
-                        if ((col + k) >= len) pv[k] = 0.f;
+                        if ((col + k) >= len) gv[k] = pv[k] = 0.f;
                 }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) dot = fmaf(gv[k], pv[k], dot);
@@ -583,7 +585,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
-                if ((col0 + c * kChunk + k) >= len[p]) pv[k] = 0.f;  // past the diagonal / row end
+                if ((col0 + c * kChunk + k) >= len[p]) gv[k] = pv[k] = 0.f;  // past the diagonal / row end
                 dot = fmaf(gv[k], pv[k], dot);
             }
         }
@@ -603,6 +605,261 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             const bool st = lr < rows_here && col < sk;
             buf_st128<kStNt>(bo, pack8<T>(gv), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// LDS-staged kernels: rows beyond the register budget (sk > 32768).
+//
+// One 1024-thread block per row.  The row is read from HBM once and the later passes run
+// from LDS, where it is kept as raw 16-bit values: a gfx950 workgroup may use the whole
+// 160 KiB of its CU, which holds 81408 columns.  Rows of at most 40448 columns take half of
+// it, so that two blocks share a CU and one loads while the other stores.  The forward pass
+// stages the scores, with masked and out-of-row elements replaced by -inf, which the later
+// passes recognise and turn into exact zeros without looking at the mask again.  The
+// backward pass stages the probabilities and keeps the gradient packed in registers.  Each
+// wave stages and re-reads its own chunks only, so the only barriers are those of the
+// reductions.
+// ---------------------------------------------------------------------------------
+constexpr int kLdsWaves = 16;
+constexpr int kLdsThreads = kLdsWaves * kWave;
+constexpr int kLdsBytes = 159 * 1024;        // one block per CU; the last KiB of the CU's 160 is left to the reductions
+constexpr int kLdsHalf = 79 * 1024;          // two blocks per CU
+constexpr int kMaxLdsRow = kLdsBytes / 2;    // 81408 columns (159 chunks)
+constexpr int kMaxLdsHalfRow = kLdsHalf / 2; // 40448 columns (79 chunks)
+constexpr int kLdsUnroll = 4;                // chunks of a wave whose loads are in flight together
+
+// Waves per SIMD a kernel with a staging area of `bytes` is compiled for: the register budget
+// that lets as many blocks share a CU as its LDS allows.
+constexpr int lds_waves_per_simd(int bytes) { return (bytes <= kLdsHalf ? 2 : 1) * kLdsWaves / 4; }
+
+template <typename T>
+struct NegInf16;  // -inf of the storage type, as bits
+template <>
+struct NegInf16<F16> { static constexpr uint32_t bits = 0xFC00u; };
+template <>
+struct NegInf16<BF16> { static constexpr uint32_t bits = 0xFF80u; };
+
+// Replaces the elements whose keep bit is clear by -inf (8 packed elements, bit k = element k).
+template <typename T>
+__device__ __forceinline__ u32x4 stage_masked(const u32x4& raw, uint32_t keep) {
+    constexpr uint32_t ninf = NegInf16<T>::bits;
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t lo = ((keep >> (2 * k)) & 1u) ? (w[k] & 0xffffu) : ninf;
+        const uint32_t hi = ((keep >> (2 * k + 1)) & 1u) ? (w[k] & 0xffff0000u) : (ninf << 16);
+        o[k] = lo | hi;
+    }
+    return u32x4{o[0], o[1], o[2], o[3]};
+}
+
+// BYTES: size of the staging area, at least 2 * sk.
+template <typename T, Mask MASK, int BYTES>
+__global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softmax_fwd_lds_kernel(SoftmaxArgs a) {
+    __shared__ __align__(16) char staged[BYTES];
+    __shared__ float red_max[kLdsWaves];
+    __shared__ float red_sum[kLdsWaves];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sk = a.sk;
+    const float ninf = -__builtin_inff();
+    const RowPos pos = locate<MASK>(blockIdx.x, a);
+    const int len = pos.len;
+    const int data_chunks = (len + kChunk - 1) / kChunk;  // chunks that hold columns of the row
+    const int all_chunks = (sk + kChunk - 1) / kChunk;
+
+    const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2,
+                                (uint32_t)((len + kVec - 1) & ~(kVec - 1)) * 2u);
+    rsrc_t rm = rx;
+    if constexpr (MASK == Mask::Bytes) {
+        const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
+        rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)len);
+    }
+
+    // ---- pass 1: HBM -> LDS, running maximum of the scaled scores
+    float mx = ninf;
+    bool hidden = false;  // wave-uniform: this wave staged a -inf in place of a masked or out-of-row element
+    for (int c0 = wib; c0 < data_chunks; c0 += kLdsWaves * kLdsUnroll) {
+        u32x4 raw[kLdsUnroll];
+        u32x2 mk[kLdsUnroll];
+#pragma unroll
+        for (int u = 0; u < kLdsUnroll; ++u) {
+            const int c = c0 + u * kLdsWaves;  // wave-uniform; chunks past the data load nothing
+            raw[u] = buf_ld128<true>(rx, c * kChunk * 2 + lane * 16, 0);
+            if constexpr (MASK == Mask::Bytes) mk[u] = buf_ld64(rm, c * kChunk + lane * 8, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kLdsUnroll; ++u) {
+            const int c = c0 + u * kLdsWaves;
+            if (c < data_chunks) {
+                const int col = c * kChunk + lane * kVec;
+                float v[8];
+                unpack8<T>(raw[u], v);
+                bool plain = (c + 1) * kChunk <= len;  // no lane of the wave crosses the row end
+                if constexpr (MASK == Mask::Bytes) plain = plain && (__ballot((mk[u].x | mk[u].y) != 0u) == 0ull);
+                u32x4 keep_raw = raw[u];
+                if (plain) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) mx = fmaxf(mx, v[k] * a.scale);
+                } else {
+                    hidden = true;
+                    uint32_t keep = 0;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        bool kept = (col + k) < len;
+                        if constexpr (MASK == Mask::Bytes) {
+                            const uint32_t w = (k < 4) ? mk[u].x : mk[u].y;
+                            kept = kept && (((w >> (8 * (k & 3))) & 0xffu) == 0);
+                        }
+                        keep |= (kept ? 1u : 0u) << k;
+                        mx = fmaxf(mx, kept ? v[k] * a.scale : ninf);
+                    }
+                    keep_raw = stage_masked<T>(raw[u], keep);
+                }
+                *reinterpret_cast<u32x4*>(staged + c * kChunk * 2 + lane * 16) = keep_raw;
+            }
+        }
+    }
+    mx = wave_reduce<OpMax>(mx);
+    if (lane == 0) red_max[wib] = mx;
+    __syncthreads();
+    mx = red_max[0];
+#pragma unroll
+    for (int w = 1; w < kLdsWaves; ++w) mx = fmaxf(mx, red_max[w]);
+    // a row whose every key is masked: uniform over the sk columns, as the unfused path gives
+    const bool all_masked = (MASK == Mask::Bytes) && (mx == ninf);
+
+    // ---- pass 2: sum of the exponentials, from LDS.  Only a wave that staged a -inf looks for them.
+    float sum = 0.f;
+    auto add_chunks = [&](auto with_hidden) {
+        for (int c = wib; c < data_chunks; c += kLdsWaves) {
+            float v[8];
+            unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), v);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float e = fast_exp2(v[k] * a.scale - mx);
+                sum += (decltype(with_hidden)::value && v[k] == ninf) ? 0.f : e;
+            }
+        }
+    };
+    if (hidden) add_chunks(std::true_type{});
+    else add_chunks(std::false_type{});
+    sum = wave_reduce<OpSum>(sum);
+    if (lane == 0) red_sum[wib] = sum;
+    __syncthreads();
+    sum = red_sum[0];
+#pragma unroll
+    for (int w = 1; w < kLdsWaves; ++w) sum += red_sum[w];
+    const float inv = all_masked ? 1.0f / (float)len : 1.0f / sum;
+
+    // ---- pass 3: normalise and store; chunks above the diagonal store zeros
+    const rsrc_t ry = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, (uint32_t)sk * 2u);
+    auto store_chunks = [&](auto with_hidden) {
+        for (int c = wib; c < all_chunks; c += kLdsWaves) {
+            u32x4 o = u32x4{0, 0, 0, 0};
+            if (c < data_chunks) {
+                float v[8];
+                unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), v);
+                const int col = c * kChunk + lane * kVec;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const float e = fast_exp2(v[k] * a.scale - mx) * inv;
+                    if constexpr (decltype(with_hidden)::value) {
+                        v[k] = (v[k] == ninf) ? 0.f : e;
+                        if (all_masked) v[k] = ((col + k) < len) ? inv : 0.f;
+                    } else {
+                        v[k] = e;
+                    }
+                }
+                o = pack8<T>(v);
+            }
+            buf_st128<true>(ry, o, c * kChunk * 2 + lane * 16, 0);
+        }
+    };
+    if (hidden) store_chunks(std::true_type{});
+    else store_chunks(std::false_type{});
+}
+
+// NCH: chunks per wave, kLdsWaves * NCH * 512 >= sk; BYTES: size of the staging area, >= 2 * sk.
+template <typename T, Mask MASK, int NCH, int BYTES>
+__global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softmax_bwd_lds_kernel(SoftmaxArgs a) {
+    static_assert(NCH * kLdsWaves * kChunk * 2 >= BYTES, "the waves' chunks must cover the staging area");
+    __shared__ __align__(16) char staged[BYTES];  // the probabilities of the row
+    __shared__ float red_sum[kLdsWaves];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sk = a.sk;
+    const RowPos pos = locate<MASK>(blockIdx.x, a);
+    const int len = pos.len;
+    const int data_chunks = (len + kChunk - 1) / kChunk;
+    const uint32_t bytes = (uint32_t)((len + kVec - 1) & ~(kVec - 1)) * 2u;
+    const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2, bytes);
+    const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
+
+    // ---- pass 1: the gradient into registers (chunk wib + 16 u; chunks past the data load
+    // nothing), the probabilities into LDS, their dot product on the way
+    u32x4 rg[NCH];
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) rg[u] = buf_ld128<true>(bg, (wib + u * kLdsWaves) * kChunk * 2 + lane * 16, 0);
+    float dot = 0.f;
+#pragma unroll
+    for (int u0 = 0; u0 < NCH; u0 += kLdsUnroll) {
+        u32x4 rp[kLdsUnroll];
+#pragma unroll
+        for (int u = 0; u < kLdsUnroll; ++u)
+            if (u0 + u < NCH) rp[u] = buf_ld128<true>(by, (wib + (u0 + u) * kLdsWaves) * kChunk * 2 + lane * 16, 0);
+#pragma unroll
+        for (int u = 0; u < kLdsUnroll; ++u) {
+            if (u0 + u >= NCH) continue;
+            const int c = wib + (u0 + u) * kLdsWaves;
+            if (c < data_chunks) {
+                const int col = c * kChunk + lane * kVec;
+                float gv[8], pv[8];
+                unpack8<T>(rg[u0 + u], gv);
+                unpack8<T>(rp[u], pv);
+                u32x4 keep = rp[u];
+                if ((c + 1) * kChunk > len) {
+                    // the lane at the diagonal may have loaded columns past it
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        if ((col + k) >= len) gv[k] = pv[k] = 0.f;
+                    keep = pack8<T>(pv);
+                    rg[u0 + u] = pack8<T>(gv);
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) dot = fmaf(gv[k], pv[k], dot);
+                *reinterpret_cast<u32x4*>(staged + c * kChunk * 2 + lane * 16) = keep;
+            }
+        }
+        // the loads of the next group are not to be moved up here: they would not fit the registers
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    dot = wave_reduce<OpSum>(dot);
+    if (lane == 0) red_sum[wib] = dot;
+    __syncthreads();
+    dot = red_sum[0];
+#pragma unroll
+    for (int w = 1; w < kLdsWaves; ++w) dot += red_sum[w];
+
+    // ---- pass 2: dx.  It may alias dy: a wave has read its chunks of the row before it writes them
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) forget_origin(rg[u]);  // the gradient stays packed in between
+    const rsrc_t rdx = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, (uint32_t)sk * 2u);
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+        const int c = wib + u * kLdsWaves;
+        u32x4 o = u32x4{0, 0, 0, 0};
+        if (c < data_chunks) {
+            float gv[8], pv[8];
+            unpack8<T>(rg[u], gv);
+            unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), pv);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) gv[k] = a.scale * (pv[k] * (gv[k] - dot));  // pv = 0 past the row
+            o = pack8<T>(gv);
+        }
+        buf_st128<true>(rdx, o, c * kChunk * 2 + lane * 16, 0);  // chunks past the row end store nothing
     }
 }
 

@@ -87,6 +87,12 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
 
 // Streaming 128-bit access: every byte of these kernels is touched exactly once,
 // so the loads/stores carry the non-temporal hint and do not displace each other in L2.
+// The compiler learns nothing about `w` across this point: values it derived from `w` earlier
+// (an unpacked copy, say) are computed again afterwards rather than kept in registers.
+__device__ __forceinline__ void forget_origin(u32x4& w) {
+    asm volatile("" : "+v"(w.x), "+v"(w.y), "+v"(w.z), "+v"(w.w));
+}
+
 __device__ __forceinline__ u32x4 ld128(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }

@@ -173,10 +173,10 @@ def test_causal_sizes(device, s, dtype):
     check_causal(device, batches, s, dtype, 0.125, seed=s)
 
 
-@pytest.mark.parametrize("s", [12288, 16384, 20000, 28672, 33000])
+@pytest.mark.parametrize("s", [12288, 16384, 20000, 28672, 33000, 40448, 40456, 40968])
 def test_causal_very_long_rows(device, s):
-    # 16 waves per row with 2, 3 and 4 chunks per wave; 33000 exceeds the register-resident
-    # limit (element-wise kernels)
+    # 16 waves per row with 2, 3 and 4 chunks per wave; from 33000 on the row exceeds the register
+    # budget and is staged in LDS: in half of a CU's LDS up to 40448 columns, in all of it beyond
     x = scores((1, s, s), torch.bfloat16, device, s)
     y = causal_ext.forward(x, 0.05)
     rows = torch.tensor([0, 1, 511, 512, 513, s // 2, s - 2, s - 1], device=device)
@@ -190,6 +190,27 @@ def test_causal_very_long_rows(device, s):
     refb = R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)
     assert max_err(dx[0][rows], refb) <= TOL[torch.bfloat16]
     assert (dx[0][rows][mask] == 0).all()
+
+
+@pytest.mark.parametrize("s", [8, 24, 200, 512, 1000, 1536, 2048, 3000, 4104, 9000, 20000, 33000, 41000])
+def test_causal_kernels_ignore_what_lies_past_the_diagonal(device, s):
+    # The reference reads scores, gradient and probabilities up to the diagonal only
+    # (scaled_upper_triang_masked_softmax.h:180-196 and 304-325): NaN and Inf above it, also in
+    # the columns that share a 128-bit access with the diagonal, change nothing.
+    batches = 2 if s <= 4104 else 1
+    upper = torch.ones(s, s, dtype=torch.bool, device=device).triu_(1)
+    for dtype in (DTYPES if s <= 4104 else [torch.bfloat16]):
+        x = scores((batches, s, s), dtype, device, s)
+        g = normal((batches, s, s), dtype, device, s + 1)
+        y = causal_ext.forward(x, 0.125)
+        dx = causal_ext.backward(g.clone(), y, 0.125)
+        y_poisoned = causal_ext.forward(x.masked_fill(upper, float("nan")), 0.125)
+        assert torch.equal(y_poisoned, y)
+        y_poisoned = causal_ext.forward(x.masked_fill(upper, float("inf")), 0.125)
+        assert torch.equal(y_poisoned, y)
+        for poison_g, poison_y in ((float("nan"), float("nan")), (float("inf"), 0.0), (1.0, float("-inf"))):
+            got = causal_ext.backward(g.masked_fill(upper, poison_g), y.masked_fill(upper, poison_y), 0.125)
+            assert torch.equal(got, dx), (s, dtype, poison_g, poison_y)
 
 
 @pytest.mark.parametrize("s", [520, 1032, 2056, 4104, 8200])
@@ -447,7 +468,8 @@ def check_masked(device, b, heads, sq, sk, dtype, scale, seed, mask=None, lo=1):
 MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (3, 5, 7, 8), (2, 3, 5, 16), (2, 2, 33, 24), (2, 2, 16, 64),
                  (3, 3, 50, 72), (2, 2, 31, 128), (2, 3, 17, 200), (2, 2, 65, 256), (1, 3, 129, 384), (2, 2, 9, 512), (3, 2, 9, 520),
                  (2, 2, 33, 1000), (2, 2, 8, 1024), (1, 2, 6, 2048), (1, 1, 4, 3072), (1, 2, 3, 4096),
-                 (1, 1, 3, 8192), (1, 1, 2, 12000), (1, 1, 2, 20000), (1, 1, 2, 30000), (1, 1, 2, 40000), (1, 3, 1, 77)]
+                 (1, 1, 3, 8192), (1, 1, 2, 12000), (1, 1, 2, 20000), (1, 1, 2, 30000), (1, 1, 2, 40000), (1, 3, 1, 77),
+                 (2, 2, 3, 32776), (1, 2, 2, 65536), (1, 1, 3, 81408), (1, 1, 2, 81416)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -966,3 +988,33 @@ def test_seeded_random_rotary_layouts(device):
         else:
             oq, ok = apply_rotary_pos_emb(q[..., :d_rot], k[..., :d_rot], cos, sin, offset=offset)
             assert torch.equal(oq, want_q.to(dtype)) and torch.equal(ok, want_k.to(dtype)), tag
+
+
+# ---------------------------------------------------------------------------------
+# rows beyond the register budget: staged in LDS
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("scale", [0.5, -0.25])
+@pytest.mark.parametrize("sk", [33280, 50008])  # staged in half of a CU's LDS / in all of it
+def test_lds_staged_rows_masks_scales_and_aliasing(device, dtype, scale, sk):
+    b, heads, sq = 2, 2, 3
+    x = scores((b, heads, sq, sk), dtype, device, 91)
+    g = normal((b, heads, sq, sk), dtype, device, 92)
+    mask = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, 93)) < 0.3  # arbitrary pattern
+    mask[0, 0, 1, :] = True        # a row with every key hidden: uniform 1/sk
+    mask[1, 0, 2, 100:] = True     # a row that ends early
+    y = masked_ext.forward(x, mask, scale)
+    ref = R.softmax_fp32(x, mask, scale)
+    assert max_err(y, ref) <= TOL[dtype]
+    hidden = mask.expand_as(y).clone()
+    hidden[0, :, 1, :] = False
+    assert (y[hidden] == 0).all()
+    assert torch.allclose(y[0, :, 1, :].float(), torch.full((heads, sk), 1.0 / sk, device=device), rtol=1e-2)
+    dx = masked_ext.backward(g.clone(), y, scale)
+    refb = R.softmax_backward_fp32(g, y, scale)
+    assert max_err(dx, refb) <= TOL[dtype] * max(1.0, refb.abs().max().item())
+    buf = g.clone()  # in place on the gradient buffer
+    assert masked_ext.backward(buf, y, scale).data_ptr() == buf.data_ptr() and torch.equal(buf, dx)
+    # the mask shared by all samples
+    y1 = masked_ext.forward(x, mask[:1], scale)
+    assert max_err(y1, R.softmax_fp32(x, mask[:1], scale)) <= TOL[dtype]
