@@ -15,10 +15,13 @@ steps between device synchronisations; the JSON line carries
                  events on the launch stream, against the 8 TB/s HBM peak;
 * cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
                  this host's cores on a slice of the same batch;
-* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak, the error
-                 of the kernel's output on a slice against the oracle (max |err|, non-zero
-                 masked outputs; bit-equality for rotary) and the oracle's CPU time on a
-                 slice scaled to the full shape.
+* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak and, as part
+                 of the CPU-baseline leg, the oracle's CPU time on a slice scaled to the full
+                 shape with the error of the kernel's output on that slice against it (max
+                 |err|, non-zero masked outputs; bit-equality for rotary).
+
+The oracle is imported by the CPU-baseline leg only (--no-cpu runs never load it); the inputs
+of the measured launches are built without it.
 
 Buffers rotate over several distinct sets so that no launch finds its input in
 the 256 MB Infinity Cache left there by the previous one.
@@ -47,7 +50,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true",
+                    help="skip the CPU-baseline leg: the oracle's timings and its checks of the kernels' outputs")
     ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
     ap.add_argument("--quick", action="store_true",
                     help="few launches per table row (for counter-collection runs)")
@@ -68,9 +72,11 @@ def main():
 
     from gpt_neox_amd import _lib
     from gpt_neox_amd.positional_embeddings import RotaryEmbedding
-    # The oracle is used as the checker of the kernels' outputs and as the timed CPU baseline
-    # only; the inputs of the measured launches are built below without it.
-    from oracle import torch_ref as R
+    # The CPU-baseline leg alone uses the oracle: as the timed baseline and as the checker of
+    # the kernels' outputs on the baseline's samples.
+    R = None
+    if not args.no_cpu:
+        from oracle import torch_ref as R
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -171,6 +177,9 @@ def main():
             torch.cuda.synchronize()
             means.append(e0.elapsed_time(e1) * 1e3 / n_launch)
         return statistics.median(means), min(means)
+
+    def causal_mask(n):
+        return torch.ones(n, n, dtype=torch.bool, device=dev).triu_(1).view(1, 1, n, n)
 
     def row(name, nbytes, med_us, min_us):
         gbps = nbytes / med_us / 1e3
@@ -297,9 +306,11 @@ def main():
         return (time.perf_counter() - t0) / reps * 1e6
 
     def softmax_extras(r, x, y, mask, sc, dt, total, dy=None, dx=None):
-        """Parity of the kernels' own output on a slice (against the oracle evaluated on the
-        GPU in fp32) and the oracle's CPU time on the same slice scaled to the full batch.
-        x, y (, dy, dx): [k, sq, sk] or [k, np, sq, sk] slices; mask broadcastable to them."""
+        """CPU-baseline leg of a table row: the oracle's CPU time on a slice scaled to the full
+        batch, and the kernels' own output on that slice against the oracle (evaluated on the GPU
+        in fp32).  x, y (, dy, dx): [k, sq, sk] or [k, np, sq, sk] slices; mask broadcastable."""
+        if R is None:
+            return r
         k = x.shape[0]
         x4 = x if x.dim() == 4 else x.unsqueeze(1)
         y4 = y if y.dim() == 4 else y.unsqueeze(1)
@@ -312,23 +323,25 @@ def main():
             dx4 = dx if dx.dim() == 4 else dx.unsqueeze(1)
             r["max_abs_err"] = float((dx4.float() - R.softmax_backward_fp32(dy4, y4, sc)).abs().max())
             r["masked_nonzero"] = int((dx4[mask.expand_as(dx4)] != 0).sum())
-        if not args.no_cpu:
-            xc, mc = x4.cpu(), mask.cpu()
-            f16 = dt == torch.float16
-            if dx is None:
-                us = cpu_time_us(lambda: R.forward_torch_softmax(xc, mc, sc, f16, not f16, True))
-            else:
-                gc = dy4.cpu()
-                xin = xc.clone().requires_grad_(True)
-                yc = R.forward_torch_softmax(xin, mc, sc, f16, not f16, True)
-                us = cpu_time_us(lambda: torch.autograd.grad(yc, xin, gc, retain_graph=True))
-            r["cpu_us_per_call"] = round(us * total / k, 1)
-            r["cpu_sample"] = f"{k} of {total} along dim 0, {torch.get_num_threads()} threads, scaled"
+        xc, mc = x4.cpu(), mask.cpu()
+        f16 = dt == torch.float16
+        if dx is None:
+            us = cpu_time_us(lambda: R.forward_torch_softmax(xc, mc, sc, f16, not f16, True))
+        else:
+            gc = dy4.cpu()
+            xin = xc.clone().requires_grad_(True)
+            yc = R.forward_torch_softmax(xin, mc, sc, f16, not f16, True)
+            us = cpu_time_us(lambda: torch.autograd.grad(yc, xin, gc, retain_graph=True))
+        r["cpu_us_per_call"] = round(us * total / k, 1)
+        r["cpu_sample"] = f"{k} of {total} along dim 0, {torch.get_num_threads()} threads, scaled"
         return r
 
     def rope_extras(r, S, Bb, H, HN, DR, backward):
-        """Fresh tensors of the full shape: bit-equality with the fp32 expression rounded once
-        (all positions), CPU time of the torch expression on 256 positions scaled."""
+        """CPU-baseline leg of a rotary row.  Fresh tensors of the full shape: bit-equality with
+        the oracle's fp32 expression rounded once (all positions), CPU time of the oracle's torch
+        expression on 256 positions scaled."""
+        if R is None:
+            return r
         g0 = gen(4321)
         q = torch.randn(S, Bb, H, HN, device=dev, generator=g0).bfloat16()
         k = torch.randn(S, Bb, H, HN, device=dev, generator=g0).bfloat16()
@@ -343,16 +356,15 @@ def main():
         r["bit_equal_to_fp32_rounded_once"] = bool(
             torch.equal(t["q"][..., :DR], rq.bfloat16()) and torch.equal(t["k"][..., :DR], rk.bfloat16())
             and torch.equal(t["q"][..., DR:], q[..., DR:]))
-        if not args.no_cpu:
-            n = 256
-            qc, kc = q[:n, ..., :DR].cpu(), k[:n, ..., :DR].cpu()
-            cc, sc_ = cos4[:n].cpu(), sin4[:n].cpu()
-            if backward:
-                us = cpu_time_us(lambda: R.rotary_autograd_fp32(qc, kc, cc, sc_, qc, kc))
-            else:
-                us = cpu_time_us(lambda: R.apply_rotary_pos_emb(qc, kc, cc, sc_))
-            r["cpu_us_per_call"] = round(us * S / n, 1)
-            r["cpu_sample"] = f"{n} of {S} positions, {torch.get_num_threads()} threads, scaled"
+        n = 256
+        qc, kc = q[:n, ..., :DR].cpu(), k[:n, ..., :DR].cpu()
+        cc, sc_ = cos4[:n].cpu(), sin4[:n].cpu()
+        if backward:
+            us = cpu_time_us(lambda: R.rotary_autograd_fp32(qc, kc, cc, sc_, qc, kc))
+        else:
+            us = cpu_time_us(lambda: R.apply_rotary_pos_emb(qc, kc, cc, sc_))
+        r["cpu_us_per_call"] = round(us * S / n, 1)
+        r["cpu_sample"] = f"{n} of {S} positions, {torch.get_num_threads()} threads, scaled"
         return r
 
     if not args.no_table:
@@ -370,7 +382,7 @@ def main():
             s_ = causal_sets(B, n, dt, 1234, nsets=2, need_bwd=False)
             r = row("cfg1 causal fwd [48,2048,2048] bf16", B * 2 * (tri(n) + n * n),
                     *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100))
-            table.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], R.get_attn_mask(n, dev), sc, dt, B))
+            table.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
             del s_
         # configs[1]
         if want("cfg2"):
@@ -400,7 +412,7 @@ def main():
         if want("cfg4"):
             B, n, dt, sc = 64, 2048, torch.float16, 96 ** -0.5
             s_ = causal_sets(B, n, dt, 1237, nsets=2, need_bwd=True)
-            cm = R.get_attn_mask(n, dev)
+            cm = causal_mask(n)
             r = row("cfg4 causal fwd [64,2048,2048] fp16", B * 2 * (tri(n) + n * n),
                     *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 100))
             z = s_[0]
@@ -414,7 +426,7 @@ def main():
             torch.cuda.empty_cache()
             B, n, dt, sc = 32, 8192, torch.bfloat16, 128 ** -0.5
             s_ = causal_sets(B, n, dt, 1238, nsets=1, need_bwd=True)
-            cm = R.get_attn_mask(n, dev)
+            cm = causal_mask(n)
             r = row("cfg5 causal fwd [32,8192,8192] bf16", B * 2 * (tri(n) + n * n),
                     *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, 30, warm=5))
             z = s_[0]
@@ -467,7 +479,9 @@ def main():
             def drop_extras(r, z, k, mask, sc, fwd):
                 """Slice [:k] along dim 0: the dropped output against torch's dropout expression
                 on the kernel's own probabilities and keep pattern (bit-equality), or the
-                backward against the fp32 closed form."""
+                backward against the fp32 closed form (oracle; CPU-baseline leg only)."""
+                if R is None:
+                    return r
                 y = z["y"][:k]
                 keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
                 if fwd:
@@ -507,7 +521,7 @@ def main():
                 s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
                 for z in s_:
                     z["y2"] = torch.empty_like(z["x"])
-                cm = R.get_attn_mask(n, dev)[0]
+                cm = causal_mask(n)[0]
 
                 def cd_fwd(t):
                     ok(lib.neox_causal_softmax_dropout_fwd(
@@ -542,10 +556,11 @@ def main():
             r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
                     Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
             z = s_[0]
-            cm = R.get_attn_mask(n, dev)
-            ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
-            r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
-            r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
+            if R is not None:
+                cm = causal_mask(n)
+                ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
+                r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
+                r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
             result["fused_bias"] = [r]
             del s_, z, rpe
         # what the memory pattern of the partial rotary costs by itself: the first 64 of every 256

@@ -96,13 +96,19 @@ class _CausalMaskMemo:
         self._entries = {}
         self._limit = limit
 
-    def is_plain_causal(self, mask):
-        key = id(mask)
-        hit = self._entries.get(key)
+    def lookup(self, mask):
+        """The remembered verdict for this tensor in its current version, or None."""
+        hit = self._entries.get(id(mask))
         if hit is not None:
             ref, version, verdict = hit
             if ref() is mask and version == mask._version:
                 return verdict
+        return None
+
+    def is_plain_causal(self, mask):
+        verdict = self.lookup(mask)
+        if verdict is not None:
+            return verdict
         sq, sk = mask.shape[-2], mask.shape[-1]
         cols = torch.arange(sk, device=mask.device)
         rows = torch.arange(sq, device=mask.device)
@@ -113,7 +119,7 @@ class _CausalMaskMemo:
             self._entries = {k: v for k, v in self._entries.items() if v[0]() is not None}
             if len(self._entries) >= self._limit:
                 self._entries.clear()
-        self._entries[key] = (weakref.ref(mask), mask._version, verdict)
+        self._entries[id(mask)] = (weakref.ref(mask), mask._version, verdict)
         return verdict
 
 
@@ -424,12 +430,13 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     @staticmethod
     def mask_is_plain_causal(mask):
         """True if ``mask`` hides exactly the keys ``j > i``.  Decided once per mask tensor
-        (see ``_CausalMaskMemo``); while a HIP graph is being captured the check cannot
-        synchronise, so the answer is False and the mask-tensor kernel is used."""
+        (see ``_CausalMaskMemo``).  While a HIP graph is being captured the check cannot
+        synchronise: a mask decided before the capture keeps its verdict, for any other the
+        answer is False and the mask-tensor kernel is used."""
         if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
             return False
         if mask.is_cuda and torch.cuda.is_current_stream_capturing():
-            return False
+            return bool(_causal_memo.lookup(mask))
         return _causal_memo.is_plain_causal(mask)
 
     def forward_torch_softmax(self, input, mask):

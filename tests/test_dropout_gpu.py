@@ -435,8 +435,13 @@ def test_fused_dropout_in_a_hip_graph_draws_a_fresh_pattern_per_replay(device):
         step()  # eager warm-up on the capture stream: takes the host generator, not the device state
         side.synchronize()
         assert live.tolist() == first
+        fresh_mask = causal.clone()
         with torch.cuda.graph(graph, stream=side):
             step()
+            # a mask decided before the capture keeps its verdict; one first seen inside it cannot
+            # be examined (that would synchronise) and goes to the mask-tensor kernel
+            verdicts = (mc.mask_is_plain_causal(causal), mc.mask_is_plain_causal(fresh_mask))
+    assert verdicts == (True, False)
     assert live.tolist() == first  # capturing executes nothing
 
     seen = []
