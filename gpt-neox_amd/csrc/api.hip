@@ -172,8 +172,12 @@ struct SoftmaxCall {
         a.in1 = y;
         a.scale = scale;
     }
-    int launch(Launcher fn, Mask m, void* stream) const {
-        return check_launch(fn(a, m, dtype, vec_ok && a.sk % kVec == 0, (hipStream_t)stream), what);
+    // `ragged`, if given, serves rows that rule out aligned 128-bit accesses; without it (or
+    // outside its range of row lengths) those go to `fn`'s element-wise kernels.
+    int launch(Launcher fn, Mask m, void* stream, Launcher ragged = nullptr) const {
+        const bool vec = vec_ok && a.sk % kVec == 0;
+        if (!vec && ragged != nullptr && a.sk >= kVec && a.sk <= kMaxRegisterRow) fn = ragged;
+        return check_launch(fn(a, m, dtype, vec, (hipStream_t)stream), what);
     }
 
   private:
@@ -266,7 +270,7 @@ int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches
     c.causal_rows(batches, sq, sk);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
 }
 
 int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, float scale, int32_t b,
@@ -276,7 +280,7 @@ int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, f
     c.alibi(slopes, np);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
 }
 
 int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
@@ -285,7 +289,7 @@ int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     c.causal_rows(batches, sq, sk);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_bwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_bwd, Mask::Causal, stream, launch_softmax_ragged_bwd);
 }
 
 int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
@@ -296,7 +300,7 @@ int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float s
     c.mask(mask, b, np, mask_b);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Bytes, stream);
+    return c.launch(launch_softmax_fwd, Mask::Bytes, stream, launch_softmax_ragged_fwd);
 }
 
 int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows,
@@ -305,7 +309,7 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     c.plain_rows(rows, sk);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_bwd, Mask::None, stream);
+    return c.launch(launch_softmax_bwd, Mask::None, stream, launch_softmax_ragged_bwd);
 }
 
 int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
@@ -316,7 +320,7 @@ int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float
     c.bias(bias, b, np, bias_b);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_bias_fwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_bias_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
 }
 
 int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
@@ -329,7 +333,7 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
     c.bias(bias, b, np, bias_b);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_bias_fwd, Mask::Bytes, stream);
+    return c.launch(launch_softmax_bias_fwd, Mask::Bytes, stream, launch_softmax_ragged_fwd);
 }
 
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const float* alibi_slopes,

@@ -14,7 +14,8 @@ namespace neox {
 int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
 // Launchers: pick the kernel shape for the row length and launch on `stream`.
-// `vec_ok` says that 128-bit accesses are legal (sk % 8 == 0, pointers 16-byte aligned).
+// `vec_ok` says that every row starts on a 16-byte boundary (sk % 8 == 0, pointers 16-byte
+// aligned); without it these launchers use their element-wise kernels.
 hipError_t launch_softmax_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                               hipStream_t stream);
 hipError_t launch_softmax_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
@@ -27,6 +28,12 @@ hipError_t launch_softmax_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype
 // Forward with an additive bias tensor (a.bias, a.bias_rows, a.bias_bytes).
 hipError_t launch_softmax_bias_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                    hipStream_t stream);
+// Rows at any 2-byte alignment with 8 <= sk <= kMaxRegisterRow (a.bias optional in the forward
+// pass, no dropout); `vec_ok` is ignored.
+hipError_t launch_softmax_ragged_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                     hipStream_t stream);
+hipError_t launch_softmax_ragged_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                     hipStream_t stream);
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream);
 

@@ -15,8 +15,11 @@
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
-//   anything else  element-wise kernels (sk % 8 != 0, unaligned pointers, longer rows still, and
-//                  rows beyond 32768 columns with ALiBi, bias or dropout)
+//   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768, no dropout)
+//                  the same one- to sixteen-wave row kernels with the kRagged flag; rows up to
+//                  512 columns get one wave each
+//   anything else  element-wise kernels (ragged rows with dropout or outside that range, rows
+//                  beyond 81408 columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
 
 #include <type_traits>
@@ -26,15 +29,15 @@
 namespace neox {
 
 // Forward features selected at run time on top of a translation unit's EXTRA flags: the
-// ALiBi slopes (causal kernels) and, in the dropout unit, a bias tensor.  `launch` is called
-// with the resulting flag set as a compile-time constant.
+// ALiBi slopes (causal kernels) and, in the dropout and ragged units, a bias tensor.  `launch`
+// is called with the resulting flag set as a compile-time constant.
 template <Mask M, bool BWD, int EXTRA, typename Launch>
 static hipError_t with_runtime_flags(const SoftmaxArgs& a, Launch&& launch) {
     if constexpr (!BWD && (EXTRA & kBias) == 0) {
         if constexpr (M == Mask::Causal) {
             if (a.slopes != nullptr) return launch(std::integral_constant<int, EXTRA | kAlibi>{});
         }
-        if constexpr ((EXTRA & kDropout) != 0) {
+        if constexpr ((EXTRA & (kDropout | kRagged)) != 0) {
             if (a.bias != nullptr) return launch(std::integral_constant<int, EXTRA | kBias>{});
         }
     }
@@ -104,9 +107,10 @@ static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
     return launch_packed<T, M, BWD, EXTRA, 64>(a, st);
 }
 
+// The shapes that need 16-byte aligned rows: element-wise kernels when they are not, LDS-staged
+// and packed kernels.  hipErrorNotReady: none of them applies, the row kernels take the call.
 template <typename T, Mask M, bool BWD, int EXTRA>
-static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
-    const int chunks = (a.sk + kChunk - 1) / kChunk;
+static hipError_t dispatch_aligned(const SoftmaxArgs& a, bool vec_ok, int chunks, hipStream_t st) {
     if (!vec_ok) return launch_generic<T, M, BWD, EXTRA>(a, st);
     if (a.sk > kMaxRegisterRow) {
         // beyond the register budget: the row is staged in LDS (plain kernels only), in half
@@ -140,6 +144,20 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if (chunks == 2) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
         if (chunks == 3) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
         if (chunks == 4) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 4>(a, st);
+    }
+    return hipErrorNotReady;
+}
+
+template <typename T, Mask M, bool BWD, int EXTRA>
+static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
+    const int chunks = (a.sk + kChunk - 1) / kChunk;
+    if constexpr ((EXTRA & kRagged) != 0) {
+        // rows at any alignment: the row kernels below, one wave per row up to 512 columns
+        if (a.sk < kVec || a.sk > kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+        if (chunks == 1) return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
+    } else {
+        const hipError_t e = dispatch_aligned<T, M, BWD, EXTRA>(a, vec_ok, chunks, st);
+        if (e != hipErrorNotReady) return e;
     }
     if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
     if (chunks == 3) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);

@@ -59,7 +59,53 @@ constexpr int kDropout = 8;
 // Forward adds a bias tensor to the scores before the scale: softmax(scale * (x + bias)), the sum
 // taken in fp32 (the unfused path rounds x + bias to half precision first).
 constexpr int kBias = 16;
+// Ragged rows: the tensors start at any 2-byte boundary and sk is any number >= 8, so a row
+// starts wherever the previous one ends.  128-bit buffer accesses work at any alignment on
+// gfx950 and their range check acts per dword: against a buffer of exactly the row's bytes,
+// every dword inside the row is transferred and only a dword that crosses the row end is
+// dropped.  For 16-bit data that is the last element of an odd-length row, which these kernels
+// move by a 16-bit access of its own; for the mask bytes it is the last len % 4 bytes, fetched
+// again by a dword load that ends with the row.  (Row kernels only; not with kDropout, whose
+// groups of 8 elements would straddle rows.)
+constexpr int kRagged = 32;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
+constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;  // a byte offset no buffer contains
+
+// kRagged: the element at column len - 1 of an odd-length row, fetched by every lane of the
+// wave in one broadcast access (no access when len is even).
+__device__ __forceinline__ uint32_t ragged_tail16(rsrc_t r, int len) {
+    return buf_ld16(r, (len & 1) ? (uint32_t)(len - 1) * 2u : kOutOfRange);
+}
+// kRagged: the lane whose 8 columns (from `col`) hold column len - 1 of an odd-length row puts
+// `tail` where the range check left a zero dword.
+__device__ __forceinline__ void ragged_patch16(u32x4& raw, int col, int len, uint32_t tail) {
+    const int e = len - 1 - col;  // even: len is odd, col a multiple of 8
+    if ((len & 1) && e >= 0 && e < 8) {
+        raw.x = (e == 0) ? tail : raw.x;
+        raw.y = (e == 2) ? tail : raw.y;
+        raw.z = (e == 4) ? tail : raw.z;
+        raw.w = (e == 6) ? tail : raw.w;
+    }
+}
+// kRagged: the last len % 4 mask bytes of a row (len >= 4), in the low bytes of the result.
+__device__ __forceinline__ uint32_t ragged_tail_mask(rsrc_t rm, int len) {
+    const uint32_t last4 = buf_ld32(rm, (len & 3) ? (uint32_t)(len - 4) : kOutOfRange);
+    return (len & 3) ? last4 >> (8 * (4 - (len & 3))) : 0u;
+}
+__device__ __forceinline__ void ragged_patch_mask(u32x2& mk, int col, int len, uint32_t tail) {
+    const int e = (len & ~3) - col;  // first dropped byte, relative to the lane's 8 bytes
+    if ((len & 3) && e >= 0 && e < 8) {
+        mk.x = (e == 0) ? tail : mk.x;
+        mk.y = (e == 4) ? tail : mk.y;
+    }
+}
+// kRagged: 16-bit store of element sk - 1 of an odd-length row from the packed vector that holds it.
+__device__ __forceinline__ void ragged_store16(rsrc_t r, const u32x4& o, int col, int sk) {
+    const int e = sk - 1 - col;
+    const bool own = (sk & 1) && e >= 0 && e < 8;
+    const uint32_t v = (e == 0) ? o.x : (e == 2) ? o.y : (e == 4) ? o.z : o.w;
+    buf_st16(r, v, own ? (uint32_t)(sk - 1) * 2u : kOutOfRange);
+}
 
 // Row of the bias tensor that belongs to score row `row`
 __device__ __forceinline__ uint32_t bias_row(uint32_t row, const SoftmaxArgs& a) {
@@ -122,6 +168,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     __shared__ float red_max[WPR * RPB];
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    constexpr bool kRag = (FLAGS & kRagged) != 0;
+    static_assert(!(kRag && (FLAGS & kDropout) != 0), "no dropout on ragged rows");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave in block
@@ -142,23 +190,28 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     u32x4 raw[NCH];
     u32x4 rawb[NCH];  // kBias
     u32x2 mk[NCH];
+    uint32_t tail_x = 0, tail_b = 0, tail_m = 0;  // kRagged: what the range check drops at the row end
     {
         // ---- issue every load of the row before the first use
         const char* x = static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2;
-        const uint32_t row_bytes = (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
+        // whole 128-bit accesses up to the valid length; a ragged row ends where the next one begins
+        const uint32_t row_bytes = (uint32_t)(kRag ? pos.len : (pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
         const rsrc_t rx = make_rsrc(x, row_bytes);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) raw[c] = buf_ld128<kLdNt>(rx, voff + c * WPR * kChunk * 2, 0);
+        if constexpr (kRag) tail_x = ragged_tail16(rx, pos.len);
         if constexpr ((FLAGS & kBias) != 0) {
             const rsrc_t rb = make_rsrc(static_cast<const char*>(a.bias) + (size_t)bias_row(pos.row, a) * sk * 2, row_bytes);
 #pragma unroll
             for (int c = 0; c < NCH; ++c) rawb[c] = buf_ld128<false>(rb, voff + c * WPR * kChunk * 2, 0);
+            if constexpr (kRag) tail_b = ragged_tail16(rb, pos.len);
         }
         if constexpr (MASK == Mask::Bytes) {
             const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
             const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)pos.len);
 #pragma unroll
             for (int c = 0; c < NCH; ++c) mk[c] = buf_ld64(rm, lane * 8 + (wir + c * WPR) * kChunk, 0);
+            if constexpr (kRag) tail_m = ragged_tail_mask(rm, pos.len);
         }
     }
     {
@@ -171,6 +224,14 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
             if (c0 < len) {
+                const int col = c0 + lane * kVec;
+                if constexpr (kRag) {
+                    if (c0 + kChunk >= len) {  // the chunk that holds the row end
+                        ragged_patch16(raw[c], col, len, tail_x);
+                        if constexpr ((FLAGS & kBias) != 0) ragged_patch16(rawb[c], col, len, tail_b);
+                        if constexpr (MASK == Mask::Bytes) ragged_patch_mask(mk[c], col, len, tail_m);
+                    }
+                }
                 unpack8<T>(raw[c], v[c]);
                 if constexpr ((FLAGS & kBias) != 0) {
                     float bv[8];
@@ -178,7 +239,6 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
                     for (int k = 0; k < 8; ++k) v[c][k] += bv[k];
                 }
-                const int col = c0 + lane * kVec;
                 bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
                 if constexpr (MASK == Mask::Bytes) {
                     plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
@@ -263,6 +323,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 o[c] = pack8<T>(v[c]);
             }
             buf_st128<kStNt>(ry, o[c], voff + c * WPR * kChunk * 2, 0);
+            if constexpr (kRag) {
+                if (c0 < sk && c0 + kChunk >= sk) ragged_store16(ry, o[c], c0 + lane * kVec, sk);
+            }
         }
         if constexpr ((FLAGS & kDropout) != 0) {
             // second output after the first: each stream is written in runs of whole rows
@@ -287,6 +350,8 @@ template <typename T, int NCH, int WPR, int RPB, Mask MASK, int FLAGS = kDefault
 __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArgs a) {
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    constexpr bool kRag = (FLAGS & kRagged) != 0;
+    static_assert(!(kRag && (FLAGS & kDropout) != 0), "no dropout on ragged rows");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -299,14 +364,19 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     u32x4 rg[NCH], rp[NCH];
+    uint32_t tail_g = 0, tail_p = 0;  // kRagged: what the range check drops at the row end
     {
-        const uint32_t bytes = (uint32_t)((pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
+        const uint32_t bytes = (uint32_t)(kRag ? pos.len : (pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
         const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2, bytes);
         const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             rg[c] = buf_ld128<kLdNt>(bg, voff + c * WPR * kChunk * 2, 0);
             rp[c] = buf_ld128<kLdNt>(by, voff + c * WPR * kChunk * 2, 0);
+        }
+        if constexpr (kRag) {
+            tail_g = ragged_tail16(bg, pos.len);
+            tail_p = ragged_tail16(by, pos.len);
         }
     }
     {
@@ -321,10 +391,16 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
             const int c0 = (wir + WPR * c) * kChunk;
             kb[c] = 0xffu;
             if (c0 < len) {
+                const int col = c0 + lane * kVec;
+                if constexpr (kRag) {
+                    if (c0 + kChunk >= len) {  // the chunk that holds the row end
+                        ragged_patch16(rg[c], col, len, tail_g);
+                        ragged_patch16(rp[c], col, len, tail_p);
+                    }
+                }
                 float gv[8], pv[8];
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
-                const int col = c0 + lane * kVec;
                 if constexpr ((FLAGS & kDropout) != 0) {
                     kb[c] = keep_bits8(drop, drop_group(pos.row, sk, c0) + lane);
 #pragma unroll
@@ -363,6 +439,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                 o = pack8<T>(gv);
             }
             buf_st128<kStNt>(rdx, o, voff + c * WPR * kChunk * 2, 0);
+            if constexpr (kRag) {
+                if (c0 < sk && c0 + kChunk >= sk) ragged_store16(rdx, o, c0 + lane * kVec, sk);
+            }
         }
     }
 }
@@ -383,7 +462,6 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
 // nothing to fetch.  Reductions stay inside the lane group.
 // ---------------------------------------------------------------------------------
 constexpr int kPackedPasses = 4;  // default number of passes R
-constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;
 
 // (i0 + lr) mod sq for lr below the rows of a wave: one conditional subtraction when a
 // matrix has at least that many rows, a division only for tiny matrices.
@@ -865,8 +943,10 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
 
 // ---------------------------------------------------------------------------------
 // Any-shape kernels: one 256-thread block per row, element-wise accesses, the row
-// is re-read for each pass (from L2).  Used when sk is not a multiple of 8, a
-// pointer is not 16-byte aligned, or the row exceeds the register-resident limit.
+// is re-read for each pass (from L2).  Used for what no other kernel takes: rows shorter
+// than 8 columns, rows beyond the LDS-staged limit, ragged rows (sk not a multiple of 8 or
+// a pointer not 16-byte aligned) beyond the register-resident limit or with dropout, and
+// rows beyond the register-resident limit with ALiBi, a bias tensor or dropout.
 // ---------------------------------------------------------------------------------
 constexpr int kGenericThreads = 256;
 

@@ -85,14 +85,14 @@ __device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
     return w;
 }
 
-// Streaming 128-bit access: every byte of these kernels is touched exactly once,
-// so the loads/stores carry the non-temporal hint and do not displace each other in L2.
 // The compiler learns nothing about `w` across this point: values it derived from `w` earlier
 // (an unpacked copy, say) are computed again afterwards rather than kept in registers.
 __device__ __forceinline__ void forget_origin(u32x4& w) {
     asm volatile("" : "+v"(w.x), "+v"(w.y), "+v"(w.z), "+v"(w.w));
 }
 
+// Streaming 128-bit access: every byte of these kernels is touched exactly once,
+// so the loads/stores carry the non-temporal hint and do not displace each other in L2.
 __device__ __forceinline__ u32x4 ld128(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
@@ -125,6 +125,16 @@ __device__ __forceinline__ void buf_st128(rsrc_t r, const u32x4& v, int voffset,
 }
 __device__ __forceinline__ u32x2 buf_ld64(rsrc_t r, int voffset, int soffset) {
     return __builtin_amdgcn_raw_buffer_load_b64(r, voffset, soffset, 0);
+}
+// Narrow accesses for the ends of rows that are not a whole number of dwords.
+__device__ __forceinline__ uint32_t buf_ld32(rsrc_t r, int voffset) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voffset, 0, 0);
+}
+__device__ __forceinline__ uint32_t buf_ld16(rsrc_t r, int voffset) {
+    return __builtin_amdgcn_raw_buffer_load_b16(r, voffset, 0, 0);
+}
+__device__ __forceinline__ void buf_st16(rsrc_t r, uint32_t v, int voffset) {
+    __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, r, voffset, 0, 0);
 }
 
 // ---- wave64 reductions --------------------------------------------------------

@@ -111,7 +111,12 @@ def test_golden_dropout(device, golden, name, dtype):
 # forward
 # ---------------------------------------------------------------------------------
 def check_forward(y, dropped, y_plain, p, seed, offset, device):
-    assert torch.equal(y, y_plain)  # the saved probabilities are the plain kernels'
+    if y.shape[-1] % 8 == 0 or y.shape[-1] < 8:
+        assert torch.equal(y, y_plain)  # the saved probabilities are the plain kernels'
+    else:
+        # ragged rows: the plain call runs the ragged row kernels, the dropout call the
+        # element-wise ones; their fp32 sums run in different orders
+        assert max_err(y, y_plain) <= (2.0**-8 if y.dtype == torch.bfloat16 else 2.0**-11)
     keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
     assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
     return keep

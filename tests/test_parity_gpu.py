@@ -1018,3 +1018,142 @@ def test_lds_staged_rows_masks_scales_and_aliasing(device, dtype, scale, sk):
     # the mask shared by all samples
     y1 = masked_ext.forward(x, mask[:1], scale)
     assert max_err(y1, R.softmax_fp32(x, mask[:1], scale)) <= TOL[dtype]
+
+
+# ---------------------------------------------------------------------------------
+# ragged rows: sk not a multiple of 8, tensors at any 2-byte alignment
+# ---------------------------------------------------------------------------------
+RAGGED_CAUSAL = [9, 15, 17, 33, 63, 65, 127, 129, 255, 511, 513, 1001, 1023, 1025, 1537, 2047, 2049, 3001, 4095, 4097,
+                 5003, 8191, 10001, 20003, 32767]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("s", RAGGED_CAUSAL)
+def test_ragged_causal_sizes(device, s, dtype):
+    # three matrices: rows start at every 2-byte alignment, row lengths of both parities
+    check_causal(device, 3 if s <= 2049 else 1, s, dtype, 0.125, seed=s, chunk=1)
+
+
+RAGGED_MASKED = [(2, 3, 5, 9), (2, 2, 7, 33), (3, 2, 9, 129), (2, 2, 6, 250), (2, 3, 5, 515), (2, 2, 5, 1001), (1, 2, 3, 2047),
+                 (2, 2, 3, 2050), (1, 2, 3, 4099), (1, 1, 3, 9001), (1, 1, 3, 16388), (1, 1, 2, 32767)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", RAGGED_MASKED)
+def test_ragged_masked_shapes(device, shape, dtype):
+    b, heads, sq, sk = shape
+    check_masked(device, b, heads, sq, sk, dtype, 0.125, seed=sum(shape))
+    # an arbitrary pattern, and the last one to three keys of a row hidden or alone visible: the
+    # mask bytes next to the row end travel by an access of their own
+    pattern = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, sk)) < 0.4
+    for i in range(sq):
+        tail = 1 + i % 3
+        pattern[0, 0, i, :] = False
+        pattern[0, 0, i, sk - tail:] = True
+        if b > 1:
+            pattern[1, 0, i, :] = True
+            pattern[1, 0, i, sk - tail:] = False
+    check_masked(device, b, heads, sq, sk, dtype, 0.5, seed=sk, mask=pattern)
+    check_masked(device, b, heads, sq, sk, dtype, 0.5, seed=sk, mask=pattern[:1])
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3, 4, 7])
+@pytest.mark.parametrize("sk", [16, 512, 1000, 1001, 2048, 4099])
+def test_tensors_at_any_two_byte_alignment(device, sk, offset):
+    # every tensor of the call starts `offset` elements into its allocation (the mask `offset` bytes)
+    dtype, b, heads, sq, scale = torch.float16, 2, 2, 5, 0.25
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + offset, dtype=t.dtype, device=device)
+        flat[offset:] = t.reshape(-1)
+        return flat[offset:].view(t.shape)
+
+    x = scores((b, heads, sq, sk), dtype, device, sk)
+    g = normal((b, heads, sq, sk), dtype, device, sk + 1)
+    mask = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, sk + 2)) < 0.3
+    xs, gs, ms = shifted(x), shifted(g), shifted(mask)
+    assert xs.data_ptr() % 16 == (2 * offset) % 16 and xs.is_contiguous()
+    y = masked_ext.forward(xs, ms, scale)
+    assert max_err(y, R.softmax_fp32(x, mask, scale)) <= TOL[dtype]
+    assert (y[mask.expand_as(y)] == 0).all()
+    ys = shifted(y)
+    dx = masked_ext.backward(gs, ys, scale)
+    assert dx.data_ptr() == gs.data_ptr()
+    assert max_err(dx, R.softmax_backward_fp32(g, y, scale)) <= TOL[dtype]
+    # causal, square
+    n = min(sk, 1001)
+    xc = scores((3, n, n), dtype, device, sk + 3)
+    yc = causal_ext.forward(shifted(xc), scale)
+    assert max_err(yc.unsqueeze(0), R.softmax_fp32(xc.unsqueeze(0), R.get_attn_mask(n, device), scale)) <= TOL[dtype]
+    gc = normal((3, n, n), dtype, device, sk + 4)
+    dxc = causal_ext.backward(shifted(gc), shifted(yc), scale)
+    assert max_err(dxc, R.softmax_backward_fp32(gc, yc, scale)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("sk", [9, 515, 1001, 2047, 4099, 9001])
+def test_ragged_rows_write_exactly_their_output(device, sk):
+    # outputs surrounded by guard elements, every element of the output pre-set: the kernels
+    # write each element of the rows (zeros above the diagonal included) and nothing else
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    guard = 64
+    for dtype in DTYPES:
+        code = _lib.dtype_code(dtype)
+        for kind in ("causal", "masked"):
+            rows_shape = (2, sk, sk) if kind == "causal" and sk <= 2047 else (2, 1, 5, sk)
+            causal = len(rows_shape) == 3
+            x = scores(rows_shape, dtype, device, sk)
+            g = normal(rows_shape, dtype, device, sk + 1)
+            n = x.numel()
+            for pad in (guard, guard + 1, guard + 3):  # output base at different alignments
+                out = torch.full((n + 2 * guard + 8,), 7.0, dtype=dtype, device=device)
+                dxo = torch.full((n + 2 * guard + 8,), 7.0, dtype=dtype, device=device)
+                y, dx = out[pad : pad + n], dxo[pad : pad + n]
+                if causal:
+                    _lib.check(lib.neox_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), 0.125, 2, sk, sk, code, stream))
+                    want = R.softmax_fp32(x.unsqueeze(0), R.get_attn_mask(sk, device), 0.125)[0]
+                    _lib.check(lib.neox_causal_softmax_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), 0.125, 2, sk, sk, code, stream))
+                else:
+                    mask = torch.rand(2, 1, 5, sk, device=device, generator=gen(device, sk)) < 0.3
+                    _lib.check(lib.neox_masked_softmax_fwd(y.data_ptr(), x.data_ptr(), mask.data_ptr(), 0.125, 2, 1, 5, sk, 2, code, stream))
+                    want = R.softmax_fp32(x, mask, 0.125)
+                    _lib.check(lib.neox_masked_softmax_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), 0.125, 10, sk, code, stream))
+                assert max_err(y.view(rows_shape), want) <= TOL[dtype], (sk, kind, pad)
+                wantb = R.softmax_backward_fp32(g, y.view(rows_shape), 0.125)
+                assert max_err(dx.view(rows_shape), wantb) <= TOL[dtype], (sk, kind, pad)
+                for buf in (out, dxo):
+                    assert (buf[:pad] == 7.0).all() and (buf[pad + n:] == 7.0).all(), (sk, kind, pad)
+
+
+@pytest.mark.parametrize("s", [9, 513, 1001, 2047, 4099])
+def test_ragged_causal_kernels_ignore_what_lies_past_the_diagonal(device, s):
+    upper = torch.ones(s, s, dtype=torch.bool, device=device).triu_(1)
+    for dtype in DTYPES:
+        x = scores((2, s, s), dtype, device, s)
+        g = normal((2, s, s), dtype, device, s + 1)
+        y = causal_ext.forward(x, 0.125)
+        dx = causal_ext.backward(g.clone(), y, 0.125)
+        assert torch.equal(causal_ext.forward(x.masked_fill(upper, float("nan")), 0.125), y)
+        for poison_g, poison_y in ((float("nan"), float("nan")), (float("inf"), 0.0), (1.0, float("-inf"))):
+            got = causal_ext.backward(g.masked_fill(upper, poison_g), y.masked_fill(upper, poison_y), 0.125)
+            assert torch.equal(got, dx), (s, dtype, poison_g, poison_y)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 3, 9, 9), (2, 2, 65, 65), (1, 3, 513, 513), (2, 2, 1001, 1001), (1, 2, 2047, 2047)])
+def test_ragged_rows_with_alibi_and_bias(device, shape, dtype):
+    b, heads, sq, sk = shape
+    x = scores(shape, dtype, device, sk)
+    slopes = torch.rand(heads, device=device, generator=gen(device, 3)) * 0.5
+    causal = R.get_attn_mask(sk, device)
+    y = causal_ext.forward_alibi(x, slopes, 0.25)
+    bias = R.alibi_bias_fp32(slopes.cpu(), sq, sk).to(device)
+    assert max_err(y, R.softmax_fp32(x.float() + bias, causal, 0.25)) <= TOL[dtype]
+    for shared in (True, False):
+        rpe = normal((1 if shared else b, heads, sq, sk), dtype, device, sk + 5)
+        yb = causal_ext.forward_bias(x, rpe, 0.25)
+        assert max_err(yb, R.softmax_fp32(x.float() + rpe.float(), causal, 0.25)) <= TOL[dtype]
+        assert (yb[causal.expand_as(yb)] == 0).all()
+        pad = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, sk + 6)) < 0.3
+        ym = masked_ext.forward_bias(x, pad, rpe, 0.25)
+        assert max_err(ym, R.softmax_fp32(x.float() + rpe.float(), pad, 0.25)) <= TOL[dtype]
