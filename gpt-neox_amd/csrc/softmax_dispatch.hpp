@@ -12,6 +12,8 @@
 //   chunks <= 8    4 waves per row                                   (sk <= 4096)
 //   chunks <= 16   8 waves per row, 512-thread block                 (sk <= 8192)
 //   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
+//                  forward, in the lower 3/4 of each of these three ranges (7/8 of the last):
+//                  half as many waves with 3 (4) chunks each
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
@@ -166,6 +168,17 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if constexpr (!BWD && M == Mask::Causal && (EXTRA & kDropout) != 0)
             return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
         return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
+    }
+    if constexpr (!BWD) {
+        // Forward, rows that would leave a quarter or more of the 2-chunk shape's slots empty:
+        // half as many waves with 3 or 4 chunks each.  Measured in an interleaved comparison:
+        // +20-50 % just above a power of two (2056, 4104, 8200 columns), +4-15 % up to 3/4 (7/8 with
+        // 4 chunks) of the range, while full rows lose 2-3 % with 4 chunks per wave and the
+        // backward pass gains nothing.
+        if (chunks <= 6) return launch_shape<T, M, BWD, EXTRA, 3, 2, 2>(a, st);
+        if (chunks > 8 && chunks <= 12) return launch_shape<T, M, BWD, EXTRA, 3, 4, 1>(a, st);
+        if (chunks > 16 && chunks <= 24) return launch_shape<T, M, BWD, EXTRA, 3, 8, 1>(a, st);
+        if (chunks > 24 && chunks <= 28) return launch_shape<T, M, BWD, EXTRA, 4, 8, 1>(a, st);
     }
     if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
     if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);

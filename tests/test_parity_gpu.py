@@ -162,8 +162,8 @@ def check_causal(device, batches, s, dtype, scale, seed, chunk=4):
 # row lengths chosen to hit: 1 column; lanes partly filled; not a multiple of 8 (element-wise
 # kernels); 1 and 2 chunks of 512 columns on one wave; the 2-, 4- and 8-wave kernels with rows
 # that fill their last chunk exactly, partly, or leave whole chunks of a wave empty.
-CAUSAL_SIZES = [1, 2, 7, 8, 16, 24, 37, 40, 64, 72, 120, 128, 200, 256, 264, 384, 504, 512, 520, 1000, 1024, 1536, 2048, 2056, 3072, 4096,
-                5000, 6144, 8192]
+CAUSAL_SIZES = [1, 2, 7, 8, 16, 24, 37, 40, 64, 72, 120, 128, 200, 256, 264, 384, 504, 512, 520, 1000, 1024, 1536, 2048, 2056, 2560, 3072,
+                4096, 4104, 5000, 6144, 8192]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -173,7 +173,7 @@ def test_causal_sizes(device, s, dtype):
     check_causal(device, batches, s, dtype, 0.125, seed=s)
 
 
-@pytest.mark.parametrize("s", [12288, 16384, 20000, 28672, 33000, 40448, 40456, 40968])
+@pytest.mark.parametrize("s", [8200, 10240, 12288, 13312, 14336, 16384, 20000, 28672, 33000, 40448, 40456, 40968])
 def test_causal_very_long_rows(device, s):
     # 16 waves per row with 2, 3 and 4 chunks per wave; from 33000 on the row exceeds the register
     # budget and is staged in LDS: in half of a CU's LDS up to 40448 columns, in all of it beyond
@@ -469,7 +469,8 @@ MASKED_SHAPES = [(2, 3, 4, 1), (2, 2, 5, 37), (1, 2, 8, 8), (3, 5, 7, 8), (2, 3,
                  (3, 3, 50, 72), (2, 2, 31, 128), (2, 3, 17, 200), (2, 2, 65, 256), (1, 3, 129, 384), (2, 2, 9, 512), (3, 2, 9, 520),
                  (2, 2, 33, 1000), (2, 2, 8, 1024), (1, 2, 6, 2048), (1, 1, 4, 3072), (1, 2, 3, 4096),
                  (1, 1, 3, 8192), (1, 1, 2, 12000), (1, 1, 2, 20000), (1, 1, 2, 30000), (1, 1, 2, 40000), (1, 3, 1, 77),
-                 (2, 2, 3, 32776), (1, 2, 2, 65536), (1, 1, 3, 81408), (1, 1, 2, 81416)]
+                 (2, 2, 3, 32776), (1, 2, 2, 65536), (1, 1, 3, 81408), (1, 1, 2, 81416),
+                 (1, 2, 3, 2560), (1, 2, 3, 4104), (1, 1, 3, 10240), (1, 1, 2, 13312), (1, 1, 2, 14344)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
