@@ -18,8 +18,7 @@
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
 //   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768, no dropout)
-//                  the same one- to sixteen-wave row kernels with the kRagged flag; rows up to
-//                  512 columns get one wave each
+//                  the same packed and one- to sixteen-wave row kernels with the kRagged flag
 //   anything else  element-wise kernels (ragged rows with dropout or outside that range, rows
 //                  beyond 81408 columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
@@ -154,9 +153,14 @@ template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     const int chunks = (a.sk + kChunk - 1) / kChunk;
     if constexpr ((EXTRA & kRagged) != 0) {
-        // rows at any alignment: the row kernels below, one wave per row up to 512 columns
+        // rows at any alignment: the packed kernels up to 512 columns, the row kernels below beyond
         if (a.sk < kVec || a.sk > kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
-        if (chunks == 1) return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
+        if (chunks == 1) {
+            const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
+                                (a.bias == nullptr || a.bias_bytes != 0);
+            if (fits32) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
+            return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
+        }
     } else {
         const hipError_t e = dispatch_aligned<T, M, BWD, EXTRA>(a, vec_ok, chunks, st);
         if (e != hipErrorNotReady) return e;

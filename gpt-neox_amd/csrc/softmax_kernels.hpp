@@ -470,6 +470,72 @@ __device__ __forceinline__ uint32_t wrap_row(uint32_t i, uint32_t sq) {
     return i % sq;
 }
 
+// kRagged in the packed kernels.  A wave's rows lie back to back behind one buffer, so the lane
+// that holds the end of a row must not touch the columns that follow: they belong to the next
+// row.  Every row ends the same way, with rem = sk % 8 columns in its last lane, and that lane
+// moves them by a 64-, a 32- and a 16-bit access instead of one of 128 bits -- rem = 4a + 2b + c;
+// a piece that rem does not contain is skipped by the whole wave, and the lanes that are not at
+// a row end aim the others out of range.
+//
+// 128-bit access of the packed kernels: whole when the lane's 8 columns lie inside its row (always
+// so without RAG), in pieces at a ragged row end, nothing for an inactive lane.  `off`: byte
+// offset of the lane's first column; `left`: columns from there to the row end; `rem`: sk % 8.
+template <bool NT, bool RAG>
+__device__ __forceinline__ u32x4 packed_ld(rsrc_t r, uint32_t off, int left, bool active, int rem) {
+    u32x4 v = buf_ld128<NT>(r, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
+    if constexpr (RAG) {
+        const bool end = active && left < kVec;  // a row-end lane: left == rem
+        if (rem & 4) {
+            const u32x2 a = buf_ld64(r, end ? off : kOutOfRange, 0);
+            v.x |= a.x;
+            v.y |= a.y;
+        }
+        if (rem & 2) {
+            const uint32_t b = buf_ld32(r, end ? off + (uint32_t)(rem & 4) * 2u : kOutOfRange);
+            if (rem & 4) v.z |= b;
+            else v.x |= b;
+        }
+        if (rem & 1) {
+            const uint32_t c = buf_ld16(r, end ? off + (uint32_t)(rem & 6) * 2u : kOutOfRange);
+            if (rem == 1) v.x |= c;
+            else if (rem == 3) v.y |= c;
+            else if (rem == 5) v.z |= c;
+            else v.w |= c;
+        }
+    }
+    return v;
+}
+template <bool NT, bool RAG>
+__device__ __forceinline__ void packed_st(rsrc_t r, const u32x4& v, uint32_t off, int left, bool active, int rem) {
+    buf_st128<NT>(r, v, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
+    if constexpr (RAG) {
+        const bool end = active && left < kVec;
+        if (rem & 4) buf_st64(r, u32x2{v.x, v.y}, end ? off : kOutOfRange);
+        if (rem & 2) buf_st32(r, (rem & 4) ? v.z : v.x, end ? off + (uint32_t)(rem & 4) * 2u : kOutOfRange);
+        if (rem & 1)
+            buf_st16(r, rem == 1 ? v.x : rem == 3 ? v.y : rem == 5 ? v.z : v.w,
+                     end ? off + (uint32_t)(rem & 6) * 2u : kOutOfRange);
+    }
+}
+// The lane's 8 mask bytes, likewise (pieces of 4, 2 and 1 bytes at a ragged row end).
+template <bool RAG>
+__device__ __forceinline__ u32x2 packed_ld_mask(rsrc_t r, uint32_t off, int left, bool active, int rem) {
+    u32x2 v = buf_ld64(r, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
+    if constexpr (RAG) {
+        const bool end = active && left < kVec;
+        uint32_t low = 0;  // the bytes after the 4-byte piece
+        if (rem & 2) low = buf_ld16(r, end ? off + (uint32_t)(rem & 4) : kOutOfRange);
+        if (rem & 1) low |= buf_ld8(r, end ? off + (uint32_t)(rem & 6) : kOutOfRange) << (8 * (rem & 2));
+        if (rem & 4) {
+            v.x |= buf_ld32(r, end ? off : kOutOfRange);
+            v.y |= low;
+        } else {
+            v.x |= low;
+        }
+    }
+    return v;
+}
+
 template <int G, int R = kPackedPasses>
 struct Packed {
     static constexpr int kRowsPerPass = kWave / G;
@@ -482,12 +548,15 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     static_assert(C == 1 || G == kWave, "several chunks per row need a whole wave per row");
     constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    constexpr bool kRag = (FLAGS & kRagged) != 0;
+    static_assert(!kRag || (C == 1 && (FLAGS & kDropout) == 0), "ragged rows: one chunk, no dropout");
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t row0 = wave * RPW;  // first row of this wave
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
     const int sk = a.sk;
+    const int rem = sk & (kVec - 1);  // kRagged: columns in the last lane of a row
     const int grp = lane / G;
     const int col0 = (lane % G) * kVec;
     DropoutArgs drop = a.drop;
@@ -526,15 +595,15 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
-            raw[p][c] = buf_ld128<kLdNt>(rx, col < len[p] ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            raw[p][c] = packed_ld<kLdNt, kRag>(rx, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
             if constexpr ((FLAGS & kBias) != 0) {
                 const uint32_t boff = (bias_row(row, a) * (uint32_t)sk + col) * 2u;
-                rawb[p][c] = buf_ld128<false>(rb, col < len[p] ? boff : kOutOfRange, 0);
+                rawb[p][c] = packed_ld<false, kRag>(rb, boff, sk - col, col < len[p], rem);
             }
             if constexpr (MASK == Mask::Bytes) {
                 const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
                 const uint32_t moff = (mb * (uint32_t)a.sq + i) * sk + col;
-                mk[p][c] = buf_ld64(rm, col < len[p] ? moff : kOutOfRange, 0);
+                mk[p][c] = packed_ld_mask<kRag>(rm, moff, sk - col, col < len[p], rem);
             }
         }
     }
@@ -601,7 +670,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
             for (int k = 0; k < 8; ++k) v[c][k] *= inv;  // lanes of absent rows hold NaN and store nothing
             const bool st = lr < rows_here && col < sk;
             const u32x4 o = pack8<T>(v[c]);
-            buf_st128<kStNt>(ry, o, st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            packed_st<kStNt, kRag>(ry, o, (lr * sk + col) * 2u, sk - col, st, rem);
             if constexpr ((FLAGS & kDropout) != 0) {
                 const uint32_t bits = keep_bits8(drop, drop_group(row0 + lr, sk, col));
                 buf_st128<kStNt>(ry2, dropout8<T>(o, bits, drop.scale), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
@@ -615,12 +684,15 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     static_assert(C == 1 || G == kWave, "several chunks per row need a whole wave per row");
     constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
+    constexpr bool kRag = (FLAGS & kRagged) != 0;
+    static_assert(!kRag || (C == 1 && (FLAGS & kDropout) == 0), "ragged rows: one chunk, no dropout");
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t row0 = wave * RPW;
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
     const int sk = a.sk;
+    const int rem = sk & (kVec - 1);  // kRagged: columns in the last lane of a row
     const int grp = lane / G;
     const int col0 = (lane % G) * kVec;
     DropoutArgs drop = a.drop;
@@ -642,9 +714,8 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
-            const uint32_t o = col < len[p] ? (lr * sk + col) * 2u : kOutOfRange;
-            rg[p][c] = buf_ld128<kLdNt>(bg, o, 0);
-            rp[p][c] = buf_ld128<kLdNt>(by, o, 0);
+            rg[p][c] = packed_ld<kLdNt, kRag>(bg, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
+            rp[p][c] = packed_ld<kLdNt, kRag>(by, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
         }
     }
 #pragma unroll
@@ -681,7 +752,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
                 if ((col + k) >= len[p]) gv[k] = 0.f;
             }
             const bool st = lr < rows_here && col < sk;
-            buf_st128<kStNt>(bo, pack8<T>(gv), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+            packed_st<kStNt, kRag>(bo, pack8<T>(gv), (lr * sk + col) * 2u, sk - col, st, rem);
         }
     }
 }

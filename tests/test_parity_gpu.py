@@ -1158,3 +1158,21 @@ def test_ragged_rows_with_alibi_and_bias(device, shape, dtype):
         pad = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, sk + 6)) < 0.3
         ym = masked_ext.forward_bias(x, pad, rpe, 0.25)
         assert max_err(ym, R.softmax_fp32(x.float() + rpe.float(), pad, 0.25)) <= TOL[dtype]
+
+
+def test_ragged_short_rows_every_row_end_and_group_size(device):
+    # rows of 8m + r columns, r = 1..7, for every lane-group size of the several-rows-per-wave
+    # kernels: the lane at a row end moves its r columns in pieces of 4, 2 and 1
+    for m in (1, 2, 3, 4, 8, 16, 32, 63):
+        for r in range(1, 8):
+            sk = 8 * m + r
+            dtype = DTYPES[(m + r) % 2]
+            check_causal(device, 3, sk, dtype, 0.25, seed=sk, chunk=3)
+            mask = torch.rand(2, 1, 5, sk, device=device, generator=gen(device, sk)) < 0.3
+            mask[0, 0, 1, :] = True                      # a row with every key hidden
+            mask[1, 0, 2, :] = False
+            mask[1, 0, 2, sk - r:] = True                # exactly the columns of the row-end lane hidden
+            mask[1, 0, 3, :] = True
+            mask[1, 0, 3, sk - r:] = False               # ... and those alone visible
+            check_masked(device, 2, 3, 5, sk, dtype, 0.25, seed=sk, mask=mask)
+            check_masked(device, 2, 3, 5, sk, dtype, 0.25, seed=sk, mask=mask[:1])
