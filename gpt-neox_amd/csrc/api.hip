@@ -352,7 +352,7 @@ int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const 
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_dropout_fwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_dropout_fwd, Mask::Causal, stream, launch_softmax_ragged_dropout_fwd);
 }
 
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
@@ -364,7 +364,7 @@ int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_dropout_bwd, Mask::Causal, stream);
+    return c.launch(launch_softmax_dropout_bwd, Mask::Causal, stream, launch_softmax_ragged_dropout_bwd);
 }
 
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
@@ -380,7 +380,7 @@ int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const 
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_dropout_fwd, Mask::Bytes, stream);
+    return c.launch(launch_softmax_dropout_fwd, Mask::Bytes, stream, launch_softmax_ragged_dropout_fwd);
 }
 
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
@@ -392,7 +392,7 @@ int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_dropout_bwd, Mask::None, stream);
+    return c.launch(launch_softmax_dropout_bwd, Mask::None, stream, launch_softmax_ragged_dropout_bwd);
 }
 
 int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset,

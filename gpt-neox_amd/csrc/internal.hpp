@@ -29,11 +29,15 @@ hipError_t launch_softmax_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype
 hipError_t launch_softmax_bias_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                    hipStream_t stream);
 // Rows at any 2-byte alignment with 8 <= sk <= kMaxRegisterRow (a.bias optional in the forward
-// pass, no dropout); `vec_ok` is ignored.
+// passes), without and with attention dropout; `vec_ok` is ignored.
 hipError_t launch_softmax_ragged_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                      hipStream_t stream);
 hipError_t launch_softmax_ragged_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                      hipStream_t stream);
+hipError_t launch_softmax_ragged_dropout_fwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                             hipStream_t stream);
+hipError_t launch_softmax_ragged_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
+                                             hipStream_t stream);
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream);
 

@@ -17,10 +17,10 @@
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
-//   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768, no dropout)
+//   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768)
 //                  the same packed and one- to sixteen-wave row kernels with the kRagged flag
-//   anything else  element-wise kernels (ragged rows with dropout or outside that range, rows
-//                  beyond 81408 columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
+//   anything else  element-wise kernels (ragged rows outside that range, rows beyond 81408
+//                  columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
 
 #include <type_traits>

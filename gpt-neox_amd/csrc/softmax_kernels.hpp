@@ -65,8 +65,8 @@ constexpr int kBias = 16;
 // every dword inside the row is transferred and only a dword that crosses the row end is
 // dropped.  For 16-bit data that is the last element of an odd-length row, which these kernels
 // move by a 16-bit access of its own; for the mask bytes it is the last len % 4 bytes, fetched
-// again by a dword load that ends with the row.  (Row kernels only; not with kDropout, whose
-// groups of 8 elements would straddle rows.)
+// again by a dword load that ends with the row.  With kDropout a lane's 8 columns straddle two
+// Philox groups (the pattern is a function of the row-major element index).
 constexpr int kRagged = 32;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
 constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;  // a byte offset no buffer contains
@@ -115,6 +115,22 @@ __device__ __forceinline__ uint32_t bias_row(uint32_t row, const SoftmaxArgs& a)
 // Philox group (8 consecutive elements) of column `col` (a multiple of 8) of row `row`
 __device__ __forceinline__ uint64_t drop_group(uint32_t row, int sk, int col) {
     return (uint64_t)row * (uint32_t)(sk >> 3) + (uint32_t)(col >> 3);
+}
+
+// Keep bits of the 8 columns from `col` (a multiple of 8) of row `row`.  Aligned rows: one Philox
+// group.  Ragged rows (RAG): the 8 elements straddle two groups unless the row happens to start
+// on a group boundary, which is the same for every lane of a wave.
+template <bool RAG>
+__device__ __forceinline__ uint32_t keep_bits_row8(const DropoutArgs& d, uint32_t row, int sk, int col) {
+    if constexpr (!RAG) {
+        return keep_bits8(d, drop_group(row, sk, col));
+    } else {
+        const uint64_t e = (uint64_t)row * (uint32_t)sk + (uint32_t)col;
+        const uint32_t shift = (uint32_t)e & 7u;
+        uint32_t bits = keep_bits8(d, e >> 3) >> shift;
+        if (shift != 0) bits |= keep_bits8(d, (e >> 3) + 1) << (8u - shift);
+        return bits & 0xffu;
+    }
 }
 
 // Where a wave works: the row, its position i inside its [sq, sk] matrix, the number of
@@ -169,7 +185,6 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
-    static_assert(!(kRag && (FLAGS & kDropout) != 0), "no dropout on ragged rows");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave in block
@@ -334,10 +349,13 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 const int c0 = (wir + WPR * c) * kChunk;
                 u32x4 o2 = u32x4{0, 0, 0, 0};
                 if (c0 < len) {
-                    const uint32_t bits = keep_bits8(drop, drop_group(pos.row, sk, c0) + lane);
+                    const uint32_t bits = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec);
                     o2 = dropout8<T>(o[c], bits, drop.scale);
                 }
                 buf_st128<kStNt>(ry2, o2, voff + c * WPR * kChunk * 2, 0);
+                if constexpr (kRag) {
+                    if (c0 < sk && c0 + kChunk >= sk) ragged_store16(ry2, o2, c0 + lane * kVec, sk);
+                }
             }
         }
     }
@@ -351,7 +369,6 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
-    static_assert(!(kRag && (FLAGS & kDropout) != 0), "no dropout on ragged rows");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -402,7 +419,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
                 if constexpr ((FLAGS & kDropout) != 0) {
-                    kb[c] = keep_bits8(drop, drop_group(pos.row, sk, c0) + lane);
+                    kb[c] = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec);
 #pragma unroll
                     for (int k = 0; k < 8; ++k) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 }
@@ -549,7 +566,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
-    static_assert(!kRag || (C == 1 && (FLAGS & kDropout) == 0), "ragged rows: one chunk, no dropout");
+    static_assert(!kRag || C == 1, "ragged rows: one chunk per lane group");
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t row0 = wave * RPW;  // first row of this wave
@@ -672,8 +689,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
             const u32x4 o = pack8<T>(v[c]);
             packed_st<kStNt, kRag>(ry, o, (lr * sk + col) * 2u, sk - col, st, rem);
             if constexpr ((FLAGS & kDropout) != 0) {
-                const uint32_t bits = keep_bits8(drop, drop_group(row0 + lr, sk, col));
-                buf_st128<kStNt>(ry2, dropout8<T>(o, bits, drop.scale), st ? (lr * sk + col) * 2u : kOutOfRange, 0);
+                const uint32_t bits = keep_bits_row8<kRag>(drop, row0 + lr, sk, col);
+                packed_st<kStNt, kRag>(ry2, dropout8<T>(o, bits, drop.scale), (lr * sk + col) * 2u, sk - col, st, rem);
             }
         }
     }
@@ -685,7 +702,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     constexpr int RPP = Packed<G, R>::kRowsPerPass, RPW = Packed<G, R>::kRowsPerWave;
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
-    static_assert(!kRag || (C == 1 && (FLAGS & kDropout) == 0), "ragged rows: one chunk, no dropout");
+    static_assert(!kRag || C == 1, "ragged rows: one chunk per lane group");
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t row0 = wave * RPW;
@@ -730,7 +747,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             unpack8<T>(rg[p][c], gv);
             unpack8<T>(rp[p][c], pv);
             kb[c] = 0xffu;
-            if constexpr ((FLAGS & kDropout) != 0) kb[c] = keep_bits8(drop, drop_group(row0 + lr, sk, col0 + c * kChunk));
+            if constexpr ((FLAGS & kDropout) != 0) kb[c] = keep_bits_row8<kRag>(drop, row0 + lr, sk, col0 + c * kChunk);
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
@@ -1016,8 +1033,8 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
 // Any-shape kernels: one 256-thread block per row, element-wise accesses, the row
 // is re-read for each pass (from L2).  Used for what no other kernel takes: rows shorter
 // than 8 columns, rows beyond the LDS-staged limit, ragged rows (sk not a multiple of 8 or
-// a pointer not 16-byte aligned) beyond the register-resident limit or with dropout, and
-// rows beyond the register-resident limit with ALiBi, a bias tensor or dropout.
+// a pointer not 16-byte aligned) beyond the register-resident limit, and rows beyond the
+// register-resident limit with ALiBi, a bias tensor or dropout.
 // ---------------------------------------------------------------------------------
 constexpr int kGenericThreads = 256;
 
