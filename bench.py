@@ -563,6 +563,18 @@ def main():
                 r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
             result["fused_bias"] = [r]
             del s_, z, rpe
+        # evaluation / prefill lengths: rows that are not a multiple of 8 columns long, so that every
+        # row starts at another 2-byte alignment (causal forward, the pass an evaluation runs)
+        if want("ragged"):
+            ragged = []
+            for B, n, dt, nl in ((48, 2047, torch.bfloat16, 100), (96, 1001, torch.float16, 100), (1024, 129, torch.float16, 100)):
+                sc = 0.125
+                s_ = causal_sets(B, n, dt, 1245, nsets=2, need_bwd=False)
+                name = f"causal fwd [{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} (ragged rows)"
+                r = row(name, B * 2 * (tri(n) + n * n), *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, nl))
+                ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
+                del s_
+            result["evaluation_lengths"] = ragged
         # what the memory pattern of the partial rotary costs by itself: the first 64 of every 256
         # bytes of a 134 MB buffer loaded and stored back (cfg3's q and k), and the same number of
         # bytes as one contiguous run
