@@ -544,3 +544,84 @@ def test_dropout_function_gradient_reaches_the_bias(device, shared):
         assert max_err(x.grad, xr.grad) <= tol * max(1.0, xr.grad.abs().max().item())
         assert bias.grad.shape == bias.shape
         assert max_err(bias.grad, br.grad) <= tol * max(1.0, br.grad.abs().max().item()) * (b if shared else 1)
+
+
+def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
+    # any row length (mostly not a multiple of 8), tensors starting at a random element of their
+    # allocation, and a random choice of mask kind, bias / ALiBi and dropout: every result against
+    # the oracle's fp32 expressions with the kernels' own keep pattern
+    import random
+
+    rnd = random.Random(20250101)
+
+    def shifted(t, by):
+        flat = torch.empty(t.numel() + by, dtype=t.dtype, device=device)
+        flat[by:] = t.reshape(-1)
+        return flat[by:].view(t.shape)
+
+    for case in range(60):
+        dtype = rnd.choice(DTYPES)
+        sk = rnd.choice([rnd.randint(8, 70), rnd.randint(71, 520), rnd.randint(521, 2100), rnd.randint(2101, 9000)])
+        causal = rnd.random() < 0.5
+        b, heads = rnd.randint(1, 2), rnd.randint(1, 3)
+        sq = sk if causal else rnd.randint(1, 6)
+        if causal and sk > 2100:
+            b, heads = 1, 1
+        scale = rnd.choice([0.125, 0.5, 1.0])
+        p = rnd.choice([0.0, 0.0, 0.1, 0.5])
+        extra = rnd.choice(["none", "none", "bias", "shared bias", "alibi"])
+        if extra == "alibi" and not causal:
+            extra = "none"
+        shift = rnd.randint(0, 9)
+        tag = (case, str(dtype), causal, b, heads, sq, sk, scale, p, extra, shift)
+        x = shifted(scores((b, heads, sq, sk), dtype, device, case), shift)
+        g = shifted(normal((b, heads, sq, sk), dtype, device, 1000 + case), shift)
+        bias = slopes = None
+        logits = x.float()
+        if "bias" in extra:
+            bias = shifted(normal((1 if extra == "shared bias" else b, heads, sq, sk), dtype, device, 2000 + case), shift)
+            logits = logits + bias.float()
+        if extra == "alibi":
+            slopes = torch.rand(heads, device=device, generator=gen(device, case)) * 0.5
+            logits = logits + R.alibi_bias_fp32(slopes.cpu(), sq, sk).to(device)
+        if causal:
+            mask = R.get_attn_mask(sk, device)
+        else:
+            mask = torch.rand(rnd.choice([1, b]), 1, sq, sk, device=device, generator=gen(device, 3000 + case)) < 0.3
+            mask = shifted(mask, shift)
+        want = R.softmax_fp32(logits, mask, scale)
+        seed, offset = 77 + case, 4 * case
+        if p == 0.0:
+            if causal:
+                if slopes is not None:
+                    y = causal_ext.forward_alibi(x, slopes, scale)
+                elif bias is not None:
+                    y = causal_ext.forward_bias(x, bias, scale)
+                else:
+                    y = causal_ext.forward(x.view(-1, sq, sk), scale).view(x.shape)
+                dx = causal_ext.backward(g.clone().view(-1, sq, sk), y.view(-1, sq, sk), scale).view(x.shape)
+            else:
+                y = masked_ext.forward_bias(x, mask, bias, scale) if bias is not None else masked_ext.forward(x, mask, scale)
+                dx = masked_ext.backward(g.clone(), y, scale)
+            want_dx = R.softmax_backward_fp32(g, y, scale)
+        else:
+            if causal:
+                y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
+                dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+            else:
+                y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
+                dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+            keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
+            if y.numel() <= 1 << 20:
+                assert np.array_equal(keep.cpu().numpy().reshape(-1), philox.keep_mask(y.numel(), p, seed, offset)), tag
+            assert torch.equal(dropped, R.dropout_with_mask(y, keep, p)), tag
+            want_dx = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
+        assert max_err(y, want) <= TOL[dtype], tag
+        hidden = mask.expand_as(y)
+        full_rows = hidden.all(-1, keepdim=True).expand_as(y)
+        assert (y[hidden & ~full_rows] == 0).all(), tag
+        # the bound scales with the largest gradient and allows for the rounding of values above 1
+        top = want_dx.abs().max().item()
+        half_ulp = top * (2.0**-8 if dtype == torch.bfloat16 else 2.0**-11)
+        assert max_err(dx, want_dx) <= TOL[dtype] * max(1.0, top) + half_ulp, tag
+        assert (dx[hidden & ~full_rows] == 0).all(), tag
