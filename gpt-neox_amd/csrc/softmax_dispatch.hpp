@@ -23,6 +23,7 @@
 //                  columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
 
+#include <optional>
 #include <type_traits>
 
 #include "internal.hpp"
@@ -109,9 +110,9 @@ static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
 }
 
 // The shapes that need 16-byte aligned rows: element-wise kernels when they are not, LDS-staged
-// and packed kernels.  hipErrorNotReady: none of them applies, the row kernels take the call.
+// and packed kernels.  No value: none of them applies, the row kernels take the call.
 template <typename T, Mask M, bool BWD, int EXTRA>
-static hipError_t dispatch_aligned(const SoftmaxArgs& a, bool vec_ok, int chunks, hipStream_t st) {
+static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec_ok, int chunks, hipStream_t st) {
     if (!vec_ok) return launch_generic<T, M, BWD, EXTRA>(a, st);
     if (a.sk > kMaxRegisterRow) {
         // beyond the register budget: the row is staged in LDS (plain kernels only), in half
@@ -146,7 +147,7 @@ static hipError_t dispatch_aligned(const SoftmaxArgs& a, bool vec_ok, int chunks
         if (chunks == 3) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
         if (chunks == 4) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 4>(a, st);
     }
-    return hipErrorNotReady;
+    return std::nullopt;
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA>
@@ -162,8 +163,7 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
             return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
         }
     } else {
-        const hipError_t e = dispatch_aligned<T, M, BWD, EXTRA>(a, vec_ok, chunks, st);
-        if (e != hipErrorNotReady) return e;
+        if (const auto done = dispatch_aligned<T, M, BWD, EXTRA>(a, vec_ok, chunks, st)) return *done;
     }
     if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
     if (chunks == 3) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
