@@ -9,6 +9,10 @@
  *   - validates its arguments before the first HIP call, so argument errors
  *     are reported on a machine without a GPU too.
  * The caller owns all memory.  Element type codes are neox_dtype.
+ * Pointers need the alignment of their element type only (2 bytes for fp16/bf16
+ * tensors) and row lengths need not be multiples of anything: tensors that start
+ * on a 16-byte boundary with sk % 8 == 0 take the fastest kernels, any other
+ * layout runs vectorised kernels built for rows at arbitrary 2-byte alignment.
  *
  * Each declaration cites the reference interface it replaces (paths relative
  * to the GPT-NeoX source tree).
