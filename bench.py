@@ -575,6 +575,85 @@ def main():
                 ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
                 del s_
             result["evaluation_lengths"] = ragged
+        # The reference's own fallback on this GPU, for scale: what FusedScaleMaskSoftmax runs when its
+        # predicate fails (always at sk > 2048, e.g. configs[4]) is the unfused torch branch
+        # (megatron/model/fused_softmax.py:184-199 with gpt2_attention_mask_func,
+        # megatron/model/gpt2_model.py:49-57), and the unfused rotary is the torch expression with the
+        # caller's slice and concatenate (megatron/model/transformer.py:826-860).  Both are timed
+        # here through this package's copies of those branches; the fused figure beside each is the
+        # sum of the kernels the fused modules launch for the same work.
+        if want("unfused"):
+            from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+            from gpt_neox_amd.positional_embeddings import _rotary_torch
+
+            def mask_func(scores, mask_):
+                return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+
+            def timed(fn, n, warm=3):
+                m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+                return m
+
+            fused_us = {r["op"]: r["us_per_call"] for r in table}
+            unfused = []
+
+            def softmax_row(label, shape, dt, sc, mask_, keys, n):
+                mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, SoftmaxFusionTypes.none,
+                                            mask_func, True, sc)
+                x = (torch.randn(shape, device=dev, generator=gen(77)) * 8).to(dt)
+                with torch.no_grad():
+                    f_us = timed(lambda: mod(x, mask_), n)
+                xg = x.clone().requires_grad_(True)
+                g = torch.randn(shape, device=dev, generator=gen(78)).to(dt)
+
+                def fb():
+                    mod(xg, mask_).backward(g)
+                    xg.grad = None
+
+                fb_us = timed(fb, n)
+                r = {"op": label + ": unfused torch branch", "fwd_us": round(f_us, 1), "fwd_bwd_us": round(fb_us, 1)}
+                have = [fused_us.get(k) for k in keys]
+                if have[0] is not None:
+                    r["fused_fwd_us"] = have[0]
+                    r["fwd_speedup"] = round(f_us / have[0], 1)
+                    if len(have) > 1 and have[1] is not None:
+                        r["fused_fwd_bwd_us"] = round(have[0] + have[1], 2)
+                        r["fwd_bwd_speedup"] = round(fb_us / (have[0] + have[1]), 1)
+                unfused.append(r)
+
+            if not args.quick:
+                lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(79))
+                pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+                softmax_row("cfg2 padded [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale, pad,
+                            ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 20)
+                softmax_row("cfg4 causal [1,64,2048,2048] fp16", (1, 64, 2048, 2048), torch.float16, 96 ** -0.5, causal_mask(2048),
+                            ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 20)
+                torch.cuda.empty_cache()
+                softmax_row("cfg5 causal [1,32,8192,8192] bf16", (1, 32, 8192, 8192), torch.bfloat16, 128 ** -0.5, causal_mask(8192),
+                            ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 5)
+                torch.cuda.empty_cache()
+                # partial rotary as the attention layer does it: slice, rotate, concatenate (forward)
+                S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+                t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1246, nsets=1)[0]
+                cos4 = t["cos"].view(S, 1, 1, DR).bfloat16()
+                sin4 = t["sin"].view(S, 1, 1, DR).bfloat16()
+
+                def layer_rotary():
+                    q_rot, q_pass = t["q"][..., :DR], t["q"][..., DR:]
+                    k_rot, k_pass = t["k"][..., :DR], t["k"][..., DR:]
+                    q2, k2 = _rotary_torch(q_rot, k_rot, cos4, sin4, 0)
+                    return torch.cat((q2, q_pass), dim=-1), torch.cat((k2, k_pass), dim=-1)
+
+                with torch.no_grad():
+                    r_us = timed(layer_rotary, 50)
+                r = {"op": "cfg3 partial rotary q+k [2048,4,32,128] bf16: slice + torch expression + cat",
+                     "fwd_us": round(r_us, 1)}
+                have = fused_us.get("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32")
+                if have is not None:
+                    r["fused_fwd_us"] = have
+                    r["fwd_speedup"] = round(r_us / have, 1)
+                unfused.append(r)
+                del t
+            result["unfused_reference_branches_on_this_gpu"] = unfused
         # what the memory pattern of the partial rotary costs by itself: the first 64 of every 256
         # bytes of a 134 MB buffer loaded and stored back (cfg3's q and k), and the same number of
         # bytes as one contiguous run
