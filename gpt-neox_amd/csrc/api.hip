@@ -176,7 +176,7 @@ struct SoftmaxCall {
     // outside its range of row lengths) those go to `fn`'s element-wise kernels.
     int launch(Launcher fn, Mask m, void* stream, Launcher ragged = nullptr) const {
         const bool vec = vec_ok && a.sk % kVec == 0;
-        if (!vec && ragged != nullptr && a.sk >= kVec && a.sk <= kMaxRegisterRow) fn = ragged;
+        if (!vec && ragged != nullptr && a.sk >= kVec && a.sk < kMaxRegisterRow) fn = ragged;
         return check_launch(fn(a, m, dtype, vec, (hipStream_t)stream), what);
     }
 

@@ -152,10 +152,15 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
 
 template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
-    const int chunks = (a.sk + kChunk - 1) / kChunk;
+    int chunks = (a.sk + kChunk - 1) / kChunk;
     if constexpr ((EXTRA & kRagged) != 0) {
         // rows at any alignment: the packed kernels up to 512 columns, the row kernels below beyond
-        if (a.sk < kVec || a.sk > kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+        if (a.sk < kVec || a.sk >= kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+        if (chunks > 1) {
+            // rows of odd length: the row kernels lay those that start on an odd element one
+            // position later on their lanes
+            chunks = (a.sk + (a.sk & 1) + kChunk - 1) / kChunk;
+        }
         if (chunks == 1) {
             const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
                                 (a.bias == nullptr || a.bias_bytes != 0);

@@ -63,48 +63,78 @@ constexpr int kBias = 16;
 // starts wherever the previous one ends.  128-bit buffer accesses work at any alignment on
 // gfx950 and their range check acts per dword: against a buffer of exactly the row's bytes,
 // every dword inside the row is transferred and only a dword that crosses the row end is
-// dropped.  For 16-bit data that is the last element of an odd-length row, which these kernels
-// move by a 16-bit access of its own; for the mask bytes it is the last len % 4 bytes, fetched
-// again by a dword load that ends with the row.  With kDropout a lane's 8 columns straddle two
-// Philox groups (the pattern is a function of the row-major element index).
+// dropped.  For 16-bit data that is one element, which these kernels move by a 16-bit access of
+// its own; for the mask bytes it is up to three, fetched again by a dword load that ends with the
+// row.  Accesses that are not even dword-aligned cost 10-20 % of the bandwidth, though, so a row
+// that starts on an odd element is laid over the lanes one element later (sh = 1): lane l of a
+// chunk then holds the columns 8l - 1 .. 8l + 6 and all its accesses are dword-aligned; only the
+// first lane of the row, whose access would begin in front of the row, takes its seven columns by
+// a 16-bit and a 96-bit access.  "Positions" below are columns + sh: the row occupies the
+// positions [sh, len + sh).  With kDropout a lane's 8 columns straddle two Philox groups (the
+// pattern is a function of the row-major element index).
 constexpr int kRagged = 32;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
 constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;  // a byte offset no buffer contains
 
-// kRagged: the element at column len - 1 of an odd-length row, fetched by every lane of the
-// wave in one broadcast access (no access when len is even).
-__device__ __forceinline__ uint32_t ragged_tail16(rsrc_t r, int len) {
-    return buf_ld16(r, (len & 1) ? (uint32_t)(len - 1) * 2u : kOutOfRange);
+// kRagged: 1 if the row starts on an odd element (2 mod 4 bytes) of the tensor at `base` and sk is
+// odd, so that rows alternate between the two alignments.  (With an even sk every row has the
+// alignment of the tensor; moving them all would only cost a chunk.)  Row-uniform.
+__device__ __forceinline__ int ragged_shift(const void* base, uint32_t row, int sk) {
+    if ((sk & 1) == 0) return 0;
+    return (int)(((reinterpret_cast<uintptr_t>(base) >> 1) + row) & 1u);  // row * sk has the parity of row
 }
-// kRagged: the lane whose 8 columns (from `col`) hold column len - 1 of an odd-length row puts
-// `tail` where the range check left a zero dword.
-__device__ __forceinline__ void ragged_patch16(u32x4& raw, int col, int len, uint32_t tail) {
-    const int e = len - 1 - col;  // even: len is odd, col a multiple of 8
-    if ((len & 1) && e >= 0 && e < 8) {
+// kRagged: the last element of a row of `len` columns when the dword that holds it crosses the
+// row end (len + sh odd), fetched by every lane of the wave in one broadcast access.
+__device__ __forceinline__ uint32_t ragged_tail16(rsrc_t r, int len, int sh) {
+    return buf_ld16(r, ((len + sh) & 1) ? (uint32_t)(len - 1) * 2u : kOutOfRange);
+}
+// kRagged: the lane whose 8 positions (from `pos0`) hold the last one, plen - 1, puts `tail`
+// where the range check left a zero dword (plen = len + sh, odd).
+__device__ __forceinline__ void ragged_patch16(u32x4& raw, int pos0, int plen, uint32_t tail) {
+    const int e = plen - 1 - pos0;  // even: plen is odd, pos0 a multiple of 8
+    if ((plen & 1) && e >= 0 && e < 8) {
         raw.x = (e == 0) ? tail : raw.x;
         raw.y = (e == 2) ? tail : raw.y;
         raw.z = (e == 4) ? tail : raw.z;
         raw.w = (e == 6) ? tail : raw.w;
     }
 }
-// kRagged: the last len % 4 mask bytes of a row (len >= 4), in the low bytes of the result.
-__device__ __forceinline__ uint32_t ragged_tail_mask(rsrc_t rm, int len) {
-    const uint32_t last4 = buf_ld32(rm, (len & 3) ? (uint32_t)(len - 4) : kOutOfRange);
-    return (len & 3) ? last4 >> (8 * (4 - (len & 3))) : 0u;
+// kRagged: the last (len + sh) % 4 mask bytes of a row (len >= 4), in the low bytes of the result:
+// the bytes of the dword that crosses the row end.
+__device__ __forceinline__ uint32_t ragged_tail_mask(rsrc_t rm, int len, int sh) {
+    const int n = (len + sh) & 3;
+    const uint32_t last4 = buf_ld32(rm, n ? (uint32_t)(len - 4) : kOutOfRange);
+    return n ? last4 >> (8 * (4 - n)) : 0u;
 }
-__device__ __forceinline__ void ragged_patch_mask(u32x2& mk, int col, int len, uint32_t tail) {
-    const int e = (len & ~3) - col;  // first dropped byte, relative to the lane's 8 bytes
-    if ((len & 3) && e >= 0 && e < 8) {
+__device__ __forceinline__ void ragged_patch_mask(u32x2& mk, int pos0, int plen, uint32_t tail) {
+    const int e = (plen & ~3) - pos0;  // first dropped byte, relative to the lane's 8 bytes
+    if ((plen & 3) && e >= 0 && e < 8) {
         mk.x = (e == 0) ? tail : mk.x;
         mk.y = (e == 4) ? tail : mk.y;
     }
 }
-// kRagged: 16-bit store of element sk - 1 of an odd-length row from the packed vector that holds it.
-__device__ __forceinline__ void ragged_store16(rsrc_t r, const u32x4& o, int col, int sk) {
-    const int e = sk - 1 - col;
-    const bool own = (sk & 1) && e >= 0 && e < 8;
+// kRagged: 16-bit store of the last element of a row (byte offset `last_off`) from the packed
+// vector that holds its position plen - 1, when its dword crosses the row end (plen odd).
+__device__ __forceinline__ void ragged_store16(rsrc_t r, const u32x4& o, int pos0, int plen, uint32_t last_off) {
+    const int e = plen - 1 - pos0;
+    const bool own = (plen & 1) && e >= 0 && e < 8;
     const uint32_t v = (e == 0) ? o.x : (e == 2) ? o.y : (e == 4) ? o.z : o.w;
-    buf_st16(r, v, own ? (uint32_t)(sk - 1) * 2u : kOutOfRange);
+    buf_st16(r, v, own ? last_off : kOutOfRange);
+}
+// kRagged, sh = 1: the first lane of a row holds the columns 0 .. 6 in its positions 1 .. 7.
+__device__ __forceinline__ u32x4 ragged_head_load(rsrc_t r, bool first_lane) {
+    const uint32_t h = buf_ld16(r, first_lane ? 0u : kOutOfRange);
+    const u32x3 t = buf_ld96(r, first_lane ? 2u : kOutOfRange);
+    return u32x4{h << 16, t.x, t.y, t.z};
+}
+__device__ __forceinline__ void ragged_head_store(rsrc_t r, const u32x4& o, bool first_lane) {
+    buf_st16(r, o.x >> 16, first_lane ? 0u : kOutOfRange);
+    buf_st96(r, u32x3{o.y, o.z, o.w}, first_lane ? 2u : kOutOfRange);
+}
+// kRagged, sh = 1: the first lane's mask bytes for the columns 0 .. 6, in the bytes 1 .. 7.
+__device__ __forceinline__ u32x2 ragged_head_mask(rsrc_t rm, bool first_lane) {
+    const u32x2 m = buf_ld64(rm, first_lane ? 0u : kOutOfRange, 0);
+    return u32x2{m.x << 8, (m.y << 8) | (m.x >> 24)};
 }
 
 // Row of the bias tensor that belongs to score row `row`
@@ -125,10 +155,12 @@ __device__ __forceinline__ uint32_t keep_bits_row8(const DropoutArgs& d, uint32_
     if constexpr (!RAG) {
         return keep_bits8(d, drop_group(row, sk, col));
     } else {
-        const uint64_t e = (uint64_t)row * (uint32_t)sk + (uint32_t)col;
+        // col may be -1 (the position in front of a row that starts on an odd element)
+        const int64_t e = (int64_t)row * sk + col;
         const uint32_t shift = (uint32_t)e & 7u;
-        uint32_t bits = keep_bits8(d, e >> 3) >> shift;
-        if (shift != 0) bits |= keep_bits8(d, (e >> 3) + 1) << (8u - shift);
+        const uint64_t group = (uint64_t)(e >> 3);  // arithmetic shift: -1 for e = -1, whose bits nobody uses
+        uint32_t bits = keep_bits8(d, group) >> shift;
+        if (shift != 0) bits |= keep_bits8(d, group + 1) << (8u - shift);
         return bits & 0xffu;
     }
 }
@@ -194,9 +226,13 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     const float ninf = -__builtin_inff();
     // byte offset of the lane inside the row, first chunk of its wave.  Everything goes into
     // the per-lane offset: the hardware's range check does not see the scalar offset operand.
-    const int voff = lane * 16 + wir * kChunk * 2;
-
     const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    // kRagged: the row lies one position later on the lanes when it starts on an odd element
+    int sh = 0;
+    if constexpr (kRag) sh = ragged_shift(a.in0, pos.row, sk);
+    const int voff = lane * 16 + wir * kChunk * 2 - 2 * sh;
+    const bool head = kRag && sh != 0 && wir == 0;  // wave-uniform: this wave holds the row start
+    const bool first_lane = head && lane == 0;      // its first access would begin in front of the row
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     // ALiBi: scale*(x + slope*(j - i)) = x*scale + slope2*(j - i), slope2 wave-uniform
@@ -213,38 +249,55 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         const uint32_t row_bytes = (uint32_t)(kRag ? pos.len : (pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
         const rsrc_t rx = make_rsrc(x, row_bytes);
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) raw[c] = buf_ld128<kLdNt>(rx, voff + c * WPR * kChunk * 2, 0);
-        if constexpr (kRag) tail_x = ragged_tail16(rx, pos.len);
+        for (int c = 0; c < NCH; ++c)
+            raw[c] = buf_ld128<kLdNt>(rx, (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
+        if constexpr (kRag) {
+            tail_x = ragged_tail16(rx, pos.len, sh);
+            if (head) raw[0] |= ragged_head_load(rx, first_lane);
+        }
         if constexpr ((FLAGS & kBias) != 0) {
             const rsrc_t rb = make_rsrc(static_cast<const char*>(a.bias) + (size_t)bias_row(pos.row, a) * sk * 2, row_bytes);
 #pragma unroll
-            for (int c = 0; c < NCH; ++c) rawb[c] = buf_ld128<false>(rb, voff + c * WPR * kChunk * 2, 0);
-            if constexpr (kRag) tail_b = ragged_tail16(rb, pos.len);
+            for (int c = 0; c < NCH; ++c)
+                rawb[c] = buf_ld128<false>(rb, (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
+            if constexpr (kRag) {
+                tail_b = ragged_tail16(rb, pos.len, sh);
+                if (head) rawb[0] |= ragged_head_load(rb, first_lane);
+            }
         }
         if constexpr (MASK == Mask::Bytes) {
             const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
             const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)pos.len);
 #pragma unroll
-            for (int c = 0; c < NCH; ++c) mk[c] = buf_ld64(rm, lane * 8 + (wir + c * WPR) * kChunk, 0);
-            if constexpr (kRag) tail_m = ragged_tail_mask(rm, pos.len);
+            for (int c = 0; c < NCH; ++c)
+                mk[c] = buf_ld64(rm, (c == 0 && first_lane) ? kOutOfRange : lane * 8 + (wir + c * WPR) * kChunk - sh, 0);
+            if constexpr (kRag) {
+                tail_m = ragged_tail_mask(rm, pos.len, sh);
+                if (head) {
+                    const u32x2 hm = ragged_head_mask(rm, first_lane);
+                    mk[0].x |= hm.x;
+                    mk[0].y |= hm.y;
+                }
+            }
         }
     }
     {
         const int len = pos.len;
+        const int plen = len + sh;  // the row's columns lie at the positions [sh, plen)
         float v[NCH][8];
 
         // ---- scale, mask, running maximum
         float mx = ninf;
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;  // first column of the chunk (wave-uniform)
-            if (c0 < len) {
-                const int col = c0 + lane * kVec;
+            const int c0 = (wir + WPR * c) * kChunk;  // first position of the chunk (wave-uniform)
+            if (c0 < plen) {
+                const int col = c0 + lane * kVec - sh;  // first column of the lane, -1 in front of the row
                 if constexpr (kRag) {
-                    if (c0 + kChunk >= len) {  // the chunk that holds the row end
-                        ragged_patch16(raw[c], col, len, tail_x);
-                        if constexpr ((FLAGS & kBias) != 0) ragged_patch16(rawb[c], col, len, tail_b);
-                        if constexpr (MASK == Mask::Bytes) ragged_patch_mask(mk[c], col, len, tail_m);
+                    if (c0 + kChunk >= plen) {  // the chunk that holds the row end
+                        ragged_patch16(raw[c], c0 + lane * kVec, plen, tail_x);
+                        if constexpr ((FLAGS & kBias) != 0) ragged_patch16(rawb[c], c0 + lane * kVec, plen, tail_b);
+                        if constexpr (MASK == Mask::Bytes) ragged_patch_mask(mk[c], c0 + lane * kVec, plen, tail_m);
                     }
                 }
                 unpack8<T>(raw[c], v[c]);
@@ -254,7 +307,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
                     for (int k = 0; k < 8; ++k) v[c][k] += bv[k];
                 }
-                bool plain = (c0 + kChunk <= len);  // no lane of the wave crosses the row end
+                // no lane of the wave crosses the row end (or holds the position in front of the row)
+                bool plain = (c0 + kChunk <= plen) && !(head && c == 0);
                 if constexpr (MASK == Mask::Bytes) {
                     plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
                 }
@@ -274,6 +328,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         bool keep = (col + k) < len;
+                        if constexpr (kRag) keep = keep && (col + k) >= 0;
                         if constexpr (MASK == Mask::Bytes) {
                             const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
                             keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
@@ -292,7 +347,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
-            if (c0 < len) {
+            if (c0 < plen) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     v[c][k] = fast_exp2(v[c][k] - mx);
@@ -307,10 +362,10 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 sum = 0.f;
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
-                    const int col = (wir + WPR * c) * kChunk + lane * kVec;
+                    const int col = (wir + WPR * c) * kChunk + lane * kVec - sh;
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
-                        v[c][k] = ((col + k) < len) ? 1.f : 0.f;
+                        v[c][k] = ((col + k) < len && (col + k) >= 0) ? 1.f : 0.f;
                         sum += v[c][k];
                     }
                 }
@@ -332,14 +387,16 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             o[c] = u32x4{0, 0, 0, 0};
-            if (c0 < len) {
+            if (c0 < plen) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) v[c][k] *= inv;
                 o[c] = pack8<T>(v[c]);
             }
-            buf_st128<kStNt>(ry, o[c], voff + c * WPR * kChunk * 2, 0);
+            buf_st128<kStNt>(ry, o[c], (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
             if constexpr (kRag) {
-                if (c0 < sk && c0 + kChunk >= sk) ragged_store16(ry, o[c], c0 + lane * kVec, sk);
+                if (c == 0 && head) ragged_head_store(ry, o[c], first_lane);
+                if (c0 < sk + sh && c0 + kChunk >= sk + sh)
+                    ragged_store16(ry, o[c], c0 + lane * kVec, sk + sh, (uint32_t)(sk - 1) * 2u);
             }
         }
         if constexpr ((FLAGS & kDropout) != 0) {
@@ -348,13 +405,15 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
             for (int c = 0; c < NCH; ++c) {
                 const int c0 = (wir + WPR * c) * kChunk;
                 u32x4 o2 = u32x4{0, 0, 0, 0};
-                if (c0 < len) {
-                    const uint32_t bits = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec);
+                if (c0 < plen) {
+                    const uint32_t bits = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec - sh);
                     o2 = dropout8<T>(o[c], bits, drop.scale);
                 }
-                buf_st128<kStNt>(ry2, o2, voff + c * WPR * kChunk * 2, 0);
+                buf_st128<kStNt>(ry2, o2, (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
                 if constexpr (kRag) {
-                    if (c0 < sk && c0 + kChunk >= sk) ragged_store16(ry2, o2, c0 + lane * kVec, sk);
+                    if (c == 0 && head) ragged_head_store(ry2, o2, first_lane);
+                    if (c0 < sk + sh && c0 + kChunk >= sk + sh)
+                        ragged_store16(ry2, o2, c0 + lane * kVec, sk + sh, (uint32_t)(sk - 1) * 2u);
                 }
             }
         }
@@ -375,9 +434,14 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     const int rib = wib / WPR;
     const int wir = wib % WPR;
     const int sk = a.sk;
-    const int voff = lane * 16 + wir * kChunk * 2;  // the range check ignores a scalar offset
-
     const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    // kRagged: the row lies one position later on the lanes when it starts on an odd element; the
+    // position in front of it stays zero in both tensors and is never stored
+    int sh = 0;
+    if constexpr (kRag) sh = ragged_shift(a.in0, pos.row, sk);
+    const int voff = lane * 16 + wir * kChunk * 2 - 2 * sh;  // the range check ignores a scalar offset
+    const bool head = kRag && sh != 0 && wir == 0;  // wave-uniform: this wave holds the row start
+    const bool first_lane = head && lane == 0;      // its first access would begin in front of the row
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     u32x4 rg[NCH], rp[NCH];
@@ -388,17 +452,23 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            rg[c] = buf_ld128<kLdNt>(bg, voff + c * WPR * kChunk * 2, 0);
-            rp[c] = buf_ld128<kLdNt>(by, voff + c * WPR * kChunk * 2, 0);
+            const uint32_t off = (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2;
+            rg[c] = buf_ld128<kLdNt>(bg, off, 0);
+            rp[c] = buf_ld128<kLdNt>(by, off, 0);
         }
         if constexpr (kRag) {
-            tail_g = ragged_tail16(bg, pos.len);
-            tail_p = ragged_tail16(by, pos.len);
+            tail_g = ragged_tail16(bg, pos.len, sh);
+            tail_p = ragged_tail16(by, pos.len, sh);
+            if (head) {
+                rg[0] |= ragged_head_load(bg, first_lane);
+                rp[0] |= ragged_head_load(by, first_lane);
+            }
         }
     }
     {
         // dx may alias dy: a row is read and written by the same waves only, reads first
         const int len = pos.len;
+        const int plen = len + sh;  // the row's columns lie at the positions [sh, plen)
 
         // the row stays packed; it is unpacked once for the dot product and once for dx
         float dot = 0.f;
@@ -407,23 +477,23 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             kb[c] = 0xffu;
-            if (c0 < len) {
-                const int col = c0 + lane * kVec;
+            if (c0 < plen) {
+                const int col = c0 + lane * kVec - sh;  // first column of the lane
                 if constexpr (kRag) {
-                    if (c0 + kChunk >= len) {  // the chunk that holds the row end
-                        ragged_patch16(rg[c], col, len, tail_g);
-                        ragged_patch16(rp[c], col, len, tail_p);
+                    if (c0 + kChunk >= plen) {  // the chunk that holds the row end
+                        ragged_patch16(rg[c], c0 + lane * kVec, plen, tail_g);
+                        ragged_patch16(rp[c], c0 + lane * kVec, plen, tail_p);
                     }
                 }
                 float gv[8], pv[8];
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
                 if constexpr ((FLAGS & kDropout) != 0) {
-                    kb[c] = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec);
+                    kb[c] = keep_bits_row8<kRag>(drop, pos.row, sk, col);
 #pragma unroll
                     for (int k = 0; k < 8; ++k) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 }
-                if (c0 + kChunk > len) {
+                if (c0 + kChunk > plen) {
                     // the lane holding the diagonal may have loaded columns past it
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
@@ -442,22 +512,24 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             u32x4 o = u32x4{0, 0, 0, 0};
-            if (c0 < len) {
+            if (c0 < plen) {
                 float gv[8], pv[8];
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
-                const int col = c0 + lane * kVec;
+                const int col = c0 + lane * kVec - sh;
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                     gv[k] = a.scale * (pv[k] * (gv[k] - dot));
-                    if ((c0 + kChunk > len) && (col + k) >= len) gv[k] = 0.f;
+                    if ((c0 + kChunk > plen) && (col + k) >= len) gv[k] = 0.f;
                 }
                 o = pack8<T>(gv);
             }
-            buf_st128<kStNt>(rdx, o, voff + c * WPR * kChunk * 2, 0);
+            buf_st128<kStNt>(rdx, o, (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
             if constexpr (kRag) {
-                if (c0 < sk && c0 + kChunk >= sk) ragged_store16(rdx, o, c0 + lane * kVec, sk);
+                if (c == 0 && head) ragged_head_store(rdx, o, first_lane);
+                if (c0 < sk + sh && c0 + kChunk >= sk + sh)
+                    ragged_store16(rdx, o, c0 + lane * kVec, sk + sh, (uint32_t)(sk - 1) * 2u);
             }
         }
     }

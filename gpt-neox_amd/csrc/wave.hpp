@@ -133,6 +133,13 @@ __device__ __forceinline__ uint32_t buf_ld32(rsrc_t r, int voffset) {
 __device__ __forceinline__ uint32_t buf_ld16(rsrc_t r, int voffset) {
     return __builtin_amdgcn_raw_buffer_load_b16(r, voffset, 0, 0);
 }
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+__device__ __forceinline__ u32x3 buf_ld96(rsrc_t r, int voffset) {
+    return __builtin_amdgcn_raw_buffer_load_b96(r, voffset, 0, 0);
+}
+__device__ __forceinline__ void buf_st96(rsrc_t r, const u32x3& v, int voffset) {
+    __builtin_amdgcn_raw_buffer_store_b96(v, r, voffset, 0, 0);
+}
 __device__ __forceinline__ uint32_t buf_ld8(rsrc_t r, int voffset) {
     return __builtin_amdgcn_raw_buffer_load_b8(r, voffset, 0, 0);
 }
