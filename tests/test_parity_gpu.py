@@ -1176,3 +1176,29 @@ def test_ragged_short_rows_every_row_end_and_group_size(device):
             mask[1, 0, 3, sk - r:] = False               # ... and those alone visible
             check_masked(device, 2, 3, 5, sk, dtype, 0.25, seed=sk, mask=mask)
             check_masked(device, 2, 3, 5, sk, dtype, 0.25, seed=sk, mask=mask[:1])
+
+
+def test_module_through_a_generation_loop_at_arbitrary_lengths(device):
+    # a prefill at an odd prompt length (causal kernel), then single-token steps against a growing
+    # key/value cache (mask-tensor kernel): the fused module against its own unfused branch
+    b, heads = 2, 4
+    for dtype in DTYPES:
+        fused = FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, SoftmaxFusionTypes.upper_triang,
+                                      R.gpt2_attention_mask_func, True, 0.125)
+        plain = FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, SoftmaxFusionTypes.none,
+                                      R.gpt2_attention_mask_func, True, 0.125)
+        for prompt in (37, 1001, 1537):
+            full_mask = R.get_attn_mask(prompt + 6, device)
+            x = scores((b, heads, prompt, prompt), dtype, device, prompt)
+            mask = full_mask[..., :prompt, :prompt].contiguous()
+            with torch.no_grad():
+                assert max_err(fused(x, mask), plain(x.clone(), mask)) <= 2 * TOL[dtype]
+                for t in range(prompt + 1, prompt + 6):
+                    x = scores((b, heads, 1, t), dtype, device, t)
+                    # the layer's slice of the mask for one query at position t - 1
+                    # (megatron/model/transformer.py:514-524)
+                    step_mask = full_mask[..., t - 1, :t].unsqueeze(2).contiguous()
+                    assert fused.is_kernel_available(step_mask, b, heads, 1, t)
+                    y = fused(x, step_mask)
+                    assert max_err(y, plain(x.clone(), step_mask)) <= 2 * TOL[dtype]
+                    assert torch.allclose(y.float().sum(-1), torch.ones(b, heads, 1, device=device), atol=2e-2)
