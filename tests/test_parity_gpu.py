@@ -1195,8 +1195,7 @@ def test_module_through_a_generation_loop_at_arbitrary_lengths(device):
                 assert max_err(fused(x, mask), plain(x.clone(), mask)) <= 2 * TOL[dtype]
                 for t in range(prompt + 1, prompt + 6):
                     x = scores((b, heads, 1, t), dtype, device, t)
-                    # the layer's slice of the mask for one query at position t - 1
-                    # (megatron/model/transformer.py:514-524)
+                    # the mask row of the one query, at position t - 1, against the t cached keys
                     step_mask = full_mask[..., t - 1, :t].unsqueeze(2).contiguous()
                     assert fused.is_kernel_available(step_mask, b, heads, 1, t)
                     y = fused(x, step_mask)
