@@ -546,19 +546,78 @@ def test_dropout_function_gradient_reaches_the_bias(device, shared):
         assert max_err(bias.grad, br.grad) <= tol * max(1.0, br.grad.abs().max().item()) * (b if shared else 1)
 
 
-def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
-    # any row length (mostly not a multiple of 8), tensors starting at a random element of their
-    # allocation, and a random choice of mask kind, bias / ALiBi and dropout: every result against
-    # the oracle's fp32 expressions with the kernels' own keep pattern
-    import random
-
-    rnd = random.Random(20250101)
+def check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, shift, case):
+    """One call of the kernels with the given mask kind (causal / random mask bytes), optional bias
+    tensor ("bias", "shared bias") or ALiBi slopes ("alibi"), dropout probability p and every tensor
+    starting `shift` elements into its allocation: forward and backward against the oracle's fp32
+    expressions, with the kernels' own keep pattern."""
 
     def shifted(t, by):
         flat = torch.empty(t.numel() + by, dtype=t.dtype, device=device)
         flat[by:] = t.reshape(-1)
         return flat[by:].view(t.shape)
 
+    tag = (case, str(dtype), causal, b, heads, sq, sk, scale, p, extra, shift)
+    x = shifted(scores((b, heads, sq, sk), dtype, device, case), shift)
+    g = shifted(normal((b, heads, sq, sk), dtype, device, 1000 + case), shift)
+    bias = slopes = None
+    logits = x.float()
+    if "bias" in extra:
+        bias = shifted(normal((1 if extra == "shared bias" else b, heads, sq, sk), dtype, device, 2000 + case), shift)
+        logits = logits + bias.float()
+    if extra == "alibi":
+        slopes = torch.rand(heads, device=device, generator=gen(device, case)) * 0.5
+        logits = logits + R.alibi_bias_fp32(slopes.cpu(), sq, sk).to(device)
+    if causal:
+        mask = R.get_attn_mask(sk, device)
+    else:
+        mask = torch.rand(1 if case % 2 else b, 1, sq, sk, device=device, generator=gen(device, 3000 + case)) < 0.3
+        mask = shifted(mask, shift)
+    want = R.softmax_fp32(logits, mask, scale)
+    del logits
+    seed, offset = 77 + case, 4 * case
+    if p == 0.0:
+        if causal:
+            if slopes is not None:
+                y = causal_ext.forward_alibi(x, slopes, scale)
+            elif bias is not None:
+                y = causal_ext.forward_bias(x, bias, scale)
+            else:
+                y = causal_ext.forward(x.view(-1, sq, sk), scale).view(x.shape)
+            dx = causal_ext.backward(g.clone().view(-1, sq, sk), y.view(-1, sq, sk), scale).view(x.shape)
+        else:
+            y = masked_ext.forward_bias(x, mask, bias, scale) if bias is not None else masked_ext.forward(x, mask, scale)
+            dx = masked_ext.backward(g.clone(), y, scale)
+        want_dx = R.softmax_backward_fp32(g, y, scale)
+    else:
+        if causal:
+            y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
+            dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+        else:
+            y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
+            dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
+        keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
+        if y.numel() <= 1 << 20:
+            assert np.array_equal(keep.cpu().numpy().reshape(-1), philox.keep_mask(y.numel(), p, seed, offset)), tag
+        assert torch.equal(dropped, R.dropout_with_mask(y, keep, p)), tag
+        want_dx = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
+    assert max_err(y, want) <= TOL[dtype], tag
+    hidden = mask.expand_as(y)
+    full_rows = hidden.all(-1, keepdim=True).expand_as(y)
+    assert (y[hidden & ~full_rows] == 0).all(), tag
+    # the bound scales with the largest gradient and allows for the rounding of values above 1
+    top = want_dx.abs().max().item()
+    half_ulp = top * (2.0**-8 if dtype == torch.bfloat16 else 2.0**-11)
+    assert max_err(dx, want_dx) <= TOL[dtype] * max(1.0, top) + half_ulp, tag
+    assert (dx[hidden & ~full_rows] == 0).all(), tag
+
+
+def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
+    # any row length (mostly not a multiple of 8), tensors starting at a random element of their
+    # allocation, and a random choice of mask kind, bias / ALiBi and dropout
+    import random
+
+    rnd = random.Random(20250101)
     for case in range(60):
         dtype = rnd.choice(DTYPES)
         sk = rnd.choice([rnd.randint(8, 70), rnd.randint(71, 520), rnd.randint(521, 2100), rnd.randint(2101, 9000)])
@@ -572,56 +631,32 @@ def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
         extra = rnd.choice(["none", "none", "bias", "shared bias", "alibi"])
         if extra == "alibi" and not causal:
             extra = "none"
-        shift = rnd.randint(0, 9)
-        tag = (case, str(dtype), causal, b, heads, sq, sk, scale, p, extra, shift)
-        x = shifted(scores((b, heads, sq, sk), dtype, device, case), shift)
-        g = shifted(normal((b, heads, sq, sk), dtype, device, 1000 + case), shift)
-        bias = slopes = None
-        logits = x.float()
-        if "bias" in extra:
-            bias = shifted(normal((1 if extra == "shared bias" else b, heads, sq, sk), dtype, device, 2000 + case), shift)
-            logits = logits + bias.float()
-        if extra == "alibi":
-            slopes = torch.rand(heads, device=device, generator=gen(device, case)) * 0.5
-            logits = logits + R.alibi_bias_fp32(slopes.cpu(), sq, sk).to(device)
-        if causal:
-            mask = R.get_attn_mask(sk, device)
-        else:
-            mask = torch.rand(rnd.choice([1, b]), 1, sq, sk, device=device, generator=gen(device, 3000 + case)) < 0.3
-            mask = shifted(mask, shift)
-        want = R.softmax_fp32(logits, mask, scale)
-        seed, offset = 77 + case, 4 * case
-        if p == 0.0:
-            if causal:
-                if slopes is not None:
-                    y = causal_ext.forward_alibi(x, slopes, scale)
-                elif bias is not None:
-                    y = causal_ext.forward_bias(x, bias, scale)
-                else:
-                    y = causal_ext.forward(x.view(-1, sq, sk), scale).view(x.shape)
-                dx = causal_ext.backward(g.clone().view(-1, sq, sk), y.view(-1, sq, sk), scale).view(x.shape)
-            else:
-                y = masked_ext.forward_bias(x, mask, bias, scale) if bias is not None else masked_ext.forward(x, mask, scale)
-                dx = masked_ext.backward(g.clone(), y, scale)
-            want_dx = R.softmax_backward_fp32(g, y, scale)
-        else:
-            if causal:
-                y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
-                dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
-            else:
-                y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
-                dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
-            keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
-            if y.numel() <= 1 << 20:
-                assert np.array_equal(keep.cpu().numpy().reshape(-1), philox.keep_mask(y.numel(), p, seed, offset)), tag
-            assert torch.equal(dropped, R.dropout_with_mask(y, keep, p)), tag
-            want_dx = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
-        assert max_err(y, want) <= TOL[dtype], tag
-        hidden = mask.expand_as(y)
-        full_rows = hidden.all(-1, keepdim=True).expand_as(y)
-        assert (y[hidden & ~full_rows] == 0).all(), tag
-        # the bound scales with the largest gradient and allows for the rounding of values above 1
-        top = want_dx.abs().max().item()
-        half_ulp = top * (2.0**-8 if dtype == torch.bfloat16 else 2.0**-11)
-        assert max_err(dx, want_dx) <= TOL[dtype] * max(1.0, top) + half_ulp, tag
-        assert (dx[hidden & ~full_rows] == 0).all(), tag
+        check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, rnd.randint(0, 9), case)
+
+
+# one row length per kernel shape of the dispatcher: lane groups of 1 .. 64 lanes, then 1, 2, 4, 8 and
+# 16 waves per row with 2, 3 or 4 chunks per wave
+SHAPE_LENGTHS = [8, 16, 32, 64, 128, 256, 512, 1024, 1536, 2048, 2560, 4096, 5120, 8192, 10240, 13312, 16384, 20480, 28672]
+
+
+@pytest.mark.parametrize("extra", ["none", "bias", "shared bias", "alibi"])
+@pytest.mark.parametrize("p", [0.0, 0.25])
+def test_every_kernel_shape_with_every_feature_combination(device, extra, p):
+    # each length as it is (aligned rows) and one column shorter (ragged rows of odd length), in
+    # both storage types, through the mask-tensor kernels (three rows) and, up to 4096 columns,
+    # through the causal kernels; beyond that the causal kernels take one parity and one storage
+    # type per length, varying with the feature combination
+    case = 0
+    for n in SHAPE_LENGTHS:
+        for sk in (n, n - 1 if n > 8 else 9):
+            for dtype in DTYPES:
+                case += 1
+                if extra != "alibi":
+                    check_combination(device, dtype, False, 2, 2, 3, sk, 0.25, p, extra, 0, case)
+                if sk <= 4096:
+                    check_combination(device, dtype, True, 1, 2, sk, sk, 0.25, p, extra, 0, 500 + case)
+    variant = ["none", "bias", "shared bias", "alibi"].index(extra) + (1 if p else 0)
+    for i, n in enumerate(n for n in SHAPE_LENGTHS if n > 4096):
+        sk = n - (i + variant) % 2
+        check_combination(device, DTYPES[(i + variant // 2) % 2], True, 1, 1, sk, sk, 0.25, p, extra, 0, 900 + i)
+        torch.cuda.empty_cache()

@@ -1201,3 +1201,70 @@ def test_module_through_a_generation_loop_at_arbitrary_lengths(device):
                     y = fused(x, step_mask)
                     assert max_err(y, plain(x.clone(), step_mask)) <= 2 * TOL[dtype]
                     assert torch.allclose(y.float().sum(-1), torch.ones(b, heads, 1, device=device), atol=2e-2)
+
+
+# ---------------------------------------------------------------------------------
+# kernel variants the cases above do not reach
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("half_tables", [False, True])
+@pytest.mark.parametrize("case", [
+    # rotated spans of more than 64 slots of 8, 4 and 2 dims (the pair-in-lane kernel)
+    (5, 2, 3, 3, 1024, 1024), (4, 2, 2, 2, 1028, 520), (4, 2, 2, 2, 134, 132),
+    # spans of 8-, 4- and 2-dim slots (the span kernel), also backward with half-precision tables
+    (16, 2, 4, 4, 64, 64), (9, 3, 5, 5, 96, 24), (4, 2, 3, 3, 20, 20),
+])
+def test_rotary_slot_widths_table_types_and_directions(device, case, half_tables, dtype):
+    check_rotary(device, *case, dtype, seed=sum(case), table_dtype=dtype if half_tables else torch.float)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_lds_staged_causal_rows_in_both_storage_types(device, dtype):
+    s = 33000
+    x = scores((1, s, s), dtype, device, 7)
+    y = causal_ext.forward(x, 0.05)
+    rows = torch.tensor([0, 1, 700, s // 2, s - 1], device=device)
+    mask = R.get_attn_mask(s, device)[0, 0][rows]
+    assert max_err(y[0][rows], R.softmax_fp32(x[0][rows], mask, 0.05)) <= TOL[dtype]
+    assert (y[0][rows][mask] == 0).all()
+    g = normal((1, s, s), dtype, device, 8)
+    dx = causal_ext.backward(g.clone(), y, 0.05)
+    assert max_err(dx[0][rows], R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sk", [5, 33000])
+def test_bias_tensor_on_the_element_wise_kernels(device, sk, dtype):
+    # rows shorter than 8 columns, and rows beyond the register budget with a bias tensor
+    b, heads, sq = 2, 2, (sk if sk < 8 else 3)
+    x = scores((b, heads, sq, sk), dtype, device, sk)
+    rpe = normal((1, heads, sq, sk), dtype, device, sk + 1)
+    pad = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, sk + 2)) < 0.3
+    pad[..., 0] = False
+    y = masked_ext.forward_bias(x, pad, rpe, 0.25)
+    assert max_err(y, R.softmax_fp32(x.float() + rpe.float(), pad, 0.25)) <= TOL[dtype]
+    assert (y[pad.expand_as(y)] == 0).all()
+    if sk < 8:
+        causal = R.get_attn_mask(sk, device)
+        yc = causal_ext.forward_bias(x, rpe, 0.25)
+        assert max_err(yc, R.softmax_fp32(x.float() + rpe.float(), causal, 0.25)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("offset", [1, 2, 4])
+def test_one_lane_rows_at_any_alignment(device, offset):
+    # sk = 8: one lane per row; the tensors start `offset` elements into their allocations
+    dtype, b, heads, sq, sk = torch.bfloat16, 2, 3, 8, 8
+    flat = torch.empty(b * heads * sq * sk + offset, dtype=dtype, device=device)
+    flat[offset:] = scores((b, heads, sq, sk), dtype, device, offset).reshape(-1)
+    x = flat[offset:].view(b, heads, sq, sk)
+    mask = torch.rand(b, 1, sq, sk, device=device, generator=gen(device, offset)) < 0.3
+    mask[..., 0] = False
+    y = masked_ext.forward(x, mask, 0.5)
+    assert max_err(y, R.softmax_fp32(x, mask, 0.5)) <= TOL[dtype]
+    yc = causal_ext.forward(x.view(-1, sq, sk), 0.5)
+    assert max_err(yc.view(x.shape), R.softmax_fp32(x, R.get_attn_mask(sk, device), 0.5)) <= TOL[dtype]
+    gflat = torch.empty_like(flat)
+    gflat[offset:] = normal((b, heads, sq, sk), dtype, device, offset + 1).reshape(-1)
+    g = gflat[offset:].view(b, heads, sq, sk)
+    want = R.softmax_backward_fp32(g, y, 0.5)
+    assert max_err(masked_ext.backward(g, y, 0.5), want) <= TOL[dtype]
