@@ -1268,3 +1268,38 @@ def test_one_lane_rows_at_any_alignment(device, offset):
     g = gflat[offset:].view(b, heads, sq, sk)
     want = R.softmax_backward_fp32(g, y, 0.5)
     assert max_err(masked_ext.backward(g, y, 0.5), want) <= TOL[dtype]
+    # the same rows with a bias tensor, ALiBi slopes and dropout
+    rpe = normal((1, heads, sq, sk), dtype, device, offset + 2)
+    want_b = R.softmax_fp32(x.float() + rpe.float(), mask, 0.5)
+    assert max_err(masked_ext.forward_bias(x, mask, rpe, 0.5), want_b) <= TOL[dtype]
+    causal = R.get_attn_mask(sk, device)
+    assert max_err(causal_ext.forward_bias(x, rpe, 0.5), R.softmax_fp32(x.float() + rpe.float(), causal, 0.5)) <= TOL[dtype]
+    slopes = torch.tensor([0.5, 0.25, 0.125], device=device)
+    want_a = R.softmax_fp32(x.float() + R.alibi_bias_fp32(slopes.cpu(), sq, sk).to(device), causal, 0.5)
+    assert max_err(causal_ext.forward_alibi(x, slopes, 0.5), want_a) <= TOL[dtype]
+    from gpt_neox_amd.fused_kernels import attention_dropout as rng
+    for fwd, kw in ((lambda **k: masked_ext.forward_dropout(x, mask, 0.5, 0.25, 5, 8, **k), [{}, {"bias": rpe}]),
+                    (lambda **k: causal_ext.forward_dropout(x, 0.5, 0.25, 5, 8, **k), [{}, {"bias": rpe}, {"slopes": slopes}])):
+        for extra in kw:
+            probs, dropped = fwd(**extra)
+            keep = rng.keep_mask(probs.numel(), 0.25, 5, 8, device).view(probs.shape)
+            assert torch.equal(dropped, R.dropout_with_mask(probs, keep, 0.25))
+    probs, _ = masked_ext.forward_dropout(x, mask, 0.5, 0.25, 5, 8)
+    keep = rng.keep_mask(probs.numel(), 0.25, 5, 8, device).view(probs.shape)
+    want_d = R.softmax_dropout_backward_fp32(g, probs, keep, 0.25, 0.5)
+    assert max_err(masked_ext.backward_dropout(g.clone(), probs, 0.5, 0.25, 5, 8), want_d) <= 2 * TOL[dtype]
+    assert max_err(causal_ext.backward_dropout(g.clone(), probs, 0.5, 0.25, 5, 8),
+                   R.softmax_dropout_backward_fp32(g, probs.masked_fill(causal, 0), keep, 0.25, 0.5)) <= 2 * TOL[dtype]
+
+
+def test_measurement_aids_copy_and_strided_touch(device):
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=device)
+    dst = torch.zeros_like(src)
+    _lib.check(lib.neox_copy_bytes(dst.data_ptr(), src.data_ptr(), src.numel() - 16, stream))
+    assert torch.equal(dst[:-16], src[:-16]) and (dst[-16:] == 0).all()
+    before = src.clone()
+    _lib.check(lib.neox_touch_strided(src.data_ptr(), 4096, 64, 256, stream))  # loads and stores back
+    _lib.check(lib.neox_touch_strided(src.data_ptr(), 1, 4096, 4096, stream))
+    assert torch.equal(src, before)
