@@ -1303,3 +1303,39 @@ def test_measurement_aids_copy_and_strided_touch(device):
     _lib.check(lib.neox_touch_strided(src.data_ptr(), 4096, 64, 256, stream))  # loads and stores back
     _lib.check(lib.neox_touch_strided(src.data_ptr(), 1, 4096, 4096, stream))
     assert torch.equal(src, before)
+
+
+def test_mask_and_bias_tensors_beyond_4_gib(device):
+    # short rows whose mask / bias tensor no longer fits a 32-bit buffer: the several-rows-per-wave
+    # kernels step aside for the row kernels, which address every row through its own buffer
+    if torch.cuda.get_device_properties(device).total_memory < 80 << 30:
+        pytest.skip("needs about 40 GiB of device memory")
+    dtype, sk = torch.float16, 512
+    sq = (1 << 23) + 8                      # mask: sq * 512 bytes > 4 GiB; bias: twice that
+    x = torch.empty(1, 1, sq, sk, dtype=dtype, device=device)
+    for lo in range(0, sq, 1 << 20):        # filled in pieces: no full-size fp32 temporary
+        x[0, 0, lo : lo + (1 << 20)] = scores((min(1 << 20, sq - lo), sk), dtype, device, lo)
+    mask = torch.zeros(1, 1, sq, sk, dtype=torch.bool, device=device)
+    rows = torch.tensor([0, 1, 12345, (1 << 22) + 3, (1 << 23) - 1, 1 << 23, sq - 2, sq - 1], device=device)
+    pattern = torch.rand(rows.numel(), sk, device=device, generator=gen(device, 1)) < 0.4
+    pattern[:, 0] = False
+    mask[0, 0, rows] = pattern
+    assert mask.numel() > (1 << 32)
+    y = masked_ext.forward(x, mask, 0.25)
+    assert max_err(y[0, 0, rows], R.softmax_fp32(x[0, 0, rows], pattern, 0.25)) <= TOL[dtype]
+    assert (y[0, 0, rows][pattern] == 0).all()
+    assert torch.allclose(y[0, 0, -4096:].float().sum(-1), torch.ones(4096, device=device), atol=2e-2)
+    bias = torch.zeros(1, 1, sq, sk, dtype=dtype, device=device)
+    bias[0, 0, rows] = normal((rows.numel(), sk), dtype, device, 2)
+    yb = masked_ext.forward_bias(x, mask, bias, 0.25)
+    want = R.softmax_fp32(x[0, 0, rows].float() + bias[0, 0, rows].float(), pattern, 0.25)
+    assert max_err(yb[0, 0, rows], want) <= TOL[dtype]
+    other = torch.tensor([5, (1 << 23) + 5], device=device)  # rows with a zero bias and an empty mask
+    assert torch.equal(yb[0, 0, other], y[0, 0, other])
+    del yb, bias
+    torch.cuda.empty_cache()
+    from gpt_neox_amd.fused_kernels import attention_dropout as rng
+    probs, dropped = masked_ext.forward_dropout(x, mask, 0.25, 0.25, 3, 4)
+    assert torch.equal(probs[0, 0, rows], y[0, 0, rows])
+    keep = rng.keep_mask(probs.numel(), 0.25, 3, 4, device).view(probs.shape)
+    assert torch.equal(dropped[0, 0, rows], R.dropout_with_mask(probs[0, 0, rows], keep[0, 0, rows], 0.25))
