@@ -3,18 +3,21 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table] [--quick] [--only TEXT]
 
-A step is one pass of the hot path over one batch of synthetic input with all
-tensors resident in HBM: the padding-masked scaled softmax forward + backward of
-BASELINE.json's configs[1] ([8, 16, 1024, 1024] fp16, bool mask [8, 1, 1024, 1024],
-scale 0.125, key lengths ~ U[256, 1024]).  K steps are timed after W warm-up
-steps between device synchronisations; the JSON line carries
+A step is one pass of the hot path over one batch of synthetic input with all tensors
+resident in HBM, on the largest single-GPU configuration of BASELINE.json, configs[4]: the
+long-context causal scaled softmax forward + backward on scores [1, 32, 8192, 8192] bf16
+(scale 1/sqrt(128)) plus the full rotary forward + backward on q, k [8192, 1, 32, 128] bf16 --
+four launches.  K steps are timed after W warm-up steps between device synchronisations; the
+JSON line carries
 
-* value       -- algorithmic GB/s of the step (forward + backward bytes / step time);
-* roofline    -- the dominant kernel (the backward) alone: algorithmic bytes per
+* value       -- algorithmic GB/s of the step (bytes of the four launches / step time);
+* min_pct_hbm_peak_over_configs -- the lowest % of HBM peak over every BASELINE shape and op;
+* roofline    -- the step's dominant kernel (the causal backward) alone: algorithmic bytes per
                  launch / mean launch duration of K back-to-back launches between two HIP
-                 events on the launch stream, against the 8 TB/s HBM peak;
+                 events on the launch stream, against the 8 TB/s HBM peak; `traffic` is read
+                 from the counter summary under profiles/ (it cannot be measured live);
 * cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
-                 this host's cores on a slice of the same batch;
+                 this host's cores on 1/32 of the same step;
 * all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak and, as part
                  of the CPU-baseline leg, the oracle's CPU time on a slice scaled to the full
                  shape with the error of the kernel's output on that slice against it (max
@@ -38,10 +41,6 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the dominant kernel (configs[1] backward), from the rocprofv3 counter
-# runs of this same script summarised in profiles/bench_all_configs_hbm_counters.txt:
-# fetched 536.9 MB (TCC_EA0_RDREQ x 128 B) + written 268.4 MB (WRITE_SIZE); cannot be read live.
-MEASURED_TRAFFIC_BWD_BYTES = 805.3e6
 METRIC = "softmax/rotary fwd+bwd achieved GB/s and % of MI355X HBM peak; µs per call"
 
 
@@ -58,6 +57,44 @@ def parse():
     ap.add_argument("--only", type=str, default=None,
                     help="run only the table rows whose name contains this text (profiling aid)")
     return ap.parse_args()
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of a kernel as rocprofv3's counters saw them.  They cannot be read
+    live; the counter runs of this script are summarised in profiles/hbm_traffic_counters.txt,
+    whose lines `TRAFFIC <key> fetched_bytes=.. written_bytes=..` this reads (the file names the
+    commands that produced it).  Without such a line the figure is None."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) >= 4 and parts[0] == "TRAFFIC" and parts[1] == key:
+                    kv = dict(p.split("=", 1) for p in parts[2:] if "=" in p)
+                    fetched, written = float(kv["fetched_bytes"]), float(kv["written_bytes"])
+                    return {"traffic": fetched + written,
+                            "traffic_source": "profiles/hbm_traffic_counters.txt (rocprofv3 --pmc runs of this "
+                                              "script; fetched %.4g B + written %.4g B)" % (fetched, written)}
+    except (OSError, KeyError, ValueError):
+        pass
+    return {"traffic": None, "traffic_source": "no counter summary for this kernel under profiles/"}
+
+
+def load_probes():
+    """libneox_probes.so: the memory-system probes of this benchmark (plain copy, strided touch,
+    empty kernel).  They are not part of the product library."""
+    import ctypes
+
+    path = os.path.join(ROOT, "gpt-neox_amd", "csrc", "libneox_probes.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} not found: run `make -C gpt-neox_amd/csrc`")
+    h = ctypes.CDLL(path)
+    vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+    h.neox_probe_copy.restype, h.neox_probe_copy.argtypes = ctypes.c_int, [vp, vp, i64, vp]
+    h.neox_probe_empty.restype, h.neox_probe_empty.argtypes = ctypes.c_int, [vp]
+    h.neox_probe_strided.restype = ctypes.c_int
+    h.neox_probe_strided.argtypes = [vp, i64, i32, i32, i64, i32, i32, vp]
+    return h
 
 
 def main():
@@ -82,6 +119,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     lib = _lib.lib()  # ImportError if the HIP library is not built
+    probes = load_probes()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream().cuda_stream
@@ -155,7 +193,7 @@ def main():
         # in place over the first d_rot dims of whole heads, q and k in one launch
         ok(lib.neox_rope_apply(t["q"].data_ptr(), t["k"].data_ptr(), t["q"].data_ptr(),
                                t["k"].data_ptr(), t["cos"].data_ptr(), t["sin"].data_ptr(), s, b, h,
-                               h, d_rot, t["st"], t["st"], t["st"], t["st"], d_rot, 0, code[dtype],
+                               h, d_rot, d_rot, t["st"], t["st"], t["st"], t["st"], d_rot, 0, code[dtype],
                                F32, backward, stream))
 
     def time_launches(fn, sets, n_launch, repeats=5, warm=20):
@@ -186,28 +224,41 @@ def main():
         return dict(op=name, bytes=nbytes, us_per_call=round(med_us, 2), best_us=round(min_us, 2),
                     GBps=round(gbps, 1), pct_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 1))
 
-    # ------------------------------------------------------------------ main workload (configs[1])
-    b, heads, sq, sk, dtype, scale = 8, 16, 1024, 1024, torch.float16, 0.125
-    n_elem = b * heads * sq * sk
-    fwd_bytes = 2 * n_elem * 2 + b * sq * sk
-    bwd_bytes = 3 * n_elem * 2
-    sets = masked_sets(b, heads, sq, sk, dtype, 1234 + 1, nsets=3)
+    # ------------------------------------------------------------------ main workload (configs[4])
+    # The largest single-GPU configuration: long-context causal softmax forward + backward on
+    # [1, 32, 8192, 8192] bf16 (scale 1/sqrt(128)) plus the full rotary (rotary_pct 1.0) forward +
+    # backward on q, k [8192, 1, 32, 128] bf16.  A step launches the four kernels in the order a
+    # training step meets them (rotary, softmax, softmax backward, rotary backward).  The score
+    # tensors (4.3 GB each) cannot stay in the 256 MB Infinity Cache; q and k (134 MB) could, so the
+    # rotary launches walk over six buffer sets and the backward launch of a step works on another
+    # set than its forward launch.
+    B5, n5, dt5, sc5 = 32, 8192, torch.bfloat16, 128 ** -0.5
+    S5, H5, HN5 = 8192, 32, 128
+    tri5 = n5 * (n5 + 1) // 2
+    cfwd_bytes = B5 * 2 * (tri5 + n5 * n5)
+    cbwd_bytes = B5 * 2 * (2 * tri5 + n5 * n5)
+    rope_bytes = 2 * 2 * S5 * 1 * H5 * HN5 * 2 + 2 * S5 * HN5 * 4
+    step_bytes = cfwd_bytes + cbwd_bytes + 2 * rope_bytes
+    cset = causal_sets(B5, n5, dt5, 1238, nsets=1, need_bwd=True)[0]
+    rsets = rope_sets(S5, 1, H5, HN5, HN5, dt5, 1239, nsets=6)
 
-    def step(s):
-        masked_fwd(s, b, heads, sq, sk, dtype, scale)
-        masked_bwd(s, b, heads, sq, sk, dtype, scale)
+    def step(i):
+        rope_apply(rsets[i % 6], S5, 1, H5, HN5, dt5, 0)
+        causal_fwd(cset, B5, n5, dt5, sc5)
+        causal_bwd(cset, B5, n5, dt5, sc5)
+        rope_apply(rsets[(i + 3) % 6], S5, 1, H5, HN5, dt5, 1)
 
     for i in range(args.warmup):
-        step(sets[i % len(sets)])
+        step(i)
     torch.cuda.synchronize()
     # the timed region: exactly K steps between two device synchronisations
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(sets[i % len(sets)])
+        step(i)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # each kernel alone: K launches between two HIP events on the launch stream (an event
     # between consecutive launches would add about 2 us of idle time to every launch)
@@ -215,14 +266,16 @@ def main():
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for i in range(args.steps):
-            fn(sets[i % len(sets)], b, heads, sq, sk, dtype, scale)
+            fn(i)
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / args.steps
 
-    fwd_us = launches_us(masked_fwd)
-    bwd_us = launches_us(masked_bwd)
-    bwd_gbps = bwd_bytes / bwd_us / 1e3
+    cfwd_us = launches_us(lambda i: causal_fwd(cset, B5, n5, dt5, sc5))
+    cbwd_us = launches_us(lambda i: causal_bwd(cset, B5, n5, dt5, sc5))
+    rfwd_us = launches_us(lambda i: rope_apply(rsets[i % 6], S5, 1, H5, HN5, dt5, 0))
+    rbwd_us = launches_us(lambda i: rope_apply(rsets[i % 6], S5, 1, H5, HN5, dt5, 1))
+    cbwd_gbps = cbwd_bytes / cbwd_us / 1e3
 
     result = {
         "metric": METRIC,
@@ -233,48 +286,60 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
-        "scaling": "weak",
+        "scaling": None,  # one GPU only: every row is independent, more GPUs see a smaller batch
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "configs[1]: padding-masked scaled softmax fwd+bwd, scores [8,16,1024,1024] "
-                        "fp16 storage, bool mask [8,1,1024,1024], scale 0.125, lens~U[256,1024]",
-            "step": "1 forward launch + 1 backward launch",
-            "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes,
-            "buffer_sets": len(sets),
+            "workload": "configs[4]: long-context causal scaled softmax fwd+bwd, scores [1,32,8192,8192] "
+                        "bf16 storage, scale 1/sqrt(128), plus full rotary (rotary_pct 1.0) fwd+bwd on "
+                        "q,k [8192,1,32,128] bf16, base 10000, fp32 cos/sin",
+            "step": "rotary fwd (q+k, one launch) + causal softmax fwd + causal softmax bwd + rotary bwd",
+            "algorithmic_bytes_per_step": step_bytes,
+            "rotary_buffer_sets": len(rsets),
         },
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1),
-        "us_per_call": {"fwd": round(fwd_us, 2), "bwd": round(bwd_us, 2)},
+        "min_pct_hbm_peak_over_configs": None,  # filled in from the per-config table below
+        "us_per_call": {"causal_fwd": round(cfwd_us, 2), "causal_bwd": round(cbwd_us, 2),
+                        "rotary_fwd": round(rfwd_us, 2), "rotary_bwd": round(rbwd_us, 2)},
         "roofline": {
             "bound": "hbm",
-            "kernel": "softmax_bwd_packed_kernel<F16, 64 lanes/row, no mask, 2 row passes/wave, 2 chunks of 512 columns>",
-            "achieved": round(bwd_gbps, 1),
+            "kernel": "softmax_bwd_kernel<BF16, 2 chunks of 512 columns per wave, 8 waves per row, 1 row per block, causal>",
+            "achieved": round(cbwd_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BWD_BYTES,
-            "algorithmic_bytes_per_launch": bwd_bytes,
-            "avg_launch_us": round(bwd_us, 2),
+            "frac": round(cbwd_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": cbwd_bytes,
+            "avg_launch_us": round(cbwd_us, 2),
         },
     }
-    del sets
+    result["roofline"].update(measured_traffic("cfg5_causal_bwd"))
+    del cset, rsets
     torch.cuda.empty_cache()
 
     # ------------------------------------------------------------------ CPU baseline
     if not args.no_cpu:
+        # a bounded sample of the same step: 1 of the 32 score matrices through the oracle's torch
+        # path (forward + autograd backward) and 256 of the 8192 positions through its rotary
+        # expression (forward + autograd backward) -- 1/32 of each part of the workload
         cores = torch.get_num_threads()
-        sample_b = 2
         g0 = torch.Generator().manual_seed(99)
-        xs = (torch.randn(sample_b, heads, sq, sk, generator=g0) * 8).half()
-        dys = torch.randn(sample_b, heads, sq, sk, generator=g0).half()
-        lens = torch.randint(256, sk + 1, (sample_b,), generator=g0)
-        ms = R.padding_mask(lens, sq, sk)
+        xs = (torch.randn(1, 1, n5, n5, generator=g0) * 8).bfloat16()
+        dys = torch.randn(1, 1, n5, n5, generator=g0).bfloat16()
+        cm = R.get_attn_mask(n5, torch.device("cpu"))
+        npos = S5 // B5
+        qs = torch.randn(npos, 1, H5, HN5, generator=g0).bfloat16()
+        ks = torch.randn(npos, 1, H5, HN5, generator=g0).bfloat16()
+        cos_c, sin_c = R.rotary_tables(HN5, npos)
 
         def cpu_step():
+            R.apply_rotary_pos_emb(qs, ks, cos_c, sin_c)
             xin = xs.clone().requires_grad_(True)
-            y = R.forward_torch_softmax(xin, ms, scale, input_in_fp16=True, softmax_in_fp32=True)
+            y = R.forward_torch_softmax(xin, cm, sc5, input_in_fp16=False, softmax_in_fp32=True,
+                                        input_in_bf16=True)
             y.backward(dys)
+            R.rotary_autograd_fp32(qs, ks, cos_c, sin_c, qs, ks)
             return xin.grad
 
         cpu_step()
@@ -283,20 +348,25 @@ def main():
             cpu_step()
             reps += 1
         cpu_s = (time.perf_counter() - t0) / reps
-        sample_bytes = (fwd_bytes + bwd_bytes) * sample_b // b
         result["cpu_baseline"] = {
-            "value": round(sample_bytes / cpu_s / 1e9, 3),
+            "value": round(step_bytes / B5 / cpu_s / 1e9, 3),
             "unit": "GB/s",
             "cores": cores,
             "kind": "port",
-            "sample": f"{sample_b} of the {b} batch entries of configs[1] ([{sample_b},16,1024,1024] "
-                      f"fp16), forward + autograd backward of the oracle's torch path, {reps} "
-                      f"repetitions, {cpu_s * 1e3:.1f} ms each",
-            "ms_per_step_scaled_to_full_batch": round(cpu_s * 1e3 * b / sample_b, 1),
+            "sample": f"1/32 of a step of configs[4]: 1 of the 32 score matrices ([1,1,8192,8192] bf16) "
+                      f"through the oracle's torch softmax path, forward + autograd backward, and {npos} of "
+                      f"the 8192 positions of q,k through its rotary expression, forward + autograd "
+                      f"backward; {reps} repetitions, {cpu_s * 1e3:.1f} ms each",
+            "ms_per_step_scaled_to_full_batch": round(cpu_s * 1e3 * B5, 1),
         }
-        del xs, dys, ms
+        del xs, dys, cm, qs, ks
 
     # ------------------------------------------------------------------ every BASELINE shape
+    # configs[1], used by several rows below
+    b, heads, sq, sk, dtype, scale = 8, 16, 1024, 1024, torch.float16, 0.125
+    n_elem = b * heads * sq * sk
+    fwd_bytes = 2 * n_elem * 2 + b * sq * sk
+    bwd_bytes = 3 * n_elem * 2
     def cpu_time_us(fn, budget_s=1.5):
         fn()
         reps, t0 = 0, time.perf_counter()
@@ -467,8 +537,8 @@ def main():
             src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
             dst = torch.empty_like(src)
             table.append(row("copy 1 GiB (read + write)", 2 * nbytes,
-                             *time_launches(lambda t: ok(lib.neox_copy_bytes(dst.data_ptr(), src.data_ptr(),
-                                                                            nbytes, stream)), [None], 50)))
+                             *time_launches(lambda t: ok(probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(),
+                                                                               nbytes, stream)), [None], 50)))
         # softmax + attention dropout in one kernel per pass (the op that follows the softmax in
         # the model), on the padded, the 20B and the long-context shapes; p = 0.1
         if want("dropout"):
@@ -678,6 +748,7 @@ def main():
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
         if pcts:
             result["min_pct_hbm_peak_over_configs"] = min(pcts)
+            result["min_pct_hbm_peak_row"] = next(r["op"] for r in table if r["pct_hbm_peak"] == min(pcts))
 
     print(json.dumps(result), flush=True)
 

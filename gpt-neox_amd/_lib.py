@@ -14,7 +14,7 @@ import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(_CSRC, "libneox_fused.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 NEOX_F16, NEOX_BF16, NEOX_F32 = 0, 1, 2
 _DTYPE_CODE = {torch.float16: NEOX_F16, torch.bfloat16: NEOX_BF16, torch.float32: NEOX_F32}
@@ -64,11 +64,14 @@ SIGNATURES = {
     "neox_get_batch_per_block": (ctypes.c_int, [_i32, _i32, _i32, _i32]),
     "neox_rope_apply": (
         ctypes.c_int,
-        [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _c_i64p, _c_i64p, _c_i64p,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _c_i64p, _c_i64p, _c_i64p,
          _c_i64p, _i64, _i32, _i32, _i32, _i32, _vp],
     ),
-    "neox_copy_bytes": (ctypes.c_int, [_vp, _vp, _i64, _vp]),
-    "neox_touch_strided": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp]),
+    "neox_rope_apply_freqs": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _c_i64p, _c_i64p, _c_i64p,
+         _c_i64p, _i64, _i32, _i32, _i32, _vp],
+    ),
 }
 
 _lock = threading.Lock()

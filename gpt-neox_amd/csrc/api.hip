@@ -206,40 +206,6 @@ __global__ __launch_bounds__(256) void keep_mask_kernel(uint8_t* keep, DropoutAr
         if (group * 8 + k < n) keep[group * 8 + k] = (bits >> k) & 1u;
 }
 
-// Plain copy with the same access shape (measurement aid).
-__global__ __launch_bounds__(256) void copy_kernel(u32x4* dst, const u32x4* src, size_t n16) {
-    size_t idx = (size_t)blockIdx.x * 1024 + threadIdx.x;
-    u32x4 r[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-        if (idx + k * 256 < n16) r[k] = ld128(src + idx + k * 256);
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-        if (idx + k * 256 < n16) st128(dst + idx + k * 256, r[k]);
-}
-
-// Loads the first span_bytes of every stride_bytes and stores them back unchanged, one 16-byte
-// slot per lane, consecutive lanes on consecutive slots (measurement aid: the memory pattern of an
-// in-place partial rotary without its arithmetic, tables or index computations).
-__global__ __launch_bounds__(256) void touch_strided_kernel(char* buf, uint64_t slots, uint32_t slots_per_span,
-                                                            uint64_t stride_bytes, uint32_t flip) {
-    const uint64_t g0 = (uint64_t)blockIdx.x * 1024 + threadIdx.x;
-    char* p[4];
-    u32x4 v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {  // four accesses in flight per lane, as in the kernels
-        const uint64_t g = g0 + k * 256;
-        const uint64_t span = g / slots_per_span;
-        p[k] = buf + span * stride_bytes + (g - span * slots_per_span) * 16;
-        if (g < slots) v[k] = ld128(p[k]);
-    }
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        v[k].x ^= flip;  // 0 at run time; keeps the compiler from dropping the store of an unchanged value
-        if (g0 + k * 256 < slots) st128(p[k], v[k]);
-    }
-}
-
 }  // namespace neox
 
 using namespace neox;
@@ -429,34 +395,40 @@ static int check_rope_strides(const int64_t* st, const char* what, const char* n
     return NEOX_OK;
 }
 
-int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, const void* cos,
-                    const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
-                    int32_t d_rot, const int64_t q_strides[3], const int64_t k_strides[3],
-                    const int64_t out_q_strides[3], const int64_t out_k_strides[3],
-                    int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
-                    int32_t backward, void* stream) {
-    static const char* what = "neox_rope_apply";
+}  // extern "C"
+
+// Both rotary entry points.  cs_dtype == kRopeAngles: `cos` holds fp32 angles and `sin` is not used.
+static int rope_apply(const char* what, void* out_q, void* out_k, const void* q, const void* k,
+                      const void* cos, const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
+                      int32_t d_rot, int32_t d, const int64_t q_strides[3], const int64_t k_strides[3],
+                      const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                      int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
+                      int32_t backward, void* stream) {
+    const bool angles = (cs_dtype == kRopeAngles);
+    if (angles) sin = cos;
     if (!out_q || !q || !cos || !sin) return fail(NEOX_ERR_NULL_POINTER, "%s: null tensor pointer", what);
     if ((k == nullptr) != (out_k == nullptr))
         return fail(NEOX_ERR_NULL_POINTER, "%s: k and out_k must both be given or both be null", what);
     if (int e = check_dtype(dtype, what)) return e;
-    if (cs_dtype != NEOX_F32 && cs_dtype != dtype)
+    if (!angles && cs_dtype != NEOX_F32 && cs_dtype != dtype)
         return fail(NEOX_ERR_BAD_DTYPE, "%s: cos/sin must be fp32 or have the dtype of q (code %d)", what, cs_dtype);
     const bool has_k = (k != nullptr);
     if (s < 1 || b < 1 || h_q < 1 || (has_k && h_k < 1))
         return fail(NEOX_ERR_BAD_SHAPE, "%s: s=%d b=%d h_q=%d h_k=%d must be >= 1", what, s, b, h_q, h_k);
     if (d_rot < 2 || (d_rot & 1))
         return fail(NEOX_ERR_BAD_SHAPE, "%s: d_rot=%d must be even and >= 2", what, d_rot);
+    if (d < d_rot) return fail(NEOX_ERR_BAD_SHAPE, "%s: d=%d is smaller than d_rot=%d", what, d, d_rot);
     if (b > 65535) return fail(NEOX_ERR_BAD_SHAPE, "%s: b=%d exceeds 65535", what, b);
     if (pos_offset < 0) return fail(NEOX_ERR_BAD_SHAPE, "%s: pos_offset=%d is negative", what, pos_offset);
-    if (cs_stride < d_rot) return fail(NEOX_ERR_BAD_STRIDE, "%s: cos/sin row stride %lld < d_rot=%d", what, (long long)cs_stride, d_rot);
+    if (cs_stride < d_rot)
+        return fail(NEOX_ERR_BAD_STRIDE, "%s: %s row stride %lld < d_rot=%d", what, angles ? "freqs" : "cos/sin", (long long)cs_stride, d_rot);
     if (int e = check_rope_strides(q_strides, what, "q")) return e;
     if (int e = check_rope_strides(out_q_strides, what, "out_q")) return e;
     if (has_k) {
         if (int e = check_rope_strides(k_strides, what, "k")) return e;
         if (int e = check_rope_strides(out_k_strides, what, "out_k")) return e;
     }
-    const int cs_size = (cs_dtype == NEOX_F32) ? 4 : 2;
+    const int cs_size = (angles || cs_dtype == NEOX_F32) ? 4 : 2;
     if (!aligned(q, 2) || !aligned(out_q, 2) || (has_k && (!aligned(k, 2) || !aligned(out_k, 2))) ||
         !aligned(cos, cs_size) || !aligned(sin, cs_size))
         return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
@@ -471,6 +443,7 @@ int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, cons
         };
         if (!ok_t(q, q_strides) || !ok_t(out_q, out_q_strides)) return false;
         if (has_k && (!ok_t(k, k_strides) || !ok_t(out_k, out_k_strides))) return false;
+        if (angles) return true;  // the angles are read one by one
         // table accesses are at most 128 bits wide
         const int tw = (cs_size == 4 && w > 4) ? 4 : w;
         const uintptr_t tbytes = (uintptr_t)tw * cs_size;
@@ -512,10 +485,18 @@ int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, cons
     a.half = half;
     a.lpv = lpv;
     a.nt = has_k ? 2 : 1;
+    // Out of place, the pass-through dims [d_rot, d) are copied by the same launch: by further
+    // lanes of the head's lane group when the whole head splits into at most 64 slots, else by
+    // the element-wise loop of the other kernel.
+    const bool out_of_place = (q != out_q) || (has_k && k != out_k);
+    if (out_of_place && d > d_rot) {
+        a.copy_dims = d - d_rot;
+        if (w >= 2 && a.copy_dims % w == 0 && d / w <= kWave) a.pad_slots = a.copy_dims / w;
+    }
     // In place, a rotated span that ends inside a 64-byte block is written back together with the
     // rest of that block (unchanged pass-through dims the loads fetch anyway): the memory system
     // then sees whole 64-byte writes instead of partial ones.
-    {
+    if (a.copy_dims == 0) {
         const int slot_bytes = w * 2, span_bytes = d_rot * 2;
         const int pad_bytes = (64 - span_bytes % 64) % 64;
         auto in_place_64 = [&](const void* in, const void* out, const int64_t* is, const int64_t* os) {
@@ -535,31 +516,30 @@ int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, cons
                         what);
 }
 
-int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream) {
-    static const char* what = "neox_copy_bytes";
-    if (!dst || !src) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
-    if (nbytes < 16 || nbytes % 16) return fail(NEOX_ERR_BAD_SHAPE, "%s: nbytes=%lld must be a positive multiple of 16", what, (long long)nbytes);
-    if (!aligned(dst, 16) || !aligned(src, 16)) return fail(NEOX_ERR_MISALIGNED, "%s: pointers must be 16-byte aligned", what);
-    const size_t n16 = (size_t)nbytes / 16;
-    const size_t blocks = (n16 + 1023) / 1024;
-    if (blocks > 0x7fffffffULL) return fail(NEOX_ERR_BAD_SHAPE, "%s: nbytes too large", what);
-    hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), n16);
-    return check_launch(hipGetLastError(), what);
+extern "C" {
+
+int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, const void* cos,
+                    const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
+                    int32_t d_rot, int32_t d, const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                    int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
+                    int32_t backward, void* stream) {
+    static const char* what = "neox_rope_apply";
+    if (cs_dtype != NEOX_F16 && cs_dtype != NEOX_BF16 && cs_dtype != NEOX_F32)
+        return fail(NEOX_ERR_BAD_DTYPE, "%s: cos/sin must be fp32 or have the dtype of q (code %d)", what, cs_dtype);
+    return rope_apply(what, out_q, out_k, q, k, cos, sin, s, b, h_q, h_k, d_rot, d, q_strides, k_strides,
+                      out_q_strides, out_k_strides, cs_stride, pos_offset, dtype, cs_dtype, backward, stream);
 }
 
-int neox_touch_strided(void* buf, int64_t n_spans, int32_t span_bytes, int64_t stride_bytes, void* stream) {
-    static const char* what = "neox_touch_strided";
-    if (!buf) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
-    if (n_spans < 1 || span_bytes < 16 || span_bytes % 16 || stride_bytes < span_bytes || stride_bytes % 16)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: need n_spans >= 1, span_bytes and stride_bytes multiples of 16, span <= stride", what);
-    if (!aligned(buf, 16)) return fail(NEOX_ERR_MISALIGNED, "%s: pointer must be 16-byte aligned", what);
-    const uint64_t slots = (uint64_t)n_spans * (uint32_t)(span_bytes / 16);
-    const uint64_t blocks = (slots + 1023) / 1024;
-    if (blocks > 0x7fffffffULL) return fail(NEOX_ERR_BAD_SHAPE, "%s: too many spans", what);
-    hipLaunchKernelGGL(touch_strided_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                       static_cast<char*>(buf), slots, (uint32_t)(span_bytes / 16), (uint64_t)stride_bytes, 0u);
-    return check_launch(hipGetLastError(), what);
+int neox_rope_apply_freqs(void* out_q, void* out_k, const void* q, const void* k, const float* freqs,
+                          int32_t s, int32_t b, int32_t h_q, int32_t h_k, int32_t d_rot, int32_t d,
+                          const int64_t q_strides[3], const int64_t k_strides[3],
+                          const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                          int64_t freqs_stride, int32_t pos_offset, int32_t dtype, int32_t backward,
+                          void* stream) {
+    return rope_apply("neox_rope_apply_freqs", out_q, out_k, q, k, freqs, nullptr, s, b, h_q, h_k, d_rot, d,
+                      q_strides, k_strides, out_q_strides, out_k_strides, freqs_stride, pos_offset, dtype,
+                      kRopeAngles, backward, stream);
 }
 
 }  // extern "C"

@@ -38,6 +38,8 @@ hipError_t launch_softmax_ragged_dropout_fwd(const SoftmaxArgs& a, Mask mask, in
                                              hipStream_t stream);
 hipError_t launch_softmax_ragged_dropout_bwd(const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok,
                                              hipStream_t stream);
+// cs_dtype: NEOX_F32 or the dtype of q for cos/sin tables, kRopeAngles for fp32 angles in a.cos
+constexpr int kRopeAngles = -1;
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream);
 

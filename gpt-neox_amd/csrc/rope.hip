@@ -3,6 +3,12 @@
 
 namespace neox {
 
+// LDS for the cos/sin values a block evaluates from angles: 2 x d_rot floats (at most 32 KiB)
+template <typename CS>
+static size_t angle_lds_bytes(const RopeArgs& a) {
+    return std::is_same<CS, Angles>::value ? (size_t)a.half * 4 * sizeof(float) : 0;
+}
+
 template <typename T, typename CS, int W, bool BWD>
 static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipStream_t st) {
     const int lpv = a.lpv;
@@ -21,7 +27,7 @@ static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipSt
     }
     const dim3 grid(s, n_outer, zsplit);
     const dim3 block(lpv, vpb);
-    hipLaunchKernelGGL((rope_kernel<T, CS, W, BWD>), grid, block, 0, st, a);
+    hipLaunchKernelGGL((rope_kernel<T, CS, W, BWD>), grid, block, angle_lds_bytes<CS>(a), st, a);
     return hipGetLastError();
 }
 
@@ -43,12 +49,16 @@ static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStr
     b.zsplit = (int)zsplit;
     b.outer_grid = n_outer;
     b.share = (int)((nmax + zsplit - 1) / zsplit);
-    hipLaunchKernelGGL((rope_span_kernel<T, CS, W, BWD>), dim3((unsigned)(pairs * zsplit)), dim3(256), 0, st, b);
+    hipLaunchKernelGGL((rope_span_kernel<T, CS, W, BWD>), dim3((unsigned)(pairs * zsplit)), dim3(256),
+                       angle_lds_bytes<CS>(a), st, b);
     return hipGetLastError();
 }
 
-// the rotated span is at most 64 slots of w >= 2 dims: the contiguous-span kernel applies
-static bool span_shape(const RopeArgs& a, int w) { return w >= 2 && a.lpv * 2 <= kWave; }
+// the rotated span, with the slots stored as loaded behind it, is at most 64 slots of w >= 2 dims:
+// the contiguous-span kernel applies (a pass-through copy must be covered by those slots)
+static bool span_shape(const RopeArgs& a, int w) {
+    return w >= 2 && a.lpv * 2 + a.pad_slots <= kWave && (a.copy_dims == 0 || a.pad_slots * w == a.copy_dims);
+}
 
 template <typename T, typename CS, bool BWD>
 static hipError_t launch_rope_w(const RopeArgs& a, int s, int n_outer, int w, hipStream_t st) {
@@ -77,6 +87,10 @@ static hipError_t launch_rope_dir(const RopeArgs& a, int s, int n_outer, int w, 
 
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,
                        bool backward, hipStream_t stream) {
+    if (cs_dtype == kRopeAngles) {
+        return dtype == NEOX_F16 ? launch_rope_dir<F16, Angles>(a, s, n_outer, w, backward, stream)
+                                 : launch_rope_dir<BF16, Angles>(a, s, n_outer, w, backward, stream);
+    }
     const bool cs32 = (cs_dtype == NEOX_F32);
     if (dtype == NEOX_F16) {
         return cs32 ? launch_rope_dir<F16, float>(a, s, n_outer, w, backward, stream)

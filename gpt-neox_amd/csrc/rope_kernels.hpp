@@ -20,10 +20,18 @@
 // (j, j + d_rot/2) is written by the lane(s) that read it, so in-place operation is
 // race-free.  q/k accesses carry the non-temporal hint (each byte is touched once).
 //
+// The rotation is given as cos/sin tables (fp32 or the storage type) or as fp32 angles (CS =
+// Angles): then the block evaluates sincosf once per dim of its position into LDS -- d_rot
+// evaluations per block, shared by all its heads -- and the lanes take their values from there.
+// Out of place, the kernels also copy the pass-through dims [d_rot, d) of every head in the same
+// launch (span kernel: further lanes of the head's lane group; rope_kernel: a 16-bit copy loop).
+//
 // Arithmetic is fp32 with the two products rounded separately (no fused
 // multiply-add), which is bit-identical to evaluating q*cos + rotate_half(q)*sin
 // in fp32; the result is rounded once to the storage type.
 #pragma once
+
+#include <type_traits>
 
 #include "wave.hpp"
 
@@ -47,7 +55,9 @@ struct RopeArgs {
     int32_t half;        // d_rot / 2
     int32_t lpv;         // slots per vector = half / W
     int32_t nt;          // 1: q only, 2: q and k
-    int32_t pad_slots;   // span kernel, in place: slots after the rotated span that are rewritten unchanged
+    int32_t pad_slots;   // span kernel: slots after the rotated span that are stored as loaded (in place:
+                         // the rest of a 64-byte block; out of place: the pass-through dims)
+    int32_t copy_dims;   // out of place: pass-through dims [d_rot, d_rot + copy_dims) to copy, else 0
     // span kernel, filled in by its launcher
     int32_t zsplit;      // blocks sharing the vectors of one (position, outer) pair
     int32_t outer_grid;  // extent of the outer loop in the block index
@@ -93,6 +103,22 @@ __device__ __forceinline__ void store_elems(char* p, const float (&f)[W]) {
         if constexpr (NT) __builtin_nontemporal_store(w, reinterpret_cast<P*>(p));
         else *reinterpret_cast<P*>(p) = w;
     }
+}
+
+// CS tag: the rotation is given as fp32 angles; cos and sin are evaluated in the kernel
+struct Angles {};
+
+// One position's cos/sin from its fp32 angles: every thread of the block evaluates sincosf for
+// the dims tid, tid + nthreads, ... into LDS (cos at [0, d_rot), sin at [d_rot, 2 d_rot)).  All
+// threads of the block must call this (it ends with a barrier).
+__device__ __forceinline__ void angles_to_lds(const float* angles, int d_rot, float* tab, int tid, int nthreads) {
+    for (int j = tid; j < d_rot; j += nthreads) {
+        float sv, cv;
+        sincosf(angles[j], &sv, &cv);
+        tab[j] = cv;
+        tab[d_rot + j] = sv;
+    }
+    __syncthreads();
 }
 
 // cos/sin table element access: CS = float reads fp32, otherwise 16-bit type CS
@@ -146,10 +172,23 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
 
     float cl[W], ch[W], sl[W], sh[W];
     const int64_t crow = (int64_t)(pos + a.pos_offset) * a.cs_stride;
-    load_table<CS, W>(a.cos, crow + j, cl);
-    load_table<CS, W>(a.cos, crow + j + half, ch);
-    load_table<CS, W>(a.sin, crow + j, sl);
-    load_table<CS, W>(a.sin, crow + j + half, sh);
+    if constexpr (std::is_same<CS, Angles>::value) {
+        extern __shared__ float lds_tab[];
+        angles_to_lds(reinterpret_cast<const float*>(a.cos) + crow, 2 * half, lds_tab,
+                      threadIdx.y * blockDim.x + threadIdx.x, blockDim.x * blockDim.y);
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+            cl[k] = lds_tab[j + k];
+            ch[k] = lds_tab[j + half + k];
+            sl[k] = lds_tab[2 * half + j + k];
+            sh[k] = lds_tab[3 * half + j + k];
+        }
+    } else {
+        load_table<CS, W>(a.cos, crow + j, cl);
+        load_table<CS, W>(a.cos, crow + j + half, ch);
+        load_table<CS, W>(a.sin, crow + j, sl);
+        load_table<CS, W>(a.sin, crow + j + half, sh);
+    }
 
     const int v_step = blockDim.y * gridDim.z;
     const int n0 = (outer < a.t[0].n_outer) ? a.t[0].n_inner : 0;
@@ -188,6 +227,19 @@ __global__ __launch_bounds__(256) void rope_kernel(RopeArgs a) {
             char* op = a.t[1].out + (ko + (int64_t)v * a.t[1].out_stride[2]) * 2;
             store_elems<T, W, true>(op, ol);
             store_elems<T, W, true>(op + (size_t)half * 2, oh);
+        }
+        if (a.copy_dims > 0) {
+            // out of place: the pass-through dims of this head, element by element (the shapes
+            // that reach this kernel have no common wider alignment)
+            const int e0 = 2 * half - j, e1 = e0 + a.copy_dims;  // relative to the lane's first dim
+            for (int e = e0 + (int)threadIdx.x; e < e1; e += blockDim.x) {
+                if (do_q)
+                    *reinterpret_cast<uint16_t*>(a.t[0].out + (qo + (int64_t)v * a.t[0].out_stride[2] + e) * 2) =
+                        *reinterpret_cast<const uint16_t*>(qp + (int64_t)e * 2);
+                if (do_k)
+                    *reinterpret_cast<uint16_t*>(a.t[1].out + (ko + (int64_t)v * a.t[1].out_stride[2] + e) * 2) =
+                        *reinterpret_cast<const uint16_t*>(kp + (int64_t)e * 2);
+            }
         }
     }
 }
@@ -254,8 +306,18 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
     // partner's dims with sign +,-.  Folding the sign into sin is exact.
     float c[W], sn[W];
     const int64_t crow = (int64_t)(pos + a.pos_offset) * a.cs_stride;
-    load_table<CS, W>(a.cos, crow + jt, c);
-    load_table<CS, W>(a.sin, crow + (BWD ? jp : jt), sn);
+    if constexpr (std::is_same<CS, Angles>::value) {
+        extern __shared__ float lds_tab[];
+        angles_to_lds(reinterpret_cast<const float*>(a.cos) + crow, 2 * a.half, lds_tab, threadIdx.x, 256);
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+            c[k] = lds_tab[jt + k];
+            sn[k] = lds_tab[2 * a.half + (BWD ? jp : jt) + k];
+        }
+    } else {
+        load_table<CS, W>(a.cos, crow + jt, c);
+        load_table<CS, W>(a.sin, crow + (BWD ? jp : jt), sn);
+    }
     if (second == BWD) {
 #pragma unroll
         for (int k = 0; k < W; ++k) sn[k] = -sn[k];

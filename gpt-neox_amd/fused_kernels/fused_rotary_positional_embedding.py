@@ -5,8 +5,10 @@ Same functions and checks as the reference's pybind module
 (megatron/fused_kernels/fused_rotary_positional_embedding.cpp:38-139,
 megatron/fused_kernels/fused_rotary_positional_embedding_cuda.cu:24-216):
 ``t`` is ``[s, b, h, d]`` with any s/b/h strides, the table is ``[s, 1, 1, d2]``
-with ``d2 <= d``; dims ``>= d2`` are copied through; ``transpose_output`` makes the
-result's memory ``[b, s, h, d]``.  All of it is served by ``neox_rope_apply``.
+with ``d2 <= d``; dims ``>= d2`` are copied through by the same launch;
+``transpose_output`` makes the result's memory ``[b, s, h, d]``.  The cached variants are
+served by ``neox_rope_apply``, the ``freqs`` variants by ``neox_rope_apply_freqs``, which
+evaluates cos and sin of the angles inside the kernel as the reference's does.
 Differences: arithmetic is fp32 with one rounding (the reference rounds cos/sin to
 the dtype of ``t`` first); ``t`` must be fp16 or bf16.
 """
@@ -17,25 +19,33 @@ from .. import _lib
 _HALF = (torch.float16, torch.bfloat16)
 
 
-def rope_launch(out_q, out_k, q, k, cos, sin, d_rot, pos_offset, backward):
+def rope_launch(out_q, out_k, q, k, cos, sin, d_rot, pos_offset, backward, d=None):
     """One launch over q (and k, unless None).  Tensors are 4-D ``[s, b, h, >=d_rot]``
     with last-dim stride 1; cos/sin are ``[>= pos_offset + s, .., d_rot]`` contiguous
-    in their last dim, fp32 or of q's dtype."""
+    in their last dim, fp32 or of q's dtype; ``sin is None`` means that ``cos`` holds fp32
+    angles whose cos and sin the kernel evaluates.  ``d`` (default ``d_rot``): leading dims
+    of every head delivered in the outputs -- out of place the dims ``[d_rot, d)`` are copied
+    from the inputs."""
     s, b, h_q = q.shape[0], q.shape[1], q.shape[2]
     h_k = k.shape[2] if k is not None else 0
     lib = _lib.lib()
+    head = (
+        out_q.data_ptr(), out_k.data_ptr() if k is not None else None,
+        q.data_ptr(), k.data_ptr() if k is not None else None,
+    )
+    shape = (
+        s, b, h_q, h_k, d_rot, d_rot if d is None else d,
+        _lib.strides3(q), _lib.strides3(k) if k is not None else None,
+        _lib.strides3(out_q), _lib.strides3(out_k) if k is not None else None,
+        cos.stride(0) if cos.shape[0] > 1 else d_rot, pos_offset, _lib.dtype_code(q.dtype),
+    )
+    tail = (1 if backward else 0, _lib.current_stream(q))
     with _lib.device_guard(q):
-        _lib.check(
-            lib.neox_rope_apply(
-                out_q.data_ptr(), out_k.data_ptr() if k is not None else None,
-                q.data_ptr(), k.data_ptr() if k is not None else None,
-                cos.data_ptr(), sin.data_ptr(), s, b, h_q, h_k, d_rot,
-                _lib.strides3(q), _lib.strides3(k) if k is not None else None,
-                _lib.strides3(out_q), _lib.strides3(out_k) if k is not None else None,
-                cos.stride(0) if cos.shape[0] > 1 else d_rot, pos_offset, _lib.dtype_code(q.dtype), _lib.dtype_code(cos.dtype),
-                1 if backward else 0, _lib.current_stream(q),
-            )
-        )
+        if sin is None:
+            _lib.check(lib.neox_rope_apply_freqs(*head, cos.data_ptr(), *shape, *tail))
+        else:
+            _lib.check(lib.neox_rope_apply(*head, cos.data_ptr(), sin.data_ptr(), *shape,
+                                           _lib.dtype_code(cos.dtype), *tail))
 
 
 def _check_table(t, table, name):
@@ -52,6 +62,8 @@ def _check_table(t, table, name):
 
 
 def _apply(t, cos, sin, transpose_output, backward):
+    """Out-of-place rotation of ``t`` by tables (``cos``, ``sin``) or by angles (``cos`` = freqs,
+    ``sin`` None); one launch, which also copies the dims ``>= d2``."""
     if t.dtype not in _HALF:
         raise RuntimeError("Only fp16 and bf16 are supported")
     _lib.require_gpu(t, cos, sin)
@@ -60,16 +72,15 @@ def _apply(t, cos, sin, transpose_output, backward):
     if t.stride(3) != 1:
         t = t.contiguous()
     cos = cos.contiguous()
-    sin = sin.contiguous()
+    if sin is not None:
+        sin = sin.contiguous()
     if transpose_output:
         out = torch.empty((b, s, h, d), dtype=t.dtype, device=t.device).transpose(0, 1)
     else:
         out = torch.empty((s, b, h, d), dtype=t.dtype, device=t.device)
     if t.numel() == 0:
         return out
-    rope_launch(out, None, t, None, cos, sin, d2, 0, backward)
-    if d > d2:
-        out[..., d2:].copy_(t[..., d2:])
+    rope_launch(out, None, t, None, cos, sin, d2, 0, backward, d=d)
     return out
 
 
@@ -98,15 +109,15 @@ def backward_cached(output_grads, cos, sin, transpose_output=False):
 
 
 def forward(input, freqs, transpose_output=False):
-    """Rotation angles given as ``freqs`` (fp32); cos/sin are evaluated in fp32."""
+    """Rotation angles given as ``freqs`` (fp32); cos/sin are evaluated in fp32 inside the kernel."""
     _check_table(input, freqs, "freqs")
     if freqs.dtype != torch.float32:
         raise RuntimeError("Dtype of the freqs tensor must be float")
-    return _apply(input, freqs.cos(), freqs.sin(), transpose_output, backward=False)
+    return _apply(input, freqs, None, transpose_output, backward=False)
 
 
 def backward(output_grads, freqs, transpose_output=False):
     _check_table(output_grads, freqs, "freqs")
     if freqs.dtype != torch.float32:
         raise RuntimeError("Dtype of the freqs tensor must be float")
-    return _apply(output_grads, freqs.cos(), freqs.sin(), transpose_output, backward=True)
+    return _apply(output_grads, freqs, None, transpose_output, backward=True)

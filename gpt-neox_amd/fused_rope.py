@@ -30,11 +30,12 @@ def _make_rope_function(name, n_tables, fwd, bwd, doc):
         transpose_output_memory = bool(flags[0]) if flags else False
         ctx.save_for_backward(*tables)
         ctx.transpose_output_memory = transpose_output_memory
+        ctx.n_inputs = 1 + len(rest)
         return fwd(t, *tables, transpose_output_memory)
 
     def backward(ctx, grad_output: torch.Tensor) -> Tuple[Union[torch.Tensor, None], ...]:
         grad_input = bwd(grad_output, *ctx.saved_tensors, ctx.transpose_output_memory)
-        return (grad_input,) + (None,) * (n_tables + 1)
+        return (grad_input,) + (None,) * (ctx.n_inputs - 1)
 
     return type(name, (torch.autograd.Function,),
                 {"forward": staticmethod(forward), "backward": staticmethod(backward), "__doc__": doc})

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NEOX_FUSED_ABI_VERSION 1
+#define NEOX_FUSED_ABI_VERSION 2
 
 typedef enum neox_dtype {
     NEOX_F16 = 0,  /* IEEE binary16 */
@@ -181,8 +181,8 @@ int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np);
 
 /*
  * Rotary positional embedding over the first d_rot dims of q and (optionally) k
- * in ONE launch.  Layout [s, b, h, d_rot(+pass-through)] addressed by element
- * strides {stride_s, stride_b, stride_h}; the last dim has stride 1.
+ * in ONE launch.  Layout [s, b, h, d] addressed by element strides
+ * {stride_s, stride_b, stride_h}; the last dim has stride 1.
  *   forward : out[j]      = x[j]*cos[j]           - x[j+d_rot/2]*sin[j]
  *             out[j+d/2]  = x[j+d/2]*cos[j+d/2]   + x[j]*sin[j+d/2]
  *   backward: out[j]      = g[j]*cos[j]           + g[j+d/2]*sin[j+d/2]
@@ -190,37 +190,42 @@ int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np);
  * cos/sin: [>= pos_offset + s, d_rot] rows of stride cs_stride elements, dtype
  * cs_dtype (NEOX_F32 or the same as dtype).  Arithmetic is fp32 with separately
  * rounded products (bit-equal to torch's fp32 q*cos + rotate_half(q)*sin), one
- * rounding to dtype on store.  out_* may alias the inputs (in place).  Dims >= d_rot
- * keep their values; out of place they are never read or written, in place those that
- * share a 64-byte block with the end of the rotated span may be written back unchanged
+ * rounding to dtype on store.  out_* may alias the inputs (in place).
+ * d >= d_rot is the number of leading dims of every head the call delivers in out_*:
+ * out of place (out_q != q, or out_k != k) the pass-through dims [d_rot, d) are copied
+ * from the inputs by the same launch, as the reference's kernels do; pass d = d_rot to
+ * have only the rotated span written.  In place the dims >= d_rot keep their values; those
+ * that share a 64-byte block with the end of the rotated span may be written back unchanged
  * (whole 64-byte writes are much cheaper for the memory system than partial ones).
  * k / out_k may both be NULL.
  * Replaces apply_rotary_pos_emb / apply_rotary_pos_emb_torch
  *   megatron/model/positional_embeddings.py:103-126
  * and fused_rotary_positional_embedding.forward_cached / backward_cached
  *   megatron/fused_kernels/fused_rotary_positional_embedding.cpp:83-127
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.h:126-230 (rotation and tail copy)
  */
 int neox_rope_apply(void* out_q, void* out_k, const void* q, const void* k, const void* cos,
                     const void* sin, int32_t s, int32_t b, int32_t h_q, int32_t h_k,
-                    int32_t d_rot, const int64_t q_strides[3], const int64_t k_strides[3],
+                    int32_t d_rot, int32_t d, const int64_t q_strides[3], const int64_t k_strides[3],
                     const int64_t out_q_strides[3], const int64_t out_k_strides[3],
                     int64_t cs_stride, int32_t pos_offset, int32_t dtype, int32_t cs_dtype,
                     int32_t backward, void* stream);
 
 /*
- * Plain device-to-device copy kernel (128-bit loads/stores, same launch shape as
- * the softmax kernels).  Measurement aid: gives the HBM copy rate and the
- * counter calibration the roofline figures are scaled against.  nbytes % 16 == 0.
+ * The same rotation given as angles: freqs is fp32 [>= pos_offset + s, d_rot] with rows of
+ * stride freqs_stride elements, and cos(freqs), sin(freqs) are evaluated inside the kernel in
+ * fp32 (sincosf, once per position and dim, shared by all heads).  Everything else as
+ * neox_rope_apply.
+ * Replaces fused_rotary_positional_embedding.forward / backward
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.cpp:38-81
+ *   megatron/fused_kernels/fused_rotary_positional_embedding.h:26-124 (sincosf in the kernel)
  */
-int neox_copy_bytes(void* dst, const void* src, int64_t nbytes, void* stream);
-
-/*
- * Measurement aid: loads the first span_bytes of every stride_bytes of buf (n_spans times) and
- * stores them back unchanged -- the memory pattern of an in-place partial rotary (e.g. 64 of
- * every 256 bytes) without its arithmetic.  Shows what that pattern costs on this memory system
- * whatever the kernel around it does.  span_bytes, stride_bytes: multiples of 16.
- */
-int neox_touch_strided(void* buf, int64_t n_spans, int32_t span_bytes, int64_t stride_bytes, void* stream);
+int neox_rope_apply_freqs(void* out_q, void* out_k, const void* q, const void* k, const float* freqs,
+                          int32_t s, int32_t b, int32_t h_q, int32_t h_k, int32_t d_rot, int32_t d,
+                          const int64_t q_strides[3], const int64_t k_strides[3],
+                          const int64_t out_q_strides[3], const int64_t out_k_strides[3],
+                          int64_t freqs_stride, int32_t pos_offset, int32_t dtype, int32_t backward,
+                          void* stream);
 
 #ifdef __cplusplus
 }

@@ -170,6 +170,14 @@ def rotary_tables(dim, seq_len, base=10000, precision=torch.float):
     return cos.to(precision), sin.to(precision)
 
 
+def rotary_tables_from_freqs(freqs):
+    """cos/sin of fp32 angles ``[s, 1, 1, d2]``, evaluated in fp32: what the ``freqs`` variant of
+    the fused rotary evaluates per element inside its kernel.
+    Follows megatron/fused_kernels/fused_rotary_positional_embedding.h:47-49, 95-98."""
+    freqs = freqs.float()
+    return freqs.cos(), freqs.sin()
+
+
 def rotate_half(x):
     """Follows megatron/model/positional_embeddings.py:103-107."""
     x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2 :]

@@ -89,15 +89,21 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     st = (ctypes.c_int64 * 3)(64, 32, 8)
     neg = (ctypes.c_int64 * 3)(64, -32, 8)
     rope = lib.neox_rope_apply
-    assert rope(p, None, p, None, None, p, 4, 1, 2, 0, 8, st, None, st, None, 8, 0, F16, F32, 0, None) == -1
-    assert rope(p, p, p, None, p, p, 4, 1, 2, 2, 8, st, st, st, st, 8, 0, F16, F32, 0, None) == -1
-    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 7, st, None, st, None, 8, 0, F16, F32, 0, None) == -3
-    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, neg, None, st, None, 8, 0, F16, F32, 0, None) == -4
-    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 4, 0, F16, F32, 0, None) == -4
-    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 8, 0, F16, BF16, 0, None) == -2
-    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, st, None, st, None, 8, -1, F16, F32, 0, None) == -3
-    assert lib.neox_copy_bytes(p, p, 24, None) == -3
-    assert lib.neox_copy_bytes(None, p, 32, None) == -1
+    assert rope(p, None, p, None, None, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, F32, 0, None) == -1
+    assert rope(p, p, p, None, p, p, 4, 1, 2, 2, 8, 8, st, st, st, st, 8, 0, F16, F32, 0, None) == -1
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 7, 8, st, None, st, None, 8, 0, F16, F32, 0, None) == -3
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, neg, None, st, None, 8, 0, F16, F32, 0, None) == -4
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 4, 0, F16, F32, 0, None) == -4
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, BF16, 0, None) == -2
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, -1, F16, F32, 0, None) == -3
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 6, st, None, st, None, 8, 0, F16, F32, 0, None) == -3
+    assert b"smaller than d_rot" in lib.neox_fused_last_error()
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, 9, 0, None) == -2
+    freqs = lib.neox_rope_apply_freqs
+    assert freqs(p, None, p, None, None, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, 0, None) == -1
+    assert freqs(p, None, p, None, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 4, 0, F16, 0, None) == -4
+    assert b"freqs row stride" in lib.neox_fused_last_error()
+    assert freqs(p, None, p, None, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F32, 0, None) == -2
 
 
 def test_last_error_is_kept_per_thread():

@@ -124,3 +124,17 @@ def test_partial_rotary_passes_remaining_dims_through():
     oq, ok = R.partial_rotary(q, k, cos, sin, 4)
     assert torch.equal(oq[..., 4:], q[..., 4:]) and torch.equal(ok[..., 4:], k[..., 4:])
     assert not torch.equal(oq[1:, ..., :4], q[1:, ..., :4])
+
+
+def test_tables_from_freqs_are_fp32_cos_and_sin_of_the_angles():
+    # pins rotary_tables_from_freqs: against float64 cos/sin of the same fp32 angles (1 ulp of
+    # fp32 at magnitude 1, angles up to thousands of radians), and against rotary_tables, which
+    # forms the same angles itself
+    freqs = torch.outer(torch.arange(4096).float(), 1.0 / (10000 ** (torch.arange(0, 32, 2).float() / 32)))
+    freqs = torch.cat((freqs, freqs), -1)[:, None, None, :]
+    cos, sin = R.rotary_tables_from_freqs(freqs)
+    assert cos.dtype == torch.float32 and cos.shape == freqs.shape
+    assert (cos.double() - freqs.double().cos()).abs().max().item() <= 1.2e-7
+    assert (sin.double() - freqs.double().sin()).abs().max().item() <= 1.2e-7
+    c2, s2 = R.rotary_tables(32, 4096)
+    assert torch.equal(cos, c2) and torch.equal(sin, s2)

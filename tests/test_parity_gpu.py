@@ -652,9 +652,13 @@ def test_fused_rope_extension_api(device, dtype, transpose):
     freqs = torch.outer(torch.arange(s, device=device).float(),
                         1.0 / (10000 ** (torch.arange(0, d2, 2, device=device).float() / d2)))
     freqs = torch.cat((freqs, freqs), -1)[:, None, None, :]
+    # (the kernel evaluates sincosf itself: two fp32 evaluations of cos/sin may differ in the last
+    # bit, so the bar is 1 ulp of the storage type; tests/test_fused_rope_gpu.py covers this path)
     out2 = rope_ext.forward(t, freqs, transpose)
     w2, _ = R.partial_rotary(t.float(), t.float(), freqs.cos(), freqs.sin(), d2)
-    assert torch.equal(out2, w2.to(dtype))
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    assert ((out2.float() - w2).abs() <= ulp * w2.abs() + 1e-6).all()
+    assert torch.equal(out2[..., d2:], t[..., d2:])
 
 
 def test_rotary_in_place_on_views_of_a_fused_qkv_buffer(device):
@@ -1293,16 +1297,28 @@ def test_one_lane_rows_at_any_alignment(device, offset):
 
 
 def test_measurement_aids_copy_and_strided_touch(device):
-    lib = _lib.lib()
+    # the benchmark's probes (their own library, not part of the product ABI) leave memory as the
+    # measurements assume: the copy copies, every strided variant stores back what it loaded
+    import bench
+
+    probes = bench.load_probes()
     stream = torch.cuda.current_stream().cuda_stream
     src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=device)
     dst = torch.zeros_like(src)
-    _lib.check(lib.neox_copy_bytes(dst.data_ptr(), src.data_ptr(), src.numel() - 16, stream))
+    assert probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(), src.numel() - 16, stream) == 0
     assert torch.equal(dst[:-16], src[:-16]) and (dst[-16:] == 0).all()
     before = src.clone()
-    _lib.check(lib.neox_touch_strided(src.data_ptr(), 4096, 64, 256, stream))  # loads and stores back
-    _lib.check(lib.neox_touch_strided(src.data_ptr(), 1, 4096, 4096, stream))
+    for threads in (256, 1024):
+        for in_flight in (4, 8):
+            for load, store in ((64, 64), (64, 0), (128, 64), (128, 128)):
+                assert probes.neox_probe_strided(src.data_ptr(), 4096, load, store, 256, threads, in_flight, stream) == 0
+            assert probes.neox_probe_strided(src.data_ptr(), 1, 4096, 4096, 4096, threads, in_flight, stream) == 0
+    assert probes.neox_probe_empty(stream) == 0
     assert torch.equal(src, before)
+    assert probes.neox_probe_strided(src.data_ptr(), 4096, 0, 64, 256, 256, 4, stream) == 0  # store only
+    torch.cuda.synchronize()
+    assert probes.neox_probe_strided(src.data_ptr(), 4096, 24, 64, 256, 256, 4, stream) == -3
+    assert probes.neox_probe_strided(src.data_ptr(), 4096, 64, 64, 256, 512, 4, stream) == -3
 
 
 def test_mask_and_bias_tensors_beyond_4_gib(device):
