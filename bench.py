@@ -724,26 +724,234 @@ def main():
                 unfused.append(r)
                 del t
             result["unfused_reference_branches_on_this_gpu"] = unfused
-        # what the memory pattern of the partial rotary costs by itself: the first 64 of every 256
-        # bytes of a 134 MB buffer loaded and stored back (cfg3's q and k), and the same number of
-        # bytes as one contiguous run
+        # What the memory pattern of the in-place partial rotary costs by itself (cfg3: the first 64
+        # of every 256 bytes of q and k, 134 MB, loaded and stored back), probed with several launch
+        # shapes and split into its streams, next to dense patterns that move the same useful bytes
+        # or the same HBM traffic (whole 128-byte lines are fetched: 128 B read + 64 B written per
+        # span).  `bytes` counts the bytes a row's accesses ask for.
         if want("pattern"):
-            probes = []
-            bufs = [torch.empty(2 * 2048 * 4 * 32 * 256, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(10)]
+            pr = []
             n_spans = 2 * 2048 * 4 * 32
+            bufs = [torch.empty(n_spans * 256, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(10)]
 
-            def strided(t):
-                ok(lib.neox_touch_strided(t.data_ptr(), n_spans, 64, 256, stream))
+            def strided(ld, st_, stride, threads=256, in_flight=4, spans=n_spans):
+                return lambda t: ok(probes.neox_probe_strided(t.data_ptr(), spans, ld, st_, stride, threads,
+                                                              in_flight, stream))
 
-            def dense(t):
-                ok(lib.neox_touch_strided(t.data_ptr(), 1, n_spans * 64, n_spans * 64, stream))
+            def prow(name, nbytes, fn):
+                pr.append(row("pattern probe: " + name, nbytes, *time_launches(fn, bufs, 200)))
 
-            probes.append(row("pattern probe: 64 of every 256 bytes, load + store back (cfg3's accesses)",
-                              2 * n_spans * 64, *time_launches(strided, bufs, 200)))
-            probes.append(row("pattern probe: the same bytes contiguous", 2 * n_spans * 64,
-                              *time_launches(dense, bufs, 200)))
-            result["memory_pattern_probes"] = probes
+            u = n_spans * 64
+            prow("64 of every 256 B, load + store back (cfg3's accesses), 256-thread blocks, 4 in flight", 2 * u,
+                 strided(64, 64, 256))
+            prow("the same, 1024-thread blocks", 2 * u, strided(64, 64, 256, 1024, 4))
+            prow("the same, 256-thread blocks, 8 in flight (half as many blocks)", 2 * u, strided(64, 64, 256, 256, 8))
+            prow("the same, 1024-thread blocks, 8 in flight", 2 * u, strided(64, 64, 256, 1024, 8))
+            prow("64 of every 256 B stored, the whole 128-byte line requested by the loads", 3 * u, strided(128, 64, 256))
+            prow("64 of every 256 B, load only", u, strided(64, 0, 256))
+            prow("64 of every 256 B, store only", u, strided(0, 64, 256))
+            prow("128 of every 256 B, load + store back (whole lines, half of the pages)", 4 * u, strided(128, 128, 256))
+            prow("the same useful bytes contiguous (33.5 MB loaded and stored back)", 2 * u,
+                 strided(4096, 4096, 4096, spans=u // 4096))
+            prow("the same HBM traffic contiguous (67 MB of lines loaded, half of each stored back)", 3 * u,
+                 strided(128, 64, 128))
+            pr.append(row("empty kernel, back-to-back launches", 0,
+                          *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200)))
+            result["memory_pattern_probes"] = pr
             del bufs
+            # cfg3 forward replayed from a HIP graph of 20 launches over distinct buffer sets: the
+            # kernel's time without the host's launch path between consecutive launches
+            S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1247, nsets=10)
+            side = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                stream_side = side.cuda_stream
+
+                def rope_on_side(t):
+                    ok(lib.neox_rope_apply(t["q"].data_ptr(), t["k"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
+                                           t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, t["st"], t["st"],
+                                           t["st"], t["st"], DR, 0, BF16, F32, 0, stream_side))
+
+                rope_on_side(s_[0])
+                side.synchronize()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(20):
+                        rope_on_side(s_[i % 10])
+            torch.cuda.synchronize()
+            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+            med, best = time_launches(lambda t: graph.replay(), [None], 20, warm=3)
+            result["cfg3_from_a_hip_graph"] = row("cfg3 rotary fwd q+k, 20 launches per graph replay", nb, med / 20, best / 20)
+            del s_, graph
+        # The drop-in where it is dropped in: the Python modules the attention layer calls
+        # (megatron/model/transformer.py:534 FusedScaleMaskSoftmax.forward, :850-856
+        # apply_rotary_pos_emb, :844-848 fused_apply_rotary_pos_emb_cached) -- module -> autograd
+        # Function -> ctypes -> C-ABI -> kernel.  Per row: us per call of back-to-back calls
+        # (HIP events, as above: the GPU-side cost when the host keeps ahead), the C-ABI figure of the
+        # same work from the table, and the host's own time per call (wall clock of calls on a
+        # tiny input of the same kind, where the kernel is negligible).
+        if want("module"):
+            from gpt_neox_amd.fused_rope import fused_apply_rotary_pos_emb_cached
+            from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+            from gpt_neox_amd.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_qkv_
+
+            def mask_fill(scores, mask_):
+                return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+
+            abi_us = {r["op"]: r["us_per_call"] for r in table}
+            mrows = []
+
+            def events_us(fn, n, warm=3):
+                m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+                return m
+
+            def host_us(fn, n=2000):
+                for _ in range(50):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                dt = time.perf_counter() - t0
+                torch.cuda.synchronize()
+                return dt / n * 1e6
+
+            def mrow(name, f_us, fb_us, host_f, host_fb, keys):
+                r = {"op": name, "module_fwd_us": round(f_us, 2), "host_fwd_us": round(host_f, 2)}
+                if fb_us is not None:
+                    r["module_fwd_bwd_us"] = round(fb_us, 2)
+                    r["host_fwd_bwd_us"] = round(host_fb, 2)
+                have = [abi_us.get(k) for k in keys]
+                if have and have[0] is not None:
+                    r["c_abi_fwd_us"] = have[0]
+                    if len(have) > 1 and have[1] is not None:
+                        r["c_abi_fwd_bwd_us"] = round(have[0] + have[1], 2)
+                mrows.append(r)
+
+            def softmax_module_row(name, shape, dt, sc, fusion, mask_, keys, n, with_bwd=True):
+                mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, fusion, mask_fill, True, sc)
+                x = (torch.randn(shape[0], shape[1], shape[2], shape[3], device=dev, generator=gen(81)) * 8).to(dt) \
+                    if shape[0] * shape[1] * shape[2] * shape[3] < 2 ** 30 else None
+                if x is None:  # chunked: no full-size fp32 temporary
+                    x = torch.empty(shape, device=dev, dtype=dt)
+                    for j in range(0, shape[1], 8):
+                        x[:, j : j + 8] = (torch.randn(x[:, j : j + 8].shape, device=dev, generator=gen(81 + j)) * 8).to(dt)
+                mod(x[:1, :1], mask_[:1])  # the mask's verdict is decided before the timed calls
+                with torch.no_grad():
+                    f_us = events_us(lambda: mod(x, mask_), n)
+                fb_us = host_fb = None
+                tiny = x[:1, :1, :16, :16].contiguous()
+                tmask = mask_[:1, :, :16, :16].contiguous()
+                mod(tiny, tmask)
+                with torch.no_grad():
+                    host_f = host_us(lambda: mod(tiny, tmask))
+                if with_bwd:
+                    xg = x.requires_grad_(True)
+                    g = torch.empty_like(x).normal_()
+
+                    def fb():
+                        mod(xg, mask_).backward(g)
+                        xg.grad = None
+
+                    fb_us = events_us(fb, n)
+                    tg = tiny.clone().requires_grad_(True)
+                    gg = torch.ones_like(tiny)
+
+                    def tiny_fb():
+                        mod(tg, tmask).backward(gg)
+                        tg.grad = None
+
+                    host_fb = host_us(tiny_fb)
+                mrow(name, f_us, fb_us, host_f, host_fb, keys)
+
+            softmax_module_row("cfg1 FusedScaleMaskSoftmax(upper_triang) [4,12,2048,2048] bf16", (4, 12, 2048, 2048),
+                               torch.bfloat16, 0.125, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                               ["cfg1 causal fwd [48,2048,2048] bf16"], 50, with_bwd=False)
+            lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(82))
+            pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+            softmax_module_row("cfg2 FusedScaleMaskSoftmax(general) [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale,
+                               SoftmaxFusionTypes.general, pad,
+                               ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 50)
+            softmax_module_row("cfg4 FusedScaleMaskSoftmax(upper_triang) [1,64,2048,2048] fp16", (1, 64, 2048, 2048),
+                               torch.float16, 96 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                               ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 50)
+            torch.cuda.empty_cache()
+            if not args.quick:
+                softmax_module_row("cfg5 FusedScaleMaskSoftmax(upper_triang) [1,32,8192,8192] bf16", (1, 32, 8192, 8192),
+                                   torch.bfloat16, 128 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(8192),
+                                   ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 10)
+                torch.cuda.empty_cache()
+            # a mask the module has not seen: the device-side comparison with the plain triangle and,
+            # with causal_mask_check="verify", the wait for it (paid once per new mask tensor)
+            fresh_rows = {}
+            for mode in ("verify", "lazy", "trust"):
+                mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, mask_fill, True, 0.125,
+                                            causal_mask_check=mode)
+                x = (torch.randn(1, 1, 8192, 8192, device=dev, generator=gen(83)) * 8).bfloat16()
+                big = causal_mask(8192)
+                mod(x, big)
+                torch.cuda.synchronize()
+                walls = []
+                for _ in range(5):
+                    fresh = big.clone()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    mod(x, fresh)
+                    t1 = time.perf_counter()
+                    torch.cuda.synchronize()
+                    walls.append(((t1 - t0) * 1e6, (time.perf_counter() - t0) * 1e6))
+                fresh_rows[mode] = {"host_returns_after_us": round(statistics.median(w[0] for w in walls), 1),
+                                    "gpu_done_after_us": round(statistics.median(w[1] for w in walls), 1)}
+                del x, big
+            result["module_call_with_a_fresh_causal_mask_1x1x8192x8192"] = fresh_rows
+
+            # rotary through the modules: cfg3 (partial) and cfg5 (full)
+            for label, S, Bb, H, HN, DR, keys in (
+                    ("cfg3", 2048, 4, 32, 128, 32, ["cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32",
+                                                    "cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32"]),
+                    ("cfg5", 8192, 1, 32, 128, 128, ["cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128",
+                                                     "cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128"])):
+                sets_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1250, nsets=6)
+                cos4, sin4 = sets_[0]["cos"].view(S, 1, 1, DR), sets_[0]["sin"].view(S, 1, 1, DR)
+                it = [0]
+
+                def nxt():
+                    it[0] += 1
+                    return sets_[it[0] % 6]
+
+                def sliced():  # what the attention layer does: slice, rotate (new tensors), caller concatenates
+                    t = nxt()
+                    return apply_rotary_pos_emb(t["q"][..., :DR], t["k"][..., :DR], cos4, sin4)
+
+                def fused_rope_path():  # rope_fusion: one call per tensor, pass-through dims copied in the kernel
+                    t = nxt()
+                    return fused_apply_rotary_pos_emb_cached(t["q"], cos4, sin4), fused_apply_rotary_pos_emb_cached(t["k"], cos4, sin4)
+
+                tq = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+                tk = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+                tc, ts_ = cos4[:4].contiguous(), sin4[:4].contiguous()
+                with torch.no_grad():
+                    f_us = events_us(sliced, 200)
+                    hf = host_us(lambda: apply_rotary_pos_emb(tq[..., :DR], tk[..., :DR], tc, ts_))
+                    mrow(f"{label} apply_rotary_pos_emb(q[..., :{DR}], k[..., :{DR}], cos, sin) [{S},{Bb},{H},{HN}] bf16",
+                         f_us, None, hf, None, keys[:1])
+                    f_us = events_us(fused_rope_path, 200)
+                    hf = host_us(lambda: fused_apply_rotary_pos_emb_cached(tq, tc, ts_))
+                    mrow(f"{label} fused_apply_rotary_pos_emb_cached(q) + (k): whole heads out of place "
+                         f"[{S},{Bb},{H},{HN}] bf16 d2={DR}; host figure per call", f_us, None, hf, None, [])
+                # in place on the fused QKV projection [s, b, np, 3*hn]: q and k thirds rotated, no copies
+                mixed = [torch.randn(S, Bb, H, 3 * HN, device=dev, generator=gen(1251 + i)).bfloat16() for i in range(4)]
+                tmixed = torch.randn(4, 1, 2, 3 * HN, device=dev).bfloat16()
+                with torch.no_grad():
+                    def qkv_in_place():
+                        it[0] += 1
+                        return apply_rotary_pos_emb_qkv_(mixed[it[0] % 4], cos4, sin4, 0, DR)
+
+                    f_us = events_us(qkv_in_place, 200)
+                    hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
+                mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
+                del sets_, mixed
+            result["module_api"] = mrows
         result["all_configs"] = table
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
         if pcts:

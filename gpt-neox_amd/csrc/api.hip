@@ -55,8 +55,8 @@ static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset,
     d.state = device_state;
     d.seed_lo = (uint32_t)seed;
     d.seed_hi = (uint32_t)(seed >> 32);
-    d.off_lo = (uint32_t)offset;
-    d.off_hi = (uint32_t)(offset >> 32);
+    d.off_lo = (uint32_t)(offset >> 2);  // the Philox block the offset lies in (4 outputs per block)
+    d.off_hi = (uint32_t)(offset >> 34);
     d.threshold = (uint32_t)__builtin_rint((double)p * 65536.0);
     const float keep = (float)(1.0 - (double)p);
     d.scale = p >= 1.f ? 0.f : (float)(1.0 / (double)keep);

@@ -2,11 +2,13 @@
 // attention-dropout kernels.
 //
 // Eight consecutive elements of the score tensor (one 128-bit access) share one Philox
-// block: counter = (offset_lo, offset_hi, group_lo, group_hi) with group = element index / 8,
-// key = (seed_lo, seed_hi).  This is the counter layout of torch's device generator with
-// the group index in the place of the subsequence, so a call that takes the generator's
-// (seed, offset) and advances the offset never overlaps another consumer of that
-// generator.  Element e owns the 16-bit field (word[e/2] >> 16*(e%2)) & 0xffff and is kept
+// block: counter = (c_lo, c_hi, group_lo, group_hi) with c = offset / 4 and group = element
+// index / 8, key = (seed_lo, seed_hi).  This is the counter layout of torch's device generator
+// with the group index in the place of the subsequence: a generator offset counts 32-bit
+// outputs, four to a block, so a consumer that owns the offsets [o, o + n) draws from the
+// counter values [o / 4, (o + n) / 4).  A call that takes the generator's (seed, offset) and
+// advances the offset by 4 therefore owns exactly one counter value, disjoint from what every
+// earlier and later consumer of that generator draws.  Element e owns the 16-bit field (word[e/2] >> 16*(e%2)) & 0xffff and is kept
 // iff field >= threshold, threshold = round(p * 65536): the drop probability is honoured
 // to 2^-16.
 #pragma once
@@ -17,7 +19,7 @@ namespace neox {
 
 struct DropoutArgs {
     uint32_t seed_lo, seed_hi;  // Philox key
-    uint32_t off_lo, off_hi;    // low half of the counter
+    uint32_t off_lo, off_hi;    // low half of the counter: generator offset / 4
     uint32_t threshold;         // 0 .. 65536
     float scale;                // 1/(1-p), 0 for p = 1
     // If not null: {seed, offset} in device memory, read when the kernel runs instead of the
@@ -29,11 +31,11 @@ struct DropoutArgs {
 // The parameters a kernel works with: the by-value ones, or those in device memory.
 __device__ __forceinline__ DropoutArgs resolve(DropoutArgs d) {
     if (d.state != nullptr) {
-        const uint64_t seed = d.state[0], offset = d.state[1];  // wave-uniform loads
+        const uint64_t seed = d.state[0], block = d.state[1] >> 2;  // wave-uniform loads
         d.seed_lo = (uint32_t)seed;
         d.seed_hi = (uint32_t)(seed >> 32);
-        d.off_lo = (uint32_t)offset;
-        d.off_hi = (uint32_t)(offset >> 32);
+        d.off_lo = (uint32_t)block;
+        d.off_hi = (uint32_t)(block >> 32);
     }
     return d;
 }

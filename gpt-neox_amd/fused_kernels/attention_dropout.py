@@ -14,8 +14,9 @@ import torch
 
 from .. import _lib
 
-# One Philox counter value per group of 8 elements is consumed at the offset taken;
-# torch keeps generator offsets at multiples of 4.
+# A generator offset counts 32-bit outputs, four to a Philox counter value; a fused call draws
+# every group's block at the one counter value offset / 4 and so owns the offsets
+# [offset, offset + 4).  torch keeps generator offsets at multiples of 4.
 OFFSET_STEP = 4
 # Offsets drawn from the device-resident state (HIP graphs) start far above anything the
 # host-side generator reaches, so the two never draw from the same counter.

@@ -19,13 +19,19 @@ Deliberate differences from the reference:
   runs the torch path beyond it) and need none of the ``sq % 4``,
   ``attn_batches % 4`` or ``% batch_per_block`` divisibility rules, which were
   artefacts of the CUDA launch shape -- see :meth:`is_kernel_available`;
-* the causal branch checks once per mask tensor that the mask really is the plain
-  upper-triangular one and otherwise (sliding-window masks, packed-sequence masks)
-  runs the mask-tensor kernel with the mask it was given -- the reference's causal
-  kernel ignores the mask's contents, so above its 2048 limit (torch path) and below
-  it (fused kernel) the reference computes two different things for such masks; here
-  both agree with the torch path; a causal-fusion call with ``sq != sk`` (a step against a
-  key/value cache, where the reference asserts) also runs the mask-tensor kernel;
+* by default the causal branch checks once per mask (per storage region, so ``detach()``ed
+  aliases share the verdict) that the mask really is the plain upper-triangular one and
+  otherwise (sliding-window masks, packed-sequence masks) runs the mask-tensor kernel with
+  the mask it was given -- the reference's causal kernel ignores the mask's contents, so
+  above its 2048 limit (torch path) and below it (fused kernel) the reference computes two
+  different things for such masks; here both agree with the torch path.  The constructor's
+  ``causal_mask_check`` selects how: ``"verify"`` (default) waits for the device-side
+  comparison the first time a mask is seen (one host synchronisation per new mask),
+  ``"lazy"`` never synchronises -- calls made while the comparison is in flight run the
+  mask-tensor kernel, which is right for any mask -- and ``"trust"`` restores the
+  reference's behaviour of never reading the mask
+  (megatron/model/fused_softmax.py:173-179).  A causal-fusion call with ``sq != sk`` (a step
+  against a key/value cache, where the reference asserts) also runs the mask-tensor kernel;
 * masked scores are excluded, so their probability is exactly 0 as in the torch
   path (the reference's padded kernel fills -10000), and a fully masked row is
   uniform ``1/sk`` as in the torch path;
@@ -84,43 +90,97 @@ def _recall(ctx):
     return probs, ctx.scale
 
 
+class _MaskVerdict:
+    """One remembered mask region: the storage it lives in (weakly), the version counter it had,
+    and the verdict -- True / False, or None while the device-side comparison is still running
+    (then ``pending`` holds the pinned result slot and the event that follows the copy)."""
+
+    __slots__ = ("storage", "version", "verdict", "pending")
+
+    def __init__(self, storage, version, verdict=None, pending=None):
+        self.storage = weakref.ref(storage)
+        self.version = version
+        self.verdict = verdict
+        self.pending = pending
+
+    def poll(self, wait):
+        if self.verdict is None and self.pending is not None:
+            slot, event = self.pending
+            if wait:
+                event.synchronize()
+            if wait or event.query():
+                self.verdict = bool(slot.item())  # host memory, the copy has finished: no sync
+                self.pending = None
+        return self.verdict
+
+
 class _CausalMaskMemo:
-    """Remembers, per live mask tensor, whether it equals ``triu(ones, 1)``.
+    """Remembers, per mask region, whether it equals ``triu(ones, 1)``.
 
-    The verdict costs one pass over the mask and one host synchronisation; the attention
-    mask of a training step is one tensor shared by all layers, so it is paid once per
-    step.  Entries are keyed by the tensor object (weak reference) and its version
-    counter, never by address, so a recycled allocation cannot inherit a verdict."""
+    A region is (storage address, offset, shape, strides); an entry is valid while the storage
+    object it was decided for is alive (weak reference -- a recycled allocation is another
+    storage object and cannot inherit a verdict) and the tensor's version counter is unchanged
+    (in-place writes bump it).  Aliases of one mask -- ``mask.detach()``, which activation
+    checkpointing applies to its inputs for every recomputed segment, or an equal view --
+    share the storage, the region and the version counter, hence the verdict.  (A write through
+    ``.data`` or from outside torch bumps no counter and is not seen.)
 
-    def __init__(self, limit=16):
+    The comparison runs on the device.  ``is_plain_causal(mask, wait=True)`` waits for it (one
+    host synchronisation per new mask); with ``wait=False`` it returns None while the result is
+    on its way and the caller uses a kernel that is right for any mask in the meantime."""
+
+    def __init__(self, limit=64):
         self._entries = {}
         self._limit = limit
+        self._slots = None  # pinned result slots, handed out in turn
+        self._next_slot = 0
 
-    def lookup(self, mask):
-        """The remembered verdict for this tensor in its current version, or None."""
-        hit = self._entries.get(id(mask))
-        if hit is not None:
-            ref, version, verdict = hit
-            if ref() is mask and version == mask._version:
-                return verdict
+    @staticmethod
+    def _key(mask):
+        storage = mask.untyped_storage()
+        return (storage.data_ptr(), mask.storage_offset(), tuple(mask.shape), mask.stride()), storage
+
+    def _entry(self, mask):
+        key, storage = self._key(mask)
+        hit = self._entries.get(key)
+        if hit is not None and hit.storage() is storage and hit.version == mask._version:
+            return hit
         return None
 
-    def is_plain_causal(self, mask):
-        verdict = self.lookup(mask)
-        if verdict is not None:
-            return verdict
+    def lookup(self, mask, wait=False):
+        """The verdict for this region in its current version: True, False, or None if it is
+        unknown (never asked, or still being computed and ``wait`` is False)."""
+        hit = self._entry(mask)
+        return None if hit is None else hit.poll(wait)
+
+    def _result_slot(self):
+        if self._slots is None:
+            self._slots = torch.zeros(256, dtype=torch.bool, pin_memory=True)
+        self._next_slot = (self._next_slot + 1) % self._slots.numel()
+        return self._slots[self._next_slot : self._next_slot + 1]
+
+    def is_plain_causal(self, mask, wait=True):
+        hit = self._entry(mask)
+        if hit is not None:
+            return hit.poll(wait)
         sq, sk = mask.shape[-2], mask.shape[-1]
-        cols = torch.arange(sk, device=mask.device)
-        rows = torch.arange(sq, device=mask.device)
-        expected = cols[None, :] > rows[:, None]
-        verdict = bool(torch.equal(mask.bool().expand(mask.shape[0], 1, sq, sk),
-                                   expected.expand(mask.shape[0], 1, sq, sk)))
+        expected = torch.ones(sq, sk, dtype=torch.bool, device=mask.device).triu_(1)
+        same = (mask.bool() == expected).all()  # a 0-dim tensor on the mask's device
+        key, storage = self._key(mask)
+        if mask.is_cuda:
+            slot = self._result_slot()
+            slot.copy_(same.view(1), non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+            entry = _MaskVerdict(storage, mask._version, pending=(slot, event))
+        else:
+            entry = _MaskVerdict(storage, mask._version, verdict=bool(same))
         if len(self._entries) >= self._limit:
-            self._entries = {k: v for k, v in self._entries.items() if v[0]() is not None}
+            self._entries = {k: v for k, v in self._entries.items() if v.storage() is not None}
             if len(self._entries) >= self._limit:
                 self._entries.clear()
-        self._entries[id(mask)] = (weakref.ref(mask), mask._version, verdict)
-        return verdict
+        self._entries[key] = entry
+        return entry.poll(wait)
 
 
 _causal_memo = _CausalMaskMemo()
@@ -303,14 +363,20 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     mask_func: ``mask_func(scores, mask) -> scores`` used by the torch branch.
     softmax_in_fp32: torch branch computes in fp32 (the kernels always do).
     scale: multiplier applied before the softmax, or None.
+    causal_mask_check (not in the reference): ``"verify"`` | ``"lazy"`` | ``"trust"`` -- how the
+        upper_triang fusion treats the mask it is given; see the module text.
 
     Reference: megatron/model/fused_softmax.py:92-205.
     """
 
-    def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale):
+    def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
+                 causal_mask_check="verify"):
         super().__init__()
         assert fusion_type in list(SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
         assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
+        assert causal_mask_check in ("verify", "lazy", "trust"), f"Invalid causal_mask_check {causal_mask_check}"
+        # how upper_triang fusion makes sure that the mask is the plain triangle (see the module text)
+        self.causal_mask_check = causal_mask_check
 
         self.input_in_fp16 = input_in_fp16
         self.input_in_bf16 = input_in_bf16
@@ -349,7 +415,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
             input = input + bias
         if alibi_slopes is not None:
             b, np, sq, sk = input.size()
-            if fused and self.upper_triang_mask_fusion and self.mask_is_plain_causal(mask):
+            if fused and self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask):
                 scale = 1.0 if self.scale is None else self.scale
                 return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
             input = input + alibi_bias(alibi_slopes, sq, sk, input.device, input.dtype)
@@ -427,17 +493,20 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
         return probs.view(b, np, sq, sk)
 
-    @staticmethod
-    def mask_is_plain_causal(mask):
-        """True if ``mask`` hides exactly the keys ``j > i``.  Decided once per mask tensor
-        (see ``_CausalMaskMemo``).  While a HIP graph is being captured the check cannot
-        synchronise: a mask decided before the capture keeps its verdict, for any other the
-        answer is False and the mask-tensor kernel is used."""
+    def mask_is_plain_causal(self, mask):
+        """True if the causal kernel may serve ``mask``: it hides exactly the keys ``j > i``
+        (``"verify"``, ``"lazy"``; decided once per mask region, see ``_CausalMaskMemo``), or
+        without looking (``"trust"``).  ``"lazy"`` answers False while the comparison is still
+        running.  While a HIP graph is being captured nothing can be compared: a mask decided
+        before the capture keeps its verdict, for any other the answer is False and the
+        mask-tensor kernel is used."""
+        if self.causal_mask_check == "trust":
+            return True
         if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
             return False
         if mask.is_cuda and torch.cuda.is_current_stream_capturing():
             return bool(_causal_memo.lookup(mask))
-        return _causal_memo.is_plain_causal(mask)
+        return bool(_causal_memo.is_plain_causal(mask, wait=self.causal_mask_check == "verify"))
 
     def forward_torch_softmax(self, input, mask):
         """The unfused path: optional upcast, scale, ``mask_func``, softmax, cast back."""

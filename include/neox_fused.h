@@ -134,12 +134,13 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
  * which is what torch.nn.Dropout computes from y; y_drop must not alias y.  Backward
  * takes dy = the gradient of y_drop, regenerates the keep pattern and returns
  *   dx = scale * y * (g - sum_j(g*y)),  g = keep ? dy / (1-p) : 0  (fp32, never stored).
- * Keep pattern: Philox4x32-10 with key = seed and counter = (offset, e / 8), e the
+ * Keep pattern: Philox4x32-10 with key = seed and counter = (offset / 4, e / 8), e the
  * row-major element index into the score tensor; element e owns the 16-bit field e % 8 of
  * its block and is kept iff field >= round(p * 65536).  neox_dropout_keep_mask writes that
  * pattern as bytes (1 = kept) for n elements.  (seed, offset) are the device generator's
- * Philox state; a call consumes one counter value per group, so the caller advances the
- * generator's offset by 4 (torch's granularity) per call.  0 <= p <= 1.
+ * Philox state, whose offset counts 32-bit outputs, four to a counter value; a call draws
+ * from the one counter value offset / 4, so the caller advances the generator's offset by 4
+ * per call and no other consumer of the generator draws the same blocks.  0 <= p <= 1.
  * The forward entry points take x as [b, np, sq, sk] and two optional additions to the scores,
  * NULL when absent: alibi_slopes (causal only, as neox_causal_softmax_alibi_fwd) or a bias tensor
  * [bias_b, np, sq, sk] (as neox_*_softmax_bias_fwd), not both.

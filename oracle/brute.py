@@ -103,11 +103,12 @@ def philox4x32_10(counter, key):
 def keep_element(e, p, seed, offset):
     """Whether the element with row-major index ``e`` survives a dropout of probability ``p``
     drawn from Philox state ``(seed, offset)``: its group of 8 shares the block with counter
-    ``(offset, e // 8)``; the element owns 16 bits of it and is kept iff they are not below
+    ``(offset // 4, e // 8)``; the element owns 16 bits of it and is kept iff they are not below
     ``round(p * 65536)``."""
     group = e // 8
+    block = offset // 4
     words = philox4x32_10(
-        [offset & 0xFFFFFFFF, offset >> 32, group & 0xFFFFFFFF, group >> 32],
+        [block & 0xFFFFFFFF, block >> 32, group & 0xFFFFFFFF, group >> 32],
         [seed & 0xFFFFFFFF, seed >> 32],
     )
     field = (words[(e % 8) // 2] >> (16 * (e % 2))) & 0xFFFF

@@ -13,8 +13,9 @@ can compare the kernels' keep pattern bit for bit.
   lines) and against this image's ``torch.rand`` on the GPU, which consumes the same block
   function.
 * ``keep_mask``: element ``e`` (row-major index into the score tensor) belongs to group
-  ``e // 8``; the group's 128-bit block is ``philox(counter=(offset_lo, offset_hi,
-  group_lo, group_hi), key=(seed_lo, seed_hi))``; element ``e`` owns the 16-bit field
+  ``e // 8``; the group's 128-bit block is ``philox(counter=(c_lo, c_hi, group_lo,
+  group_hi), key=(seed_lo, seed_hi))`` with ``c = offset // 4`` (a generator offset counts
+  32-bit outputs, four to a block, as in torch's device generator); element ``e`` owns the 16-bit field
   ``(word[(e % 8) // 2] >> (16 * (e % 2))) & 0xffff`` and is kept iff
   ``field >= threshold(p)``, ``threshold = round(p * 65536)``.
 """
@@ -64,8 +65,9 @@ def keep_mask(n, p, seed, offset):
     groups = (n + 7) // 8
     g = np.arange(groups, dtype=np.uint64)
     ctr = np.empty((groups, 4), dtype=np.uint64)
-    ctr[:, 0] = np.uint64(offset & 0xFFFFFFFF)
-    ctr[:, 1] = np.uint64((offset >> 32) & 0xFFFFFFFF)
+    block = offset >> 2  # the Philox block the generator offset lies in
+    ctr[:, 0] = np.uint64(block & 0xFFFFFFFF)
+    ctr[:, 1] = np.uint64((block >> 32) & 0xFFFFFFFF)
     ctr[:, 2] = g & _LO
     ctr[:, 3] = g >> _S32
     words = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF))  # [groups, 4]

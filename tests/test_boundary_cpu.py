@@ -242,7 +242,8 @@ def test_is_kernel_available_table():
 def test_plain_causal_mask_detection_and_memo():
     from oracle import torch_ref as R
 
-    f = FusedScaleMaskSoftmax.mask_is_plain_causal
+    mod = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None)
+    f = mod.mask_is_plain_causal
     plain = R.get_attn_mask(9)
     assert f(plain) and f(plain)
     assert f(plain.expand(3, 1, 9, 9).contiguous()) and f(plain.to(torch.uint8))
@@ -253,8 +254,54 @@ def test_plain_causal_mask_detection_and_memo():
     assert f(per_sample)
     per_sample[1, 0, 8, 0] = True  # version bump: the remembered verdict is dropped
     assert not f(per_sample)
-    for _ in range(40):  # the memo stays bounded and correct under churn
+    for _ in range(100):  # the memo stays bounded and correct under churn
         assert f(R.get_attn_mask(5))
+
+
+def test_aliases_of_a_mask_share_its_verdict():
+    # activation checkpointing detach()es its inputs for every recomputed segment: each layer
+    # then sees a new tensor object over the same storage, which must not cost a new comparison
+    from gpt_neox_amd import fused_softmax as fs
+    from oracle import torch_ref as R
+
+    mod = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None)
+    memo = fs._causal_memo
+    plain = R.get_attn_mask(12)
+    assert memo.lookup(plain) is None  # never asked
+    assert mod.mask_is_plain_causal(plain)
+    for alias in (plain.detach(), plain.view(1, 1, 12, 12), plain[:], plain.detach().detach()):
+        assert alias is not plain and memo.lookup(alias) is True
+    assert memo.lookup(plain[..., :11, :11]) is None  # another region of the same storage
+    assert memo.lookup(plain.clone()) is None          # another storage
+    window = R.get_attn_mask(12, sliding_window_width=3)
+    assert not mod.mask_is_plain_causal(window) and memo.lookup(window.detach()) is False
+    alias = plain.detach()
+    alias[0, 0, 11, 0] = True  # a write through an alias bumps the shared version counter
+    assert memo.lookup(plain) is None and not mod.mask_is_plain_causal(plain)
+    # a recycled allocation is another storage object: no verdict is inherited
+    addr = window.untyped_storage().data_ptr()
+    del window, alias
+    for _ in range(20):
+        fresh = torch.zeros(1, 1, 12, 12, dtype=torch.bool)
+        if fresh.untyped_storage().data_ptr() == addr:
+            assert memo.lookup(fresh) is None
+            break
+
+
+def test_causal_mask_check_modes():
+    from oracle import torch_ref as R
+
+    def module(mode):
+        return FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None, causal_mask_check=mode)
+
+    window = R.get_attn_mask(7, sliding_window_width=2)
+    assert not module("verify").mask_is_plain_causal(window)
+    assert not module("lazy").mask_is_plain_causal(window)  # CPU masks are decided at once
+    assert module("lazy").mask_is_plain_causal(R.get_attn_mask(7))
+    assert module("trust").mask_is_plain_causal(window)  # the reference never reads the mask
+    assert FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None).causal_mask_check == "verify"
+    with pytest.raises(AssertionError):
+        module("sometimes")
 
 
 def test_reference_predicate_restated():
@@ -289,8 +336,11 @@ def test_public_names_and_signatures_match_the_reference_modules():
     def params(fn):
         return list(inspect.signature(fn).parameters)
 
+    # the reference's positional parameters, plus one optional keyword that defaults to checking
     assert params(FusedScaleMaskSoftmax.__init__) == [
-        "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale"]
+        "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale",
+        "causal_mask_check"]
+    assert inspect.signature(FusedScaleMaskSoftmax.__init__).parameters["causal_mask_check"].default == "verify"
     # the reference's positional parameters, plus three optional additions that default to "off"
     assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask", "alibi_slopes", "dropout_p", "bias"]
     assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["bias"].default is None

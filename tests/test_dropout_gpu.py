@@ -72,6 +72,17 @@ def test_oracle_philox_agrees_with_the_device_library_generator(device):
     words = philox.philox4x32_10(ctr, (987654321, 0)).astype(np.float64)  # [256, 4]
     want = words[:, 0] / 2.0**32  # element t <- first word of thread t's first block
     assert np.abs(u - want).max() < 2.0**-23
+    # a generator offset counts 32-bit outputs, four to a counter value: at offset 400 the same
+    # launch draws at counter 100 -- the kernels' keep pattern uses offset / 4 likewise, so a call
+    # that owns the offsets [o, o + 4) shares no block with any other consumer
+    torch.cuda.default_generators[device.index].set_offset(400)
+    u = torch.rand(256, device=device, dtype=torch.float32).cpu().numpy().astype(np.float64)
+    ctr[:, 0] = 100
+    words = philox.philox4x32_10(ctr, (987654321, 0)).astype(np.float64)
+    assert np.abs(u - words[:, 0] / 2.0**32).max() < 2.0**-23
+    got = rng.keep_mask(2048, 0.5, 987654321, 400, device).cpu().numpy()
+    fields = philox.philox4x32_10(ctr, (987654321, 0))[:, 0] & 0xFFFF  # element 8 t <- low half of word 0
+    assert np.array_equal(got[0::8], fields >= 32768)
 
 
 def test_dropout_scale_is_the_device_library_s(device):

@@ -371,6 +371,45 @@ def test_causal_module_honours_masks_that_are_not_plain_causal(device):
         assert max_err(fused(x, plain), R.softmax_fp32(x, plain, 0.25)) <= TOL[dtype]
 
 
+def test_causal_mask_check_lazy_and_trust(device):
+    # "lazy": no host synchronisation -- while the device-side comparison of a new mask is in
+    # flight the mask-tensor kernel serves the call (right for any mask), afterwards the causal
+    # kernel; "trust": the mask is never read, as in megatron/model/fused_softmax.py:173-179
+    from gpt_neox_amd import fused_softmax as fs
+
+    s, dtype = 520, torch.bfloat16
+    x = scores((2, 3, s, s), dtype, device, 91)
+    g = normal((2, 3, s, s), dtype, device, 92)
+    mods = {m: FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func,
+                                     True, 0.25, causal_mask_check=m) for m in ("verify", "lazy", "trust")}
+    plain = R.get_attn_mask(s, device)
+    want = R.softmax_fp32(x, plain, 0.25)
+    ref = mods["verify"](x, plain)
+    assert max_err(ref, want) <= TOL[dtype]
+    for fresh in (plain.clone(), plain.clone()):
+        assert fs._causal_memo.lookup(fresh) is None
+        first = mods["lazy"](x, fresh)  # verdict possibly still in flight
+        torch.cuda.synchronize()
+        assert fs._causal_memo.lookup(fresh) is True  # arrived: read without a synchronisation
+        assert fs._causal_memo.lookup(fresh.detach()) is True
+        second = mods["lazy"](x, fresh)
+        assert torch.equal(first, ref) and torch.equal(second, ref)  # both kernels give the same bits
+    window = R.get_attn_mask(s, device, sliding_window_width=5)
+    for _ in range(2):
+        out = mods["lazy"](x, window)
+        assert max_err(out, R.softmax_fp32(x, window, 0.25)) <= TOL[dtype]
+        torch.cuda.synchronize()
+    assert fs._causal_memo.lookup(window) is False
+    # trust: the window mask is ignored, the plain triangle applied
+    assert torch.equal(mods["trust"](x, window), ref)
+    # gradients through the lazy module, first call (mask-tensor kernels) and later (causal kernels)
+    dx_want = R.softmax_backward_fp32(g, ref, 0.25)
+    for fresh in (plain.clone(), plain):
+        xin = x.clone().requires_grad_(True)
+        mods["lazy"](xin, fresh).backward(g.clone())
+        assert max_err(xin.grad, dx_want) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(2, 4, 8), (1, 6, 40), (2, 3, 136), (1, 8, 520), (2, 2, 1000), (1, 4, 2048),
                                    (1, 2, 2568), (1, 2, 4104), (1, 3, 37)])
