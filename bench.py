@@ -55,7 +55,8 @@ def parse():
     ap.add_argument("--quick", action="store_true",
                     help="few launches per table row (for counter-collection runs)")
     ap.add_argument("--only", type=str, default=None,
-                    help="run only the table rows whose name contains this text (profiling aid)")
+                    help="run only the table rows whose name contains this text, or one of several texts "
+                         "separated by commas (profiling aid)")
     return ap.parse_args()
 
 
@@ -441,7 +442,7 @@ def main():
         table = []
 
         def want(name):
-            return args.only is None or args.only in name
+            return args.only is None or any(part in name for part in args.only.split(","))
 
         def tri(n):
             return n * (n + 1) // 2
@@ -477,6 +478,38 @@ def main():
             r = row("cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
                     *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
             table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
+            # the same rotation as the attention layer's call receives it (megatron/model/transformer.py:
+            # 826-856): the first 32 dims sliced off as views, new dense tensors returned; its backward
+            # pass works on dense gradients.  Same algorithmic bytes, dense writes.
+            for z in s_:
+                z["oq"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+                z["ok"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+                z["ost"] = _lib.strides3(z["oq"])
+
+            def rope_sliced(t, backward):
+                src_q, src_k, st_in = (t["oq"], t["ok"], t["ost"]) if backward else (t["q"], t["k"], t["st"])
+                ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), src_q.data_ptr(), src_k.data_ptr(),
+                                       t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, st_in, st_in,
+                                       t["ost"], t["ost"], DR, 0, BF16, F32, backward, stream))
+
+            table.append(row("cfg3 rotary fwd q+k, rotary dims sliced off as views [2048,4,32,:32], dense tensors out", nb,
+                             *time_launches(lambda t: rope_sliced(t, 0), s_, 200)))
+            table.append(row("cfg3 rotary bwd q+k, dense gradients [2048,4,32,32] in place", nb,
+                             *time_launches(lambda t: rope_sliced(t, 1), s_, 200)))
+            # the rope_fusion path (megatron/model/transformer.py:844-848): whole heads out of place, the
+            # pass-through dims copied by the same launch; reads and writes all of q and k
+            for z in s_:
+                z.pop("ok"), z.pop("ost")
+                z["oq"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+                z["ok"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+
+            def rope_whole(t):
+                ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
+                                       t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, HN, t["st"], t["st"],
+                                       t["st"], t["st"], DR, 0, BF16, F32, 0, stream))
+
+            table.append(row("cfg3 rotary fwd q+k, whole heads out of place with the pass-through dims copied (rope_fusion)",
+                             2 * 2 * S * Bb * H * HN * 2 + 2 * S * DR * 4, *time_launches(rope_whole, s_, 200)))
             del s_
         # configs[3]: 20B shape
         if want("cfg4"):

@@ -46,10 +46,36 @@ static hipError_t with_runtime_flags(const SoftmaxArgs& a, Launch&& launch) {
     return launch(std::integral_constant<int, EXTRA>{});
 }
 
+#ifndef NEOX_XCD_AFFINITY
+#define NEOX_XCD_AFFINITY 1
+#endif
+
+// Switches the XCD-aware block -> unit mapping on (see xcd_slot) when the work units of a block
+// -- `units` of them, `unit_bytes` each, consecutive in memory -- tile 4 KiB pieces exactly and
+// the output starts on a 4 KiB boundary.
+static SoftmaxArgs with_xcd_mapping(const SoftmaxArgs& a, uint64_t unit_bytes, uint32_t units, uint32_t blocks) {
+    SoftmaxArgs b = a;
+    b.units_per_piece = 0;
+    b.affine_blocks = 0;
+#if NEOX_XCD_AFFINITY
+    const bool aligned = (reinterpret_cast<uintptr_t>(a.out) & 4095u) == 0 &&
+                         (a.out2 == nullptr || (reinterpret_cast<uintptr_t>(a.out2) & 4095u) == 0);
+    if (aligned && unit_bytes > 0 && unit_bytes <= 4096 && 4096 % unit_bytes == 0 && blocks >= 8) {
+        const uint32_t upp = (uint32_t)(4096 / unit_bytes);
+        if (units % upp == 0 && units / upp >= 1) {
+            b.units_per_piece = upp;
+            b.affine_blocks = blocks & ~7u;
+        }
+    }
+#endif
+    return b;
+}
+
 template <typename T, Mask M, bool BWD, int EXTRA, int NCH, int WPR, int RPB>
-static hipError_t launch_shape(const SoftmaxArgs& a, hipStream_t st) {
-    const dim3 grid((a.rows + RPB - 1) / RPB);
+static hipError_t launch_shape(const SoftmaxArgs& a0, hipStream_t st) {
+    const dim3 grid((a0.rows + RPB - 1) / RPB);
     const dim3 block(kWave * WPR * RPB);
+    const SoftmaxArgs a = with_xcd_mapping(a0, (uint64_t)a0.sk * 2, RPB, grid.x);
     return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
         constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
         if constexpr (BWD) {
@@ -74,9 +100,13 @@ static hipError_t launch_generic(const SoftmaxArgs& a, hipStream_t st) {
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA, int G, int R, int C>
-static hipError_t launch_packed_shape(const SoftmaxArgs& a, hipStream_t st) {
+static hipError_t launch_packed_shape(const SoftmaxArgs& a0, hipStream_t st) {
     const uint32_t per_block = Packed<G, R>::kRowsPerBlock;
-    const dim3 grid((a.rows + per_block - 1) / per_block);
+    const dim3 grid((a0.rows + per_block - 1) / per_block);
+    // the unit is a wave's run of rows: 4 waves per block.  Not for the full-row backward with
+    // several chunks per lane group: two loads per store, and the order measured 0-2 % slower there.
+    const uint64_t unit_bytes = (BWD && C > 1) ? 0 : (uint64_t)Packed<G, R>::kRowsPerWave * a0.sk * 2;
+    const SoftmaxArgs a = with_xcd_mapping(a0, unit_bytes, 4, grid.x);
     return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
         constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
         if constexpr (BWD) {
@@ -190,6 +220,9 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if (chunks > 24 && chunks <= 28) return launch_shape<T, M, BWD, EXTRA, 4, 8, 1>(a, st);
     }
     if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
+#if NEOX_RPB_8192 == 2
+    if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 2>(a, st);
+#endif
     if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);
     if (chunks <= 32) return launch_shape<T, M, BWD, EXTRA, 2, 16, 1>(a, st);
     if (chunks <= 48) return launch_shape<T, M, BWD, EXTRA, 3, 16, 1>(a, st);

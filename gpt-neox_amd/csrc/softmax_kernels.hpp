@@ -43,9 +43,17 @@ struct SoftmaxArgs {
     const void* bias;              // kBias forward: additive bias [1 or b, np, sq, sk], dtype of x
     uint32_t bias_rows;            // np*sq if the bias is shared by all samples, else 0
     uint32_t bias_bytes;           // size of the bias tensor, 0 if it does not fit 32 bits
+    // Block -> memory mapping that keeps every XCD on its own 4 KiB pieces (see xcd_slot), filled in
+    // by the launchers: work units (rows, or the rows of a wave) per 4 KiB piece, 0 = units in order
+    uint32_t units_per_piece;
+    uint32_t affine_blocks;        // leading blocks that take part: a multiple of 8
 };
 
 enum class Mask { Causal, Bytes, None };
+
+#ifndef NEOX_PAIR_ROWS
+#define NEOX_PAIR_ROWS 0
+#endif
 
 // Compile-time switches of the kernels (FLAGS): two memory hints and three optional features.
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
@@ -165,6 +173,23 @@ __device__ __forceinline__ uint32_t keep_bits_row8(const DropoutArgs& d, uint32_
     }
 }
 
+// Which work unit a block processes.  Workgroups are handed to the 8 XCDs of the chip in turn
+// (block b runs on XCD b % 8), and the memory system sustains a write stream best when every XCD
+// keeps to its own 4 KiB pieces of the address space, piece index = XCD (mod 8): a plain store
+// kernel measured 83 % of the HBM peak with that mapping against 70-75 % when a block stores
+// several consecutive pieces or the pieces rotate over the XCDs (loads do not care).  So where the
+// units of a block (U of them: rows, or the row groups of its waves) tile 4 KiB pieces exactly,
+// `upp` units per piece, the blocks of a group of 8 share the 8 * U units of the group like this:
+// block x of the group takes the pieces x, x + 8, x + 16, ... instead of U / upp consecutive ones.
+// Returns the unit index for unit l of block b; the identity for the last, incomplete group.
+__device__ __forceinline__ uint32_t xcd_slot(uint32_t b, uint32_t l, uint32_t U, const SoftmaxArgs& a) {
+    const uint32_t upp = a.units_per_piece;
+    if (upp == 0 || b >= a.affine_blocks) return b * U + l;
+    const uint32_t g = b >> 3, x = b & 7u;
+    const uint32_t j = l / upp, t = l - j * upp;  // piece of the block, unit inside the piece
+    return (g * 8u * (U / upp) + j * 8u + x) * upp + t;
+}
+
 // Where a wave works: the row, its position i inside its [sq, sk] matrix, the number of
 // columns that take part, and whether the result is stored (surplus waves of the last
 // block recompute the last row and store nothing, so that every wave of a block reaches
@@ -182,6 +207,16 @@ __device__ __forceinline__ RowPos locate(uint32_t row, const SoftmaxArgs& a) {
     p.store = row < a.rows;
     p.row = p.store ? row : a.rows - 1;
     p.i = p.row % (uint32_t)a.sq;
+#if NEOX_PAIR_ROWS
+    if constexpr (MASK == Mask::Causal) {
+        // short rows and long rows in turn: slot r of a matrix is row r/2 from the top (r even)
+        // or from the bottom (r odd)
+        const uint32_t r = p.i, sq = (uint32_t)a.sq;
+        const uint32_t i2 = (r & 1u) ? sq - 1u - (r >> 1) : (r >> 1);
+        p.row = p.row - r + i2;
+        p.i = i2;
+    }
+#endif
     p.len = (MASK == Mask::Causal) ? min((int)p.i + 1, a.sk) : a.sk;
     return p;
 }
@@ -226,7 +261,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     const float ninf = -__builtin_inff();
     // byte offset of the lane inside the row, first chunk of its wave.  Everything goes into
     // the per-lane offset: the hardware's range check does not see the scalar offset operand.
-    const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    const RowPos pos = locate<MASK>(xcd_slot(blockIdx.x, rib, RPB, a), a);
     // kRagged: the row lies one position later on the lanes when it starts on an odd element
     int sh = 0;
     if constexpr (kRag) sh = ragged_shift(a.in0, pos.row, sk);
@@ -434,7 +469,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     const int rib = wib / WPR;
     const int wir = wib % WPR;
     const int sk = a.sk;
-    const RowPos pos = locate<MASK>(blockIdx.x * RPB + rib, a);
+    const RowPos pos = locate<MASK>(xcd_slot(blockIdx.x, rib, RPB, a), a);
     // kRagged: the row lies one position later on the lanes when it starts on an odd element; the
     // position in front of it stays zero in both tensors and is never stored
     int sh = 0;
@@ -640,7 +675,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     constexpr bool kRag = (FLAGS & kRagged) != 0;
     static_assert(!kRag || C == 1, "ragged rows: one chunk per lane group");
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wave = xcd_slot(blockIdx.x, __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), 4, a);
     const uint32_t row0 = wave * RPW;  // first row of this wave
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
@@ -776,7 +811,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     constexpr bool kRag = (FLAGS & kRagged) != 0;
     static_assert(!kRag || C == 1, "ragged rows: one chunk per lane group");
     const int lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t wave = xcd_slot(blockIdx.x, __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), 4, a);
     const uint32_t row0 = wave * RPW;
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);

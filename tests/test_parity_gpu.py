@@ -371,6 +371,53 @@ def test_causal_module_honours_masks_that_are_not_plain_causal(device):
         assert max_err(fused(x, plain), R.softmax_fp32(x, plain, 0.25)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("sk", [64, 128, 256, 512, 1024, 2048])
+def test_xcd_aware_block_order_covers_every_row_once(device, sk):
+    # Rows of 4096 / 2^k bytes: the kernels hand the 4 KiB pieces of the tensors to their blocks so
+    # that block x of every group of 8 keeps to the pieces x, x + 8, ... (one XCD, one piece
+    # residue).  Whatever the order, every row must be computed exactly once -- with a grid that
+    # is not a multiple of 8 blocks, a last block that is only partly filled, and several matrices.
+    dtype = torch.float16
+    for batches, sq in ((3, 1000), (5, 333), (1, 77)):
+        x = scores((batches, sq, sk), dtype, device, 7 + sk)
+        g = normal((batches, sq, sk), dtype, device, 8 + sk)
+        causal = torch.ones(sq, sk, dtype=torch.bool, device=device).triu_(1)
+        y = causal_ext.forward(x, 0.25)
+        assert max_err(y, R.softmax_fp32(x, causal, 0.25)) <= TOL[dtype]
+        assert (y[:, causal] == 0).all()
+        dx = causal_ext.backward(g.clone(), y, 0.25)
+        assert max_err(dx, R.softmax_backward_fp32(g, y, 0.25)) <= TOL[dtype]
+        lens = torch.randint(1, sk + 1, (batches,), device=device, generator=gen(device, sk))
+        mask = R.padding_mask(lens, sq, sk, device)
+        x4 = x.view(batches, 1, sq, sk).expand(batches, 2, sq, sk).contiguous()
+        y4 = masked_ext.forward(x4, mask, 0.25)
+        assert max_err(y4, R.softmax_fp32(x4, mask, 0.25)) <= TOL[dtype]
+        assert (y4[mask.expand_as(y4)] == 0).all()
+        g4 = g.view(batches, 1, sq, sk).expand(batches, 2, sq, sk).contiguous()
+        dx4 = masked_ext.backward(g4.clone(), y4, 0.25)
+        assert max_err(dx4, R.softmax_backward_fp32(g4, y4, 0.25)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("shape,d_rot", [((37, 3, 16, 128), 32), ((37, 3, 16, 128), 128), ((129, 1, 24, 64), 64),
+                                         ((50, 2, 8, 256), 64), ((9, 5, 32, 128), 32)])
+def test_rotary_piece_order_covers_every_head_once(device, shape, d_rot):
+    # dense q and k whose heads tile 4 KiB pieces take the XCD-aware kernel: unit counts that are
+    # not a multiple of a block's 8 units or of a group of 8 blocks, in place and out of place
+    s, b, h, hn = shape
+    dtype = torch.bfloat16
+    q, k = normal(shape, dtype, device, 3), normal(shape, dtype, device, 4)
+    cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + 5))
+    want_q, want_k = R.partial_rotary(q.float(), k.float(), cos, sin, d_rot, offset=5)
+    q1, k1 = q.clone(), k.clone()
+    apply_rotary_pos_emb_(q1, k1, cos, sin, 5, d_rot)
+    assert torch.equal(q1, want_q.to(dtype)) and torch.equal(k1, want_k.to(dtype))
+    out = rope_ext.forward_cached(q, cos[5 : 5 + s], sin[5 : 5 + s], False)
+    assert torch.equal(out, want_q.to(dtype))
+    gq, gk = R.rotary_autograd_fp32(q[..., :d_rot], k[..., :d_rot], cos, sin, q[..., :d_rot], k[..., :d_rot], offset=5)
+    back = rope_ext.backward_cached(q, cos[5 : 5 + s], sin[5 : 5 + s], False)
+    assert torch.equal(back[..., :d_rot], gq.to(dtype)) and torch.equal(back[..., d_rot:], q[..., d_rot:])
+
+
 def test_causal_mask_check_lazy_and_trust(device):
     # "lazy": no host synchronisation -- while the device-side comparison of a new mask is in
     # flight the mask-tensor kernel serves the call (right for any mask), afterwards the causal
