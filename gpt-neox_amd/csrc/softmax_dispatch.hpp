@@ -220,9 +220,6 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if (chunks > 24 && chunks <= 28) return launch_shape<T, M, BWD, EXTRA, 4, 8, 1>(a, st);
     }
     if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
-#if NEOX_RPB_8192 == 2
-    if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 2>(a, st);
-#endif
     if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);
     if (chunks <= 32) return launch_shape<T, M, BWD, EXTRA, 2, 16, 1>(a, st);
     if (chunks <= 48) return launch_shape<T, M, BWD, EXTRA, 3, 16, 1>(a, st);

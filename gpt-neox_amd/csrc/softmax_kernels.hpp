@@ -51,9 +51,6 @@ struct SoftmaxArgs {
 
 enum class Mask { Causal, Bytes, None };
 
-#ifndef NEOX_PAIR_ROWS
-#define NEOX_PAIR_ROWS 0
-#endif
 
 // Compile-time switches of the kernels (FLAGS): two memory hints and three optional features.
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
@@ -207,16 +204,6 @@ __device__ __forceinline__ RowPos locate(uint32_t row, const SoftmaxArgs& a) {
     p.store = row < a.rows;
     p.row = p.store ? row : a.rows - 1;
     p.i = p.row % (uint32_t)a.sq;
-#if NEOX_PAIR_ROWS
-    if constexpr (MASK == Mask::Causal) {
-        // short rows and long rows in turn: slot r of a matrix is row r/2 from the top (r even)
-        // or from the bottom (r odd)
-        const uint32_t r = p.i, sq = (uint32_t)a.sq;
-        const uint32_t i2 = (r & 1u) ? sq - 1u - (r >> 1) : (r >> 1);
-        p.row = p.row - r + i2;
-        p.i = i2;
-    }
-#endif
     p.len = (MASK == Mask::Causal) ? min((int)p.i + 1, a.sk) : a.sk;
     return p;
 }

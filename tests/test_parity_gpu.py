@@ -30,6 +30,7 @@ from gpt_neox_amd.positional_embeddings import (
     apply_rotary_pos_emb_qkv_,
     apply_rotary_pos_emb_torch,
 )
+from gpt_neox_amd.fused_kernels.attention_dropout import keep_mask as rng_keep
 from oracle import torch_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -396,6 +397,41 @@ def test_xcd_aware_block_order_covers_every_row_once(device, sk):
         g4 = g.view(batches, 1, sq, sk).expand(batches, 2, sq, sk).contiguous()
         dx4 = masked_ext.backward(g4.clone(), y4, 0.25)
         assert max_err(dx4, R.softmax_backward_fp32(g4, y4, 0.25)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batches,sq,sk", [(3, 4096, 4096), (2, 8192, 8192), (5, 100, 4096), (2, 5000, 6144),
+                                           (1, 9000, 8192), (3, 2052, 16384), (7, 8, 8192)])
+def test_long_causal_rows_store_every_piece_exactly_once(device, dtype, batches, sq, sk):
+    # rows of several KiB, most of them zeros above the diagonal, in matrices that are square, wide
+    # and tall.  Outputs pre-filled with NaN: every element must have been written, the zeros
+    # included; forward, backward and the two outputs of the dropout forward.
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    code = _lib.dtype_code(dtype)
+    x = scores((batches, sq, sk), dtype, device, 13)
+    g = normal((batches, sq, sk), dtype, device, 14)
+    hidden = torch.ones(sq, sk, dtype=torch.bool, device=device).triu_(1)
+    y = torch.full_like(x, float("nan"))
+    _lib.check(lib.neox_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), 0.125, batches, sq, sk, code, stream))
+    assert not torch.isnan(y).any() and (y[:, hidden] == 0).all()
+    for m in range(batches):
+        assert max_err(y[m], R.softmax_fp32(x[m], hidden, 0.125)) <= TOL[dtype]
+    dx = torch.full_like(x, float("nan"))
+    _lib.check(lib.neox_causal_softmax_bwd(dx.data_ptr(), g.data_ptr(), y.data_ptr(), 0.125, batches, sq, sk, code, stream))
+    assert not torch.isnan(dx).any() and (dx[:, hidden] == 0).all()
+    for m in range(batches):
+        assert max_err(dx[m], R.softmax_backward_fp32(g[m], y[m], 0.125)) <= TOL[dtype]
+    y1, y2 = torch.full_like(x, float("nan")), torch.full_like(x, float("nan"))
+    _lib.check(lib.neox_causal_softmax_dropout_fwd(y2.data_ptr(), y1.data_ptr(), x.data_ptr(), None, None, 0, 0.125, 0.25,
+                                                   77, 8, None, batches, 1, sq, sk, code, stream))
+    assert torch.equal(y1, y) and not torch.isnan(y2).any() and (y2[:, hidden] == 0).all()
+    keep = rng_keep(y.numel(), 0.25, 77, 8, device).view(y.shape)
+    assert torch.equal(y2, R.dropout_with_mask(y, keep, 0.25))
+    # in place (the reference overwrites the gradient): the zero pieces are written, not left
+    buf = g.clone()
+    _lib.check(lib.neox_causal_softmax_bwd(buf.data_ptr(), buf.data_ptr(), y.data_ptr(), 0.125, batches, sq, sk, code, stream))
+    assert torch.equal(buf, dx)
 
 
 @pytest.mark.parametrize("shape,d_rot", [((37, 3, 16, 128), 32), ((37, 3, 16, 128), 128), ((129, 1, 24, 64), 64),
