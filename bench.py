@@ -984,6 +984,18 @@ def main():
                     hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
                 mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
                 del sets_, mixed
+            # for scale: what the host spends on torch's own smallest differentiable step
+            tx = torch.randn(16, 16, device=dev, dtype=torch.float16, requires_grad=True)
+            tgg = torch.ones_like(tx)
+
+            def torch_floor():
+                (tx * 2.0).backward(tgg)
+                tx.grad = None
+
+            with torch.no_grad():
+                floor_f = host_us(lambda: tx * 2.0)
+            mrows.append({"op": "torch's own floor on this host: y = x * 2 (forward), then y.backward(g)",
+                          "host_fwd_us": round(floor_f, 2), "host_fwd_bwd_us": round(host_us(torch_floor), 2)})
             result["module_api"] = mrows
         result["all_configs"] = table
         pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]

@@ -163,12 +163,30 @@ def device_guard(tensor):
     return torch.cuda.device(tensor.device)
 
 
+try:  # the raw handle of torch's current stream without building a Stream object (a few us less)
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:  # pragma: no cover - older/newer torch without the private accessor
+    _raw_stream = None
+
+
 def current_stream(tensor):
     """hipStream_t of torch's current stream on the tensor's device, as an integer."""
+    if _raw_stream is not None:
+        return _raw_stream(tensor.device.index)
     return torch.cuda.current_stream(tensor.device).cuda_stream
 
 
+_strides3_cache = {}
+
+
 def strides3(t):
-    """First three element strides of a 4-D tensor as a C int64[3]."""
+    """First three element strides of a 4-D tensor as a C int64[3] (read-only for the callee, so
+    one array per distinct stride triple is kept and reused)."""
     s = t.stride()
-    return (ctypes.c_int64 * 3)(s[0], s[1], s[2])
+    key = (s[0], s[1], s[2])
+    arr = _strides3_cache.get(key)
+    if arr is None:
+        if len(_strides3_cache) > 4096:
+            _strides3_cache.clear()
+        arr = _strides3_cache[key] = (ctypes.c_int64 * 3)(*key)
+    return arr

@@ -486,10 +486,16 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
             # from the mask itself
             if bias is not None:
                 return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale)
+            if not (torch.is_grad_enabled() and input.requires_grad):
+                return _masked_ext.forward(input, mask, _fp32(scale))
             return ScaledMaskedSoftmax.apply(input, mask, scale)
         if bias is not None:
             return ScaledUpperTriangMaskedSoftmaxBias.apply(input, bias, scale)
         # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
+        if not (torch.is_grad_enabled() and input.requires_grad):
+            # nothing to record: straight to the extension (the autograd Function costs the host
+            # several microseconds per call)
+            return _causal_ext.forward(input.view(-1, sq, sk), _fp32(scale)).view(b, np, sq, sk)
         probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
         return probs.view(b, np, sq, sk)
 

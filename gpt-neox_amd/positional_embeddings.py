@@ -130,6 +130,8 @@ def _rotary_torch(q, k, cos, sin, offset):
 
 def _as_table(t, d_rot, need_rows):
     """View a ``[seq, 1, 1, d]`` (or ``[seq, d]``) table as rows the kernel can index."""
+    if t.dim() == 2 and t.shape[1] == d_rot and t.shape[0] >= need_rows and t.stride(1) == 1 and t.stride(0) >= d_rot:
+        return t  # already rows (the tables the autograd Functions keep for their backward pass)
     if t.shape[-1] != d_rot or t.numel() != t.shape[0] * d_rot:
         raise RuntimeError(
             f"cos/sin must have shape [seq, 1, 1, {d_rot}], got {tuple(t.shape)}"
@@ -148,19 +150,37 @@ def _dense_last(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
+def _on(t, device):
+    """``t`` on ``device``; the tensor itself when it is already there (the usual case, and
+    cheaper than asking ``Tensor.to`` to find that out)."""
+    return t if t.device == device else t.to(device)
+
+
+def _needs_grad(*tensors):
+    """Whether autograd has to record the call (else the autograd Function, which costs the host
+    several microseconds per call, is bypassed)."""
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def _rotary_out_of_place(q, k, cos, sin, offset):
+    """New tensors ``rotary(q), rotary(k)`` in one launch; returns them and the table rows used."""
+    d_rot = q.shape[-1]
+    cos2 = _as_table(cos, d_rot, offset + q.shape[0])
+    sin2 = _as_table(sin, d_rot, offset + q.shape[0])
+    q, k = _dense_last(q), _dense_last(k)
+    out_q = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    out_k = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    if q.numel() or k.numel():
+        _rope_ext.rope_launch(out_q, out_k, q, k, cos2, sin2, d_rot, offset, backward=False)
+    return out_q, out_k, cos2, sin2
+
+
 class _FusedRotary(torch.autograd.Function):
     """q' , k' = rotary(q), rotary(k) in one launch; gradients in one launch."""
 
     @staticmethod
     def forward(ctx, q, k, cos, sin, offset):
-        d_rot = q.shape[-1]
-        cos2 = _as_table(cos, d_rot, offset + q.shape[0])
-        sin2 = _as_table(sin, d_rot, offset + q.shape[0])
-        q, k = _dense_last(q), _dense_last(k)
-        out_q = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        out_k = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-        if q.numel() or k.numel():
-            _rope_ext.rope_launch(out_q, out_k, q, k, cos2, sin2, d_rot, offset, backward=False)
+        out_q, out_k, cos2, sin2 = _rotary_out_of_place(q, k, cos, sin, offset)
         ctx.save_for_backward(cos2, sin2)
         ctx.offset = offset
         return out_q, out_k
@@ -199,7 +219,9 @@ def apply_rotary_pos_emb(q, k, cos, sin, offset: int = 0):
     ``offset .. offset+sq`` (megatron/model/positional_embeddings.py:110-116).
     q, k: ``[sq, b, heads, d_rot]``; cos, sin: ``[seq, 1, 1, d_rot]``."""
     if _fusable(q, k, cos, sin):
-        return _FusedRotary.apply(q, k, cos.to(q.device), sin.to(q.device), offset)
+        if not _needs_grad(q, k):
+            return _rotary_out_of_place(q, k, _on(cos, q.device), _on(sin, q.device), offset)[:2]
+        return _FusedRotary.apply(q, k, _on(cos, q.device), _on(sin, q.device), offset)
     return _rotary_torch(q, k, cos, sin, offset)
 
 
@@ -210,13 +232,18 @@ def apply_rotary_pos_emb_torch(q, k, cos, sin, offset: int = 0):
     return apply_rotary_pos_emb(q, k, cos, sin, offset)
 
 
+def _rotary_in_place(q, k, cos, sin, offset, d_rot):
+    cos2 = _as_table(cos, d_rot, offset + q.shape[0])
+    sin2 = _as_table(sin, d_rot, offset + q.shape[0])
+    if q.numel() or k.numel():
+        _rope_ext.rope_launch(q, k, q, k, cos2, sin2, d_rot, offset, backward=False)
+    return cos2, sin2
+
+
 class _FusedRotaryInplace(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, cos, sin, offset, d_rot):
-        cos2 = _as_table(cos, d_rot, offset + q.shape[0])
-        sin2 = _as_table(sin, d_rot, offset + q.shape[0])
-        if q.numel() or k.numel():
-            _rope_ext.rope_launch(q, k, q, k, cos2, sin2, d_rot, offset, backward=False)
+        cos2, sin2 = _rotary_in_place(q, k, cos, sin, offset, d_rot)
         ctx.mark_dirty(q, k)
         ctx.save_for_backward(cos2, sin2)
         ctx.offset, ctx.d_rot = offset, d_rot
@@ -247,7 +274,10 @@ def apply_rotary_pos_emb_(q, k, cos, sin, offset: int = 0, rotary_ndims=None):
         )
     if d_rot > q.shape[-1] or d_rot % 2:
         raise RuntimeError(f"rotary_ndims={d_rot} must be even and <= head size {q.shape[-1]}")
-    return _FusedRotaryInplace.apply(q, k, cos.to(q.device), sin.to(q.device), offset, d_rot)
+    if not _needs_grad(q, k):
+        _rotary_in_place(q, k, _on(cos, q.device), _on(sin, q.device), offset, d_rot)
+        return q, k
+    return _FusedRotaryInplace.apply(q, k, _on(cos, q.device), _on(sin, q.device), offset, d_rot)
 
 
 class _FusedQKVRotary(torch.autograd.Function):
@@ -302,7 +332,12 @@ def apply_rotary_pos_emb_qkv_(mixed_x_layer, cos, sin, offset: int = 0, rotary_n
             "cos/sin in fp32 or its dtype"
         )
     dev = mixed_x_layer.device
-    mixed = _FusedQKVRotary.apply(mixed_x_layer, cos.to(dev), sin.to(dev), offset, d_rot)
+    if not _needs_grad(mixed_x_layer):
+        mixed = mixed_x_layer
+        if mixed.numel():
+            _rotary_in_place(mixed[..., :hn], mixed[..., hn : 2 * hn], _on(cos, dev), _on(sin, dev), offset, d_rot)
+        return mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]
+    mixed = _FusedQKVRotary.apply(mixed_x_layer, _on(cos, dev), _on(sin, dev), offset, d_rot)
     return mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]
 
 
