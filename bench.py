@@ -95,6 +95,9 @@ def load_probes():
     h.neox_probe_empty.restype, h.neox_probe_empty.argtypes = ctypes.c_int, [vp]
     h.neox_probe_strided.restype = ctypes.c_int
     h.neox_probe_strided.argtypes = [vp, i64, i32, i32, i64, i32, i32, vp]
+    h.neox_probe_pieces.restype, h.neox_probe_pieces.argtypes = ctypes.c_int, [vp, vp, i64, i32, i32, i32, vp]
+    h.neox_probe_strided_pieces.restype = ctypes.c_int
+    h.neox_probe_strided_pieces.argtypes = [vp, i64, i32, i32, i32, vp]
     return h
 
 
@@ -790,8 +793,32 @@ def main():
                  strided(128, 64, 128))
             pr.append(row("empty kernel, back-to-back launches", 0,
                           *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200)))
+            # the same pattern by 4 KiB pieces, one piece per wave access, with the pieces of a block
+            # consecutive or 8 apart (every XCD on its own piece residue: the order the kernels use)
+            for per_wave in (1, 2):
+                for order, oname in ((0, "consecutive pieces"), (1, "pieces 8 apart (XCD-aware)")):
+                    prow(f"64 of every 256 B, load + store back, one 4 KiB piece per wave access, {per_wave} per wave, {oname}",
+                         2 * u, lambda t, pw=per_wave, od=order: ok(probes.neox_probe_strided_pieces(
+                             t.data_ptr(), n_spans * 256, 0, pw, od, stream)))
+            for op, opname in ((1, "load only"), (2, "store only")):
+                for order, oname in ((0, "consecutive pieces"), (1, "pieces 8 apart (XCD-aware)")):
+                    prow(f"64 of every 256 B, {opname}, one 4 KiB piece per wave access, 1 per wave, {oname}", u,
+                         lambda t, o=op, od=order: ok(probes.neox_probe_strided_pieces(t.data_ptr(), n_spans * 256, o, 1, od, stream)))
             result["memory_pattern_probes"] = pr
             del bufs
+            # Dense streams of 1 GiB in 4 KiB pieces against the block -> piece order: workgroups go to the
+            # 8 XCDs in turn, so "8 apart" keeps every XCD on one piece residue (mod 8), "consecutive"
+            # gives it 2 or 4 residues, "rotating" all 8.
+            xp = []
+            big = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
+            for op, opname, moved in ((0, "write", 1 << 30), (1, "read", 1 << 30), (2, "copy", 2 << 30)):
+                for per_block, order, oname in ((1, 0, "1 piece per block, in order"), (1, 2, "1 piece per block, rotating over the XCDs"),
+                                                (4, 0, "4 consecutive pieces per block"), (4, 1, "4 pieces per block, 8 apart")):
+                    xp.append(row(f"{opname} 1 GiB: {oname}", moved, *time_launches(
+                        lambda t, o=op, pb=per_block, od=order: ok(probes.neox_probe_pieces(
+                            big[0].data_ptr(), big[1].data_ptr(), 1 << 30, o, pb, od, stream)), [None], 30)))
+            result["xcd_order_probes"] = xp
+            del big
             # cfg3 forward replayed from a HIP graph of 20 launches over distinct buffer sets: the
             # kernel's time without the host's launch path between consecutive launches
             S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
