@@ -58,17 +58,10 @@ static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStr
     return hipGetLastError();
 }
 
-#ifndef NEOX_ROPE_PIECES
-#define NEOX_ROPE_PIECES 1
-#endif
-
 // Dense tensors laid out alike: the XCD-aware piece kernel (see rope_piece_kernel).  `a` comes
 // from launch_rope_span's preparation (lph, spw set).  Returns false if the shape does not qualify.
 template <typename T, typename CS, int W, bool BWD>
 static bool try_launch_rope_piece(const RopeArgs& a, int s, int n_outer, hipStream_t st, hipError_t* err) {
-#if !NEOX_ROPE_PIECES
-    return false;
-#endif
     if (std::is_same<CS, Angles>::value) return false;
     const RopeTensor& q = a.t[0];
     // [s, b, h, d] dense: head vectors `vec` elements apart in one run, in and out, q and k

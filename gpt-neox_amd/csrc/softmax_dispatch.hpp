@@ -46,10 +46,6 @@ static hipError_t with_runtime_flags(const SoftmaxArgs& a, Launch&& launch) {
     return launch(std::integral_constant<int, EXTRA>{});
 }
 
-#ifndef NEOX_XCD_AFFINITY
-#define NEOX_XCD_AFFINITY 1
-#endif
-
 // Switches the XCD-aware block -> unit mapping on (see xcd_slot) when the work units of a block
 // -- `units` of them, `unit_bytes` each, consecutive in memory -- tile 4 KiB pieces exactly and
 // the output starts on a 4 KiB boundary.
@@ -57,7 +53,6 @@ static SoftmaxArgs with_xcd_mapping(const SoftmaxArgs& a, uint64_t unit_bytes, u
     SoftmaxArgs b = a;
     b.units_per_piece = 0;
     b.affine_blocks = 0;
-#if NEOX_XCD_AFFINITY
     const bool aligned = (reinterpret_cast<uintptr_t>(a.out) & 4095u) == 0 &&
                          (a.out2 == nullptr || (reinterpret_cast<uintptr_t>(a.out2) & 4095u) == 0);
     if (aligned && unit_bytes > 0 && unit_bytes <= 4096 && 4096 % unit_bytes == 0 && blocks >= 8) {
@@ -67,7 +62,6 @@ static SoftmaxArgs with_xcd_mapping(const SoftmaxArgs& a, uint64_t unit_bytes, u
             b.affine_blocks = blocks & ~7u;
         }
     }
-#endif
     return b;
 }
 
