@@ -77,6 +77,7 @@ static bool try_launch_rope_piece(const RopeArgs& a, int s, int n_outer, hipStre
     if (n_outer > 1 && q.in_stride[1] != (int64_t)q.n_inner * vec) return false;
     if (!dense(q) || (a.nt > 1 && !dense(a.t[1]))) return false;
     if (vecs_per_pos % a.spw != 0 || vecs_per_pos > 0x7fffffff) return false;
+    if ((int64_t)a.spw * vec * 2 > 0x7fffffffLL) return false;  // a unit is addressed through one 32-bit buffer
     const int64_t units = (int64_t)s * vecs_per_pos / a.spw;
     if (units > 0x7fffffffLL || (int64_t)s * vecs_per_pos > 0xffffffffLL) return false;
     RopeArgs b = a;

@@ -396,6 +396,31 @@ __global__ __launch_bounds__(256) void rope_span_kernel(RopeArgs a) {
 // ([2048, 4, 32, 128], first 32 dims) 24.0 -> 22.5 us, full rotary [8192, 1, 32, 128] 44.5 -> 43.8 us.
 // A unit lies inside one position (vecs_per_pos % spw == 0); the cos/sin values are loaded per
 // unit unless the wave's previous unit had the same position.
+// W 16-bit elements through a range-checked buffer access (non-temporal): lanes whose offset lies
+// outside the resource load zeros / store nothing
+template <int W>
+__device__ __forceinline__ void buf_ld_words(rsrc_t r, uint32_t off, uint32_t (&w)[W / 2]) {
+    if constexpr (W == 8) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, kAuxNt);
+        w[0] = v.x, w[1] = v.y, w[2] = v.z, w[3] = v.w;
+    } else if constexpr (W == 4) {
+        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, kAuxNt);
+        w[0] = v.x, w[1] = v.y;
+    } else {
+        w[0] = __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, kAuxNt);
+    }
+}
+template <int W>
+__device__ __forceinline__ void buf_st_words(rsrc_t r, uint32_t off, const uint32_t (&w)[W / 2]) {
+    if constexpr (W == 8) {
+        __builtin_amdgcn_raw_buffer_store_b128(u32x4{w[0], w[1], w[2], w[3]}, r, (int)off, 0, kAuxNt);
+    } else if constexpr (W == 4) {
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2{w[0], w[1]}, r, (int)off, 0, kAuxNt);
+    } else {
+        __builtin_amdgcn_raw_buffer_store_b32(w[0], r, (int)off, 0, kAuxNt);
+    }
+}
+
 template <typename T, typename CS, int W, bool BWD, int ITERS>
 __global__ __launch_bounds__(256) void rope_piece_kernel(RopeArgs a) {
     static_assert(!std::is_same<CS, Angles>::value, "angles go through rope_span_kernel");
@@ -404,7 +429,6 @@ __global__ __launch_bounds__(256) void rope_piece_kernel(RopeArgs a) {
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int sw = (lane * a.lph_magic) >> 16;
     const int slot = lane - sw * lph;
-    const bool active = sw < spw;
     const bool rotated = slot < lps;
     const bool second = slot >= hl;
     const int partner = (second ? lane - hl : lane + hl) & (kWave - 1);
@@ -412,10 +436,16 @@ __global__ __launch_bounds__(256) void rope_piece_kernel(RopeArgs a) {
     const int jt = rotated ? j : 0;
     const int jp = rotated ? (second ? slot - hl : slot + hl) * W : 0;
     constexpr uint32_t U = 4 * ITERS;  // units per block
+    // A unit is addressed through buffers of exactly its bytes: the lane's offset inside the unit
+    // is the same for every unit, the surplus lanes of a wave (sw == spw) lie outside and move
+    // nothing, and no branch surrounds a memory access.
+    const uint32_t unit_bytes = (uint32_t)spw * (uint32_t)a.vec_elems * 2u;
+    const uint32_t lane_off = ((uint32_t)sw * (uint32_t)a.vec_elems + (uint32_t)j) * 2u;
 
     uint32_t xq[ITERS][W / 2], xk[ITERS][W / 2];
     float c[ITERS][W], sn[ITERS][W];
-    int64_t off[ITERS];  // element offset of the lane's slot, -1: nothing to do
+    size_t base[ITERS];    // byte offset of the unit in every tensor
+    uint32_t bytes[ITERS];  // its size, 0 past the last unit
     uint32_t upos[ITERS];
 #pragma unroll
     for (int u = 0; u < ITERS; ++u) {
@@ -430,17 +460,13 @@ __global__ __launch_bounds__(256) void rope_piece_kernel(RopeArgs a) {
             const uint32_t g = b >> 3, x = b & 7u, pj = l / upp, t = l - pj * upp;
             unit = (g * 8u * (U / upp) + pj * 8u + x) * upp + t;
         }
-        const bool live = active && unit < a.n_units;
-        const uint32_t v0 = unit * (uint32_t)spw;
-        const uint32_t pos = v0 / a.vecs_per_pos;  // wave-uniform
-        off[u] = live ? ((int64_t)(v0 + sw) * a.vec_elems + j) : -1;
-#pragma unroll
-        for (int k = 0; k < W / 2; ++k) xq[u][k] = xk[u][k] = 0u;
-        if (live) {
-            load_words<W, true>(a.t[0].in + off[u] * 2, xq[u]);
-            if (a.nt > 1) load_words<W, true>(a.t[1].in + off[u] * 2, xk[u]);
-        }
-        upos[u] = live ? pos : 0u;
+        const bool live = unit < a.n_units;  // wave-uniform
+        const uint32_t v0 = live ? unit * (uint32_t)spw : 0u;
+        base[u] = (size_t)v0 * (uint32_t)a.vec_elems * 2u;
+        bytes[u] = live ? unit_bytes : 0u;
+        buf_ld_words<W>(make_rsrc(a.t[0].in + base[u], bytes[u]), lane_off, xq[u]);
+        buf_ld_words<W>(make_rsrc(a.t[1].in + base[u], a.nt > 1 ? bytes[u] : 0u), lane_off, xk[u]);
+        upos[u] = v0 / a.vecs_per_pos;
         if (u > 0 && upos[u] == upos[u - 1]) {  // wave-uniform
 #pragma unroll
             for (int k = 0; k < W; ++k) {
@@ -480,7 +506,7 @@ __global__ __launch_bounds__(256) void rope_piece_kernel(RopeArgs a) {
                 const uint32_t packed = Elem<T>::pack(o[2 * k], o[2 * k + 1]);
                 ow[k] = rotated ? packed : x[k];
             }
-            if (off[u] >= 0 && (t == 0 || a.nt > 1)) store_words<W, true>(a.t[t].out + off[u] * 2, ow);
+            buf_st_words<W>(make_rsrc(a.t[t].out + base[u], (t == 0 || a.nt > 1) ? bytes[u] : 0u), lane_off, ow);
         }
     }
 }

@@ -201,3 +201,24 @@ def test_argument_checks_follow_the_extension(device):
         rope_ext.forward(t.cpu(), f.cpu())
     empty = rope_ext.forward(t[:0], f[:0])
     assert empty.shape == (0, 2, 2, 32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_angles_for_q_and_k_in_one_launch(device, dtype):
+    # the C-ABI's angle entry point takes q and k together (the Python extension API passes one
+    # tensor per call, as the reference does): in place over the first d2 dims, k with fewer heads
+    s, b, hq, hk, d, d2 = 70, 2, 8, 2, 64, 32
+    q, k = normal((s, b, hq, d), dtype, device, 71), normal((s, b, hk, d), dtype, device, 72)
+    freqs = angles(s + 3, d2, device)
+    cos, sin = R.rotary_tables_from_freqs(freqs)
+    want_q, want_k = R.partial_rotary(q.float(), k.float(), cos, sin, d2, offset=3)
+    q1, k1 = q.clone(), k.clone()
+    rope_ext.rope_launch(q1, k1, q1, k1, freqs.view(s + 3, d2), None, d2, 3, backward=False)
+    assert_within_one_ulp(q1, want_q.to(dtype), dtype)
+    assert_within_one_ulp(k1, want_k.to(dtype), dtype)
+    assert torch.equal(q1[..., d2:], q[..., d2:]) and torch.equal(k1[..., d2:], k[..., d2:])
+    # backward = the inverse rotation: applying it to the rotated tensors returns the inputs to 2 ulp
+    rope_ext.rope_launch(q1, k1, q1, k1, freqs.view(s + 3, d2), None, d2, 3, backward=True)
+    rot = q.float()[..., :d2]
+    pair = (rot[..., : d2 // 2] ** 2 + rot[..., d2 // 2 :] ** 2).sqrt()  # a rotation mixes the two dims of a pair
+    assert ((q1.float()[..., :d2] - rot).abs() <= 3 * ULP[dtype] * torch.cat((pair, pair), -1) + 1e-6).all()
