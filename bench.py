@@ -817,8 +817,19 @@ def main():
                     xp.append(row(f"{opname} 1 GiB: {oname}", moved, *time_launches(
                         lambda t, o=op, pb=per_block, od=order: ok(probes.neox_probe_pieces(
                             big[0].data_ptr(), big[1].data_ptr(), 1 << 30, o, pb, od, stream)), [None], 30)))
+            del big
+            # the same copy over 4 GiB per tensor (the size of the long-context score tensors): the
+            # consecutive-pieces order loses more there, the XCD-aware one does not
+            torch.cuda.empty_cache()
+            big = [torch.empty(4 << 30, dtype=torch.uint8, device=dev) for _ in range(2)]
+            big[1].random_(0, 255)
+            for per_block, order, oname in ((4, 0, "4 consecutive pieces per block"), (4, 1, "4 pieces per block, 8 apart")):
+                xp.append(row(f"copy 4 GiB: {oname}", 8 << 30, *time_launches(
+                    lambda t, pb=per_block, od=order: ok(probes.neox_probe_pieces(
+                        big[0].data_ptr(), big[1].data_ptr(), 4 << 30, 2, pb, od, stream)), [None], 10, warm=3)))
             result["xcd_order_probes"] = xp
             del big
+            torch.cuda.empty_cache()
             # cfg3 forward replayed from a HIP graph of 20 launches over distinct buffer sets: the
             # kernel's time without the host's launch path between consecutive launches
             S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
