@@ -153,10 +153,18 @@ class _CausalMaskMemo:
         hit = self._entry(mask)
         return None if hit is None else hit.poll(wait)
 
-    def _result_slot(self):
+    def _result_slot(self, entry):
+        """A pinned host byte for the verdict of ``entry``.  The slots are handed out in turn; an
+        entry that still waits for the slot's previous content reads it first (its copy finished
+        long ago), so a slot is never overwritten under an entry that has not looked yet."""
         if self._slots is None:
             self._slots = torch.zeros(256, dtype=torch.bool, pin_memory=True)
+            self._slot_owner = [None] * self._slots.numel()
         self._next_slot = (self._next_slot + 1) % self._slots.numel()
+        owner = self._slot_owner[self._next_slot]
+        if owner is not None:
+            owner.poll(wait=True)
+        self._slot_owner[self._next_slot] = entry
         return self._slots[self._next_slot : self._next_slot + 1]
 
     def is_plain_causal(self, mask, wait=True):
@@ -168,11 +176,12 @@ class _CausalMaskMemo:
         same = (mask.bool() == expected).all()  # a 0-dim tensor on the mask's device
         key, storage = self._key(mask)
         if mask.is_cuda:
-            slot = self._result_slot()
+            entry = _MaskVerdict(storage, mask._version)
+            slot = self._result_slot(entry)
             slot.copy_(same.view(1), non_blocking=True)
             event = torch.cuda.Event()
             event.record()
-            entry = _MaskVerdict(storage, mask._version, pending=(slot, event))
+            entry.pending = (slot, event)
         else:
             entry = _MaskVerdict(storage, mask._version, verdict=bool(same))
         if len(self._entries) >= self._limit:

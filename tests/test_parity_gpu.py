@@ -483,6 +483,14 @@ def test_causal_mask_check_lazy_and_trust(device):
         assert max_err(out, R.softmax_fp32(x, window, 0.25)) <= TOL[dtype]
         torch.cuda.synchronize()
     assert fs._causal_memo.lookup(window) is False
+    # more new masks than the memo has result slots: an entry that never looked at its verdict
+    # keeps the right one when its slot is handed on
+    old = R.get_attn_mask(16, device, sliding_window_width=2)
+    assert fs._causal_memo.is_plain_causal(old, wait=False) in (None, False)
+    for n in range(300):
+        fs._causal_memo.is_plain_causal(torch.zeros(1, 1, 4, 4, dtype=torch.bool, device=device).triu_(1) if n % 2
+                                        else R.get_attn_mask(4, device), wait=False)
+    assert fs._causal_memo.is_plain_causal(old, wait=True) is False
     # trust: the window mask is ignored, the plain triangle applied
     assert torch.equal(mods["trust"](x, window), ref)
     # gradients through the lazy module, first call (mask-tensor kernels) and later (causal kernels)
