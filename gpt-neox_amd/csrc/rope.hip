@@ -32,6 +32,9 @@ static hipError_t launch_rope_shape(const RopeArgs& a, int s, int n_outer, hipSt
 }
 
 template <typename T, typename CS, int W, bool BWD>
+static bool try_launch_rope_piece(const RopeArgs& a, int s, int n_outer, hipStream_t st, hipError_t* err);
+
+template <typename T, typename CS, int W, bool BWD>
 static hipError_t launch_rope_span(const RopeArgs& a, int s, int n_outer, hipStream_t st) {
     RopeArgs b = a;
     b.lph = a.lpv * 2 + a.pad_slots;

@@ -133,6 +133,23 @@ static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
     return launch_packed<T, M, BWD, EXTRA, 64>(a, st);
 }
 
+// sk <= 512.  The packed forward kernels address the mask and the bias tensor through one buffer
+// each; a call whose mask or bias tensor is beyond the 32-bit range of a buffer goes to the row
+// kernel, which forms a 64-bit address per row.  (The backward pass reads neither.)
+template <typename T, Mask M, bool BWD, int EXTRA>
+static hipError_t dispatch_short_rows(const SoftmaxArgs& a, hipStream_t st) {
+    constexpr bool side_tensor = !BWD && (M == Mask::Bytes || (EXTRA & (kBias | kDropout | kRagged)) != 0);
+    if constexpr (side_tensor) {
+        const bool fits32 = (M != Mask::Bytes || a.mask_bytes != 0) && (a.bias == nullptr || a.bias_bytes != 0);
+        if (!fits32) {
+            // only a bias tensor brings a causal call here
+            constexpr int WITH = (M == Mask::Causal) ? (EXTRA | kBias) : EXTRA;
+            return launch_shape<T, M, BWD, WITH, 1, 1, 4>(a, st);
+        }
+    }
+    return dispatch_packed<T, M, BWD, EXTRA>(a, st);
+}
+
 // The shapes that need 16-byte aligned rows: element-wise kernels when they are not, LDS-staged
 // and packed kernels.  No value: none of them applies, the row kernels take the call.
 template <typename T, Mask M, bool BWD, int EXTRA>
@@ -157,14 +174,7 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
         }
         return launch_generic<T, M, BWD, EXTRA>(a, st);
     }
-    if (chunks == 1) {
-        // the forward mask kernel addresses the mask through one 32-bit-sized buffer
-        // and the bias kernel the bias tensor
-        const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
-                            (a.bias == nullptr || a.bias_bytes != 0);
-        if (fits32) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
-        return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
-    }
+    if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
     if constexpr (BWD && M == Mask::None) {
         // full rows up to 2048 columns: straight-line packed kernel, R x C = 4 accesses per tensor
         if (chunks == 2) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
@@ -185,22 +195,20 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
             // position later on their lanes
             chunks = (a.sk + (a.sk & 1) + kChunk - 1) / kChunk;
         }
-        if (chunks == 1) {
-            const bool fits32 = (BWD || M != Mask::Bytes || a.mask_bytes != 0) &&
-                                (a.bias == nullptr || a.bias_bytes != 0);
-            if (fits32) return dispatch_packed<T, M, BWD, EXTRA>(a, st);
-            return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
-        }
+        if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
     } else {
         if (const auto done = dispatch_aligned<T, M, BWD, EXTRA>(a, vec_ok, chunks, st)) return *done;
     }
-    if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
-    if (chunks == 3) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
-    if (chunks == 4) {
-        // the causal forward with two output streams (dropout) measured 3 % faster with 2 rows
-        if constexpr (!BWD && M == Mask::Causal && (EXTRA & kDropout) != 0)
-            return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
-        return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
+    // (the aligned full-row backward has taken 2 to 4 chunks with its packed kernel above)
+    if constexpr (!(BWD && M == Mask::None && (EXTRA & kRagged) == 0)) {
+        if (chunks == 2) return launch_shape<T, M, BWD, EXTRA, 2, 1, 4>(a, st);
+        if (chunks == 3) return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
+        if (chunks == 4) {
+            // the causal forward with two output streams (dropout) measured 3 % faster with 2 rows
+            if constexpr (!BWD && M == Mask::Causal && (EXTRA & kDropout) != 0)
+                return launch_shape<T, M, BWD, EXTRA, 2, 2, 2>(a, st);
+            return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
+        }
     }
     if constexpr (!BWD) {
         // Forward, rows that would leave a quarter or more of the 2-chunk shape's slots empty:

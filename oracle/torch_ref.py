@@ -144,14 +144,14 @@ def alibi_slopes(n):
     return power_of_two(below) + alibi_slopes(2 * below)[0::2][: n - below]
 
 
-def alibi_bias_fp32(slopes, sq, sk):
+def alibi_bias_fp32(slopes, sq, sk, device="cpu"):
     """fp32 ALiBi bias [np, sq, sk]: -slope_h * (i - j) on j <= i, 0 above the diagonal.
     Follows AliBi.forward, megatron/model/positional_embeddings.py:210-257 (sq == sk)."""
     assert sq == sk
-    i = torch.arange(sq).view(sq, 1)
-    j = torch.arange(sk).view(1, sk)
+    i = torch.arange(sq, device=device, dtype=torch.int32).view(sq, 1)
+    j = torch.arange(sk, device=device, dtype=torch.int32).view(1, sk)
     dist = -torch.tril(i - j).float()
-    return dist * torch.as_tensor(slopes, dtype=torch.float32).view(-1, 1, 1)
+    return dist * torch.as_tensor(slopes, dtype=torch.float32, device=device).view(-1, 1, 1)
 
 
 # --- rotary ------------------------------------------------------------------------

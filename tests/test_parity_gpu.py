@@ -1353,8 +1353,8 @@ def test_rotary_slot_widths_table_types_and_directions(device, case, half_tables
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_lds_staged_causal_rows_in_both_storage_types(device, dtype):
-    s = 33000
+@pytest.mark.parametrize("s", [33000, 40968])  # staged in half of a CU's LDS / in all of it
+def test_lds_staged_causal_rows_in_both_storage_types(device, dtype, s):
     x = scores((1, s, s), dtype, device, 7)
     y = causal_ext.forward(x, 0.05)
     rows = torch.tensor([0, 1, 700, s // 2, s - 1], device=device)
