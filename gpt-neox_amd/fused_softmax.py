@@ -133,6 +133,7 @@ class _CausalMaskMemo:
         self._entries = {}
         self._limit = limit
         self._slots = None  # pinned result slots, handed out in turn
+        self._slot_owner = None  # per slot: the entry whose verdict it holds or will hold
         self._next_slot = 0
 
     @staticmethod
@@ -178,9 +179,10 @@ class _CausalMaskMemo:
         if mask.is_cuda:
             entry = _MaskVerdict(storage, mask._version)
             slot = self._result_slot(entry)
-            slot.copy_(same.view(1), non_blocking=True)
-            event = torch.cuda.Event()
-            event.record()
+            with torch.cuda.device(mask.device):  # copy and event on the mask's device and stream
+                slot.copy_(same.view(1), non_blocking=True)
+                event = torch.cuda.Event()
+                event.record()
             entry.pending = (slot, event)
         else:
             entry = _MaskVerdict(storage, mask._version, verdict=bool(same))
