@@ -114,9 +114,15 @@ static hipError_t launch_packed_shape(const SoftmaxArgs& a0, hipStream_t st) {
 
 template <typename T, Mask M, bool BWD, int EXTRA, int G>
 static hipError_t launch_packed(const SoftmaxArgs& a, hipStream_t st) {
-    // passes per wave: 4 everywhere except the causal forward of the longer packed rows,
-    // which measured 15 % faster with 2
-    constexpr int R = (!BWD && M == Mask::Causal && G >= 32) ? 2 : kPackedPasses;
+    // passes per wave: 4, except for lane groups of 32 and 64 lanes in the causal kernels and the
+    // full-row backward, which run faster with 2 when the rows fill their lane groups (causal forward
+    // 15 %, causal backward up to 11 % at 512 columns, full-row backward 0-4 %).  With a quarter or
+    // more of the lanes idle (129-192 and 257-384 columns) 4 passes are 4-12 % faster there too.
+    constexpr int R = (M != Mask::Bytes && G >= 32) ? 2 : kPackedPasses;
+    if constexpr (R != kPackedPasses) {
+        const int lanes = (a.sk + kVec - 1) / kVec;
+        if (lanes * 4 <= G * 3) return launch_packed_shape<T, M, BWD, EXTRA, G, kPackedPasses, 1>(a, st);
+    }
     return launch_packed_shape<T, M, BWD, EXTRA, G, R, 1>(a, st);
 }
 

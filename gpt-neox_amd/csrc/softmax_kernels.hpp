@@ -582,69 +582,34 @@ __device__ __forceinline__ uint32_t wrap_row(uint32_t i, uint32_t sq) {
 }
 
 // kRagged in the packed kernels.  A wave's rows lie back to back behind one buffer, so the lane
-// that holds the end of a row must not touch the columns that follow: they belong to the next
-// row.  Every row ends the same way, with rem = sk % 8 columns in its last lane, and that lane
-// moves them by a 64-, a 32- and a 16-bit access instead of one of 128 bits -- rem = 4a + 2b + c;
-// a piece that rem does not contain is skipped by the whole wave, and the lanes that are not at
-// a row end aim the others out of range.
+// that holds the end of a row -- rem = sk % 8 columns of it -- must not touch the columns that
+// follow: they belong to the next row.  That lane moves its access back by 8 - rem columns
+// instead (`back`), so that it ends with the row: it then holds the last 8 columns of the row,
+// of which the first 8 - rem are also held by the lane before it.  Both lanes compute the same
+// values for those columns from the same inputs and store the same bits; only the row's sums
+// count them once (the lane that is moved back leaves its first `back` columns out).  Every
+// lane so makes exactly one 128-bit access per tensor, at a 2-byte alignment.
 //
-// 128-bit access of the packed kernels: whole when the lane's 8 columns lie inside its row (always
-// so without RAG), in pieces at a ragged row end, nothing for an inactive lane.  `off`: byte
-// offset of the lane's first column; `left`: columns from there to the row end; `rem`: sk % 8.
-template <bool NT, bool RAG>
-__device__ __forceinline__ u32x4 packed_ld(rsrc_t r, uint32_t off, int left, bool active, int rem) {
-    u32x4 v = buf_ld128<NT>(r, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
-    if constexpr (RAG) {
-        const bool end = active && left < kVec;  // a row-end lane: left == rem
-        if (rem & 4) {
-            const u32x2 a = buf_ld64(r, end ? off : kOutOfRange, 0);
-            v.x |= a.x;
-            v.y |= a.y;
-        }
-        if (rem & 2) {
-            const uint32_t b = buf_ld32(r, end ? off + (uint32_t)(rem & 4) * 2u : kOutOfRange);
-            if (rem & 4) v.z |= b;
-            else v.x |= b;
-        }
-        if (rem & 1) {
-            const uint32_t c = buf_ld16(r, end ? off + (uint32_t)(rem & 6) * 2u : kOutOfRange);
-            if (rem == 1) v.x |= c;
-            else if (rem == 3) v.y |= c;
-            else if (rem == 5) v.z |= c;
-            else v.w |= c;
-        }
-    }
-    return v;
+// 128-bit access of the packed kernels: nothing for an inactive lane.  `off`: byte offset of the
+// lane's first column.
+template <bool NT>
+__device__ __forceinline__ u32x4 packed_ld(rsrc_t r, uint32_t off, bool active) {
+    return buf_ld128<NT>(r, active ? off : kOutOfRange, 0);
 }
-template <bool NT, bool RAG>
-__device__ __forceinline__ void packed_st(rsrc_t r, const u32x4& v, uint32_t off, int left, bool active, int rem) {
-    buf_st128<NT>(r, v, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
-    if constexpr (RAG) {
-        const bool end = active && left < kVec;
-        if (rem & 4) buf_st64(r, u32x2{v.x, v.y}, end ? off : kOutOfRange);
-        if (rem & 2) buf_st32(r, (rem & 4) ? v.z : v.x, end ? off + (uint32_t)(rem & 4) * 2u : kOutOfRange);
-        if (rem & 1)
-            buf_st16(r, rem == 1 ? v.x : rem == 3 ? v.y : rem == 5 ? v.z : v.w,
-                     end ? off + (uint32_t)(rem & 6) * 2u : kOutOfRange);
-    }
+template <bool NT>
+__device__ __forceinline__ void packed_st(rsrc_t r, const u32x4& v, uint32_t off, bool active) {
+    buf_st128<NT>(r, v, active ? off : kOutOfRange, 0);
 }
-// The lane's 8 mask bytes, likewise (pieces of 4, 2 and 1 bytes at a ragged row end).
+// The lane's 8 mask bytes, likewise.
+__device__ __forceinline__ u32x2 packed_ld_mask(rsrc_t r, uint32_t off, bool active) {
+    return buf_ld64(r, active ? off : kOutOfRange, 0);
+}
+// Columns by which the lane that holds a ragged row end is moved back (0 for every other lane).
 template <bool RAG>
-__device__ __forceinline__ u32x2 packed_ld_mask(rsrc_t r, uint32_t off, int left, bool active, int rem) {
-    u32x2 v = buf_ld64(r, (active && (!RAG || left >= kVec)) ? off : kOutOfRange, 0);
-    if constexpr (RAG) {
-        const bool end = active && left < kVec;
-        uint32_t low = 0;  // the bytes after the 4-byte piece
-        if (rem & 2) low = buf_ld16(r, end ? off + (uint32_t)(rem & 4) : kOutOfRange);
-        if (rem & 1) low |= buf_ld8(r, end ? off + (uint32_t)(rem & 6) : kOutOfRange) << (8 * (rem & 2));
-        if (rem & 4) {
-            v.x |= buf_ld32(r, end ? off : kOutOfRange);
-            v.y |= low;
-        } else {
-            v.x |= low;
-        }
-    }
-    return v;
+__device__ __forceinline__ int ragged_back(int col0, int sk) {
+    if constexpr (!RAG) return 0;
+    const int rem = sk & (kVec - 1);
+    return (rem != 0 && col0 < sk && col0 + kVec > sk) ? kVec - rem : 0;
 }
 
 template <int G, int R = kPackedPasses>
@@ -667,9 +632,9 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
     const int sk = a.sk;
-    const int rem = sk & (kVec - 1);  // kRagged: columns in the last lane of a row
     const int grp = lane / G;
-    const int col0 = (lane % G) * kVec;
+    const int back = ragged_back<kRag>((lane % G) * kVec, sk);  // kRagged: see ragged_back
+    const int col0 = (lane % G) * kVec - back;                  // first column of the lane's accesses
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
     const float ninf = -__builtin_inff();
@@ -706,15 +671,15 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
-            raw[p][c] = packed_ld<kLdNt, kRag>(rx, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
+            raw[p][c] = packed_ld<kLdNt>(rx, (lr * sk + col) * 2u, col < len[p]);
             if constexpr ((FLAGS & kBias) != 0) {
                 const uint32_t boff = (bias_row(row, a) * (uint32_t)sk + col) * 2u;
-                rawb[p][c] = packed_ld<false, kRag>(rb, boff, sk - col, col < len[p], rem);
+                rawb[p][c] = packed_ld<false>(rb, boff, col < len[p]);
             }
             if constexpr (MASK == Mask::Bytes) {
                 const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
                 const uint32_t moff = (mb * (uint32_t)a.sq + i) * sk + col;
-                mk[p][c] = packed_ld_mask<kRag>(rm, moff, sk - col, col < len[p], rem);
+                mk[p][c] = packed_ld_mask(rm, moff, col < len[p]);
             }
         }
     }
@@ -753,7 +718,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 v[c][k] = fast_exp2(v[c][k] - mx);
-                sum += v[c][k];
+                sum += (kRag && k < back) ? 0.f : v[c][k];  // columns the lane before counts
             }
         if constexpr (MASK == Mask::Bytes) {
             // rows with every key hidden (rare): uniform over the sk columns
@@ -766,7 +731,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
                         for (int k = 0; k < 8; ++k) {
                             v[c][k] = ((col0 + c * kChunk + k) < len[p]) ? 1.f : 0.f;
-                            sum += v[c][k];
+                            sum += (kRag && k < back) ? 0.f : v[c][k];
                         }
                 }
             }
@@ -781,10 +746,10 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
             for (int k = 0; k < 8; ++k) v[c][k] *= inv;  // lanes of absent rows hold NaN and store nothing
             const bool st = lr < rows_here && col < sk;
             const u32x4 o = pack8<T>(v[c]);
-            packed_st<kStNt, kRag>(ry, o, (lr * sk + col) * 2u, sk - col, st, rem);
+            packed_st<kStNt>(ry, o, (lr * sk + col) * 2u, st);
             if constexpr ((FLAGS & kDropout) != 0) {
                 const uint32_t bits = keep_bits_row8<kRag>(drop, row0 + lr, sk, col);
-                packed_st<kStNt, kRag>(ry2, dropout8<T>(o, bits, drop.scale), (lr * sk + col) * 2u, sk - col, st, rem);
+                packed_st<kStNt>(ry2, dropout8<T>(o, bits, drop.scale), (lr * sk + col) * 2u, st);
             }
         }
     }
@@ -803,9 +768,9 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     if (row0 >= a.rows) return;
     const uint32_t rows_here = min((uint32_t)RPW, a.rows - row0);
     const int sk = a.sk;
-    const int rem = sk & (kVec - 1);  // kRagged: columns in the last lane of a row
     const int grp = lane / G;
-    const int col0 = (lane % G) * kVec;
+    const int back = ragged_back<kRag>((lane % G) * kVec, sk);  // kRagged: see ragged_back
+    const int col0 = (lane % G) * kVec - back;                  // first column of the lane's accesses
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
 
@@ -825,8 +790,8 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
-            rg[p][c] = packed_ld<kLdNt, kRag>(bg, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
-            rp[p][c] = packed_ld<kLdNt, kRag>(by, (lr * sk + col) * 2u, sk - col, col < len[p], rem);
+            rg[p][c] = packed_ld<kLdNt>(bg, (lr * sk + col) * 2u, col < len[p]);
+            rp[p][c] = packed_ld<kLdNt>(by, (lr * sk + col) * 2u, col < len[p]);
         }
     }
 #pragma unroll
@@ -846,6 +811,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
             for (int k = 0; k < 8; ++k) {
                 if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 if ((col0 + c * kChunk + k) >= len[p]) gv[k] = pv[k] = 0.f;  // past the diagonal / row end
+                if (kRag && k < back) gv[k] = 0.f;  // columns the lane before counts
                 dot = fmaf(gv[k], pv[k], dot);
             }
         }
@@ -863,7 +829,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
                 if ((col + k) >= len[p]) gv[k] = 0.f;
             }
             const bool st = lr < rows_here && col < sk;
-            packed_st<kStNt, kRag>(bo, pack8<T>(gv), (lr * sk + col) * 2u, sk - col, st, rem);
+            packed_st<kStNt>(bo, pack8<T>(gv), (lr * sk + col) * 2u, st);
         }
     }
 }
