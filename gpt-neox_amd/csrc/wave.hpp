@@ -140,17 +140,8 @@ __device__ __forceinline__ u32x3 buf_ld96(rsrc_t r, int voffset) {
 __device__ __forceinline__ void buf_st96(rsrc_t r, const u32x3& v, int voffset) {
     __builtin_amdgcn_raw_buffer_store_b96(v, r, voffset, 0, 0);
 }
-__device__ __forceinline__ uint32_t buf_ld8(rsrc_t r, int voffset) {
-    return __builtin_amdgcn_raw_buffer_load_b8(r, voffset, 0, 0);
-}
 __device__ __forceinline__ void buf_st16(rsrc_t r, uint32_t v, int voffset) {
     __builtin_amdgcn_raw_buffer_store_b16((unsigned short)v, r, voffset, 0, 0);
-}
-__device__ __forceinline__ void buf_st32(rsrc_t r, uint32_t v, int voffset) {
-    __builtin_amdgcn_raw_buffer_store_b32(v, r, voffset, 0, 0);
-}
-__device__ __forceinline__ void buf_st64(rsrc_t r, const u32x2& v, int voffset) {
-    __builtin_amdgcn_raw_buffer_store_b64(v, r, voffset, 0, 0);
 }
 
 // ---- wave64 reductions --------------------------------------------------------
