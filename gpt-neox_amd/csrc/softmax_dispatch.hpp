@@ -13,7 +13,9 @@
 //   chunks <= 16   8 waves per row, 512-thread block                 (sk <= 8192)
 //   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
 //                  forward, in the lower 3/4 of each of these three ranges (7/8 of the last):
-//                  half as many waves with 3 (4) chunks each
+//                  half as many waves with 3 (4) chunks each; causal backward likewise at
+//                  8193-12288 columns; mask-tensor forward at 513-768 columns: packed kernel,
+//                  two rows of two chunks per wave
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
@@ -181,6 +183,13 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
         return launch_generic<T, M, BWD, EXTRA>(a, st);
     }
     if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
+    if constexpr (!BWD && M == Mask::Bytes && (EXTRA & kDropout) == 0) {
+        // mask-tensor forward, 513-768 columns: the packed kernel with two rows of two chunks per wave
+        // keeps four accesses per tensor in flight where the row kernel's second chunk is mostly empty
+        // (-17 % at 520-640 columns, -8 % at 768, +1 % at 896; the causal forward loses 2-10 % with it)
+        const bool fits32 = a.mask_bytes != 0 && (a.bias == nullptr || a.bias_bytes != 0);
+        if (chunks == 2 && a.sk <= 768 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
+    }
     if constexpr (BWD && M == Mask::None) {
         // full rows up to 2048 columns: straight-line packed kernel, R x C = 4 accesses per tensor
         if (chunks == 2) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
@@ -226,6 +235,12 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if (chunks > 8 && chunks <= 12) return launch_shape<T, M, BWD, EXTRA, 3, 4, 1>(a, st);
         if (chunks > 16 && chunks <= 24) return launch_shape<T, M, BWD, EXTRA, 3, 8, 1>(a, st);
         if (chunks > 24 && chunks <= 28) return launch_shape<T, M, BWD, EXTRA, 4, 8, 1>(a, st);
+    }
+    if constexpr (BWD && M == Mask::Causal) {
+        // Causal backward just above 8192 columns: 8 waves with 3 chunks each instead of 16 with 2, of
+        // which up to half would hold nothing (-13 % at 8200 columns, -8 % at 10240, -4 % at 12288).  The
+        // same step at the shorter ranges and for the full-row backward measured -3...+5 %: not taken.
+        if (chunks > 16 && chunks <= 24) return launch_shape<T, M, BWD, EXTRA, 3, 8, 1>(a, st);
     }
     if (chunks <= 8) return launch_shape<T, M, BWD, EXTRA, 2, 4, 1>(a, st);
     if (chunks <= 16) return launch_shape<T, M, BWD, EXTRA, 2, 8, 1>(a, st);
