@@ -1,7 +1,8 @@
 """Kernel instantiations that only unusual calls reach, each against the oracle (through the C-ABI).
 
-* rows of at most 512 columns whose mask or bias tensor is larger than a 32-bit buffer range
-  (4 GiB): the row kernel with a 64-bit address per row instead of the packed kernels;
+* rows that the packed kernels take (at most 512 columns; 513-768 and 1025-1536 with a mask tensor)
+  whose mask or bias tensor is larger than a 32-bit buffer range (4 GiB): the row kernels with a
+  64-bit address per row instead;
 * packed kernels on tensors beyond 4 GiB;
 * the XCD-aware rotary kernel with 2-, 4- and 8-element slots, fp32 and 16-bit tables, forward and
   backward (it takes dense tensors that start on a 4 KiB boundary);
@@ -56,8 +57,8 @@ def sample_rows(n, device, seed):
 # softmax: short rows with tensors beyond 4 GiB
 # ---------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sk", [512, 511])  # aligned rows / ragged rows
-def test_short_rows_with_a_mask_tensor_beyond_4_gib(device, sk, dtype):
+@pytest.mark.parametrize("sk", [512, 511, 640, 1536])  # aligned / ragged short rows; the packed kernels' longer rows
+def test_rows_with_a_mask_tensor_beyond_4_gib(device, sk, dtype):
     sq = FOUR_GIB // sk + 16
     assert sq * sk > FOUR_GIB
     scale, p, seed, offset = 0.5, 0.25, 99, 8
