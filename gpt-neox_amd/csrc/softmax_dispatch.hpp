@@ -14,8 +14,9 @@
 //   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
 //                  forward, in the lower 3/4 of each of these three ranges (7/8 of the last):
 //                  half as many waves with 3 (4) chunks each; causal backward likewise at
-//                  8193-12288 columns; mask-tensor forward at 513-768 and 1025-1536 columns:
-//                  packed kernel, two rows of two chunks or one row of three chunks per wave
+//                  8193-12288 columns; mask-tensor forward at 513-768 and 1025-1536 columns and
+//                  causal forward at 1025-1408: packed kernel, two rows of two chunks or one row
+//                  of three chunks per wave
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
@@ -183,15 +184,25 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
         return launch_generic<T, M, BWD, EXTRA>(a, st);
     }
     if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
-    if constexpr (!BWD && M == Mask::Bytes && (EXTRA & kDropout) == 0) {
+    if constexpr (!BWD && M == Mask::Bytes) {
         // mask-tensor forward, 513-768 columns: the packed kernel with two rows of two chunks per wave
         // keeps four accesses per tensor in flight where the row kernel's second chunk is mostly empty
         // (-17 % at 520-640 columns, -8 % at 768, +1 % at 896; the causal forward loses 2-10 % with it);
         // 1025-1536 columns: one row of three chunks per wave instead of two waves with four slots
-        // (-9 % at 1032 and 1152 columns, -5 % at 1280, -1 % at 1536; four chunks: +2...4 %)
+        // (-9 % at 1032 and 1152 columns, -5 % at 1280, -1 % at 1536; four chunks: +2...4 %); with
+        // dropout folded in both steps gain 4-11 %
         const bool fits32 = a.mask_bytes != 0 && (a.bias == nullptr || a.bias_bytes != 0);
         if (chunks == 2 && a.sk <= 768 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
         if (chunks == 3 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
+    }
+    if constexpr (!BWD && M == Mask::Causal) {
+        // causal forward, 1025-1408 columns: one row of three chunks per wave instead of two waves with
+        // four slots (-11 % at 1032 and 1152 columns, -5 % at 1280, +1 % at 1536).  At two and at four
+        // chunks, and in the causal backward at any, the packed kernel measured 2-16 % slower.  The
+        // dropout variant follows (it loses 1-8 % here): its undropped output stays bit-equal to the
+        // plain kernel's, which needs the same order of summation.
+        const bool fits32 = a.bias == nullptr || a.bias_bytes != 0;
+        if (chunks == 3 && a.sk <= 1408 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
     }
     if constexpr (BWD && M == Mask::None) {
         // full rows up to 2048 columns: straight-line packed kernel, R x C = 4 accesses per tensor

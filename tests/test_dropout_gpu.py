@@ -646,10 +646,10 @@ def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
 
 
 # one row length per kernel shape of the dispatcher: lane groups of 1 .. 64 lanes (those of 32 and 64
-# lanes also three quarters full or less: 160 and 320 columns; 640: the mask-tensor forward's two-chunk
-# packed kernel), then 1, 2, 4, 8 and 16 waves per row
+# lanes also three quarters full or less: 160 and 320 columns; 640 and 1280: the forward passes'
+# two- and three-chunk packed kernels), then 1, 2, 4, 8 and 16 waves per row
 # with 2, 3 or 4 chunks per wave
-SHAPE_LENGTHS = [8, 16, 32, 64, 128, 160, 256, 320, 512, 640, 1024, 1536, 2048, 2560, 4096, 5120, 8192, 10240, 13312, 16384,
+SHAPE_LENGTHS = [8, 16, 32, 64, 128, 160, 256, 320, 512, 640, 1024, 1280, 1536, 2048, 2560, 4096, 5120, 8192, 10240, 13312, 16384,
                  20480, 28672]
 
 
