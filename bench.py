@@ -726,6 +726,37 @@ def main():
                 ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
                 del s_
             result["evaluation_lengths"] = ragged
+        # Every kernel family over the row lengths, the shape boundaries of the dispatcher included (one
+        # length at and one just above each power of two): % of the HBM peak by algorithmic bytes, fp16,
+        # about 600 MB per tensor, three buffer sets.  Causal rows of a few columns read whole 64-byte
+        # sectors where the algorithmic count has half a row, so their figures stop at 55-60 %.
+        if want("scan") and not args.quick:
+            scan = []
+            for n in (64, 128, 129, 256, 257, 320, 512, 520, 768, 1024, 1032, 1280, 1536, 2048, 2056, 3072, 4096, 4104,
+                      6144, 8192, 8200, 12288, 16384):
+                B = max(2, int(600e6 // (n * n * 2)))  # at least two matrices: 0.6-1.1 GB per tensor
+                sets = []
+                for _ in range(3):
+                    x = torch.empty(B, n, n, device=dev, dtype=torch.float16).normal_(0.0, 8.0)
+                    sets.append(dict(x=x, y=torch.empty_like(x), dy=torch.empty_like(x).normal_(), dx=torch.empty_like(x)))
+                mask = (torch.rand(1, 1, n, n, device=dev) < 0.2).to(torch.uint8)
+                f16 = code[torch.float16]
+                cf = time_launches(lambda t: ok(lib.neox_causal_softmax_fwd(
+                    t["y"].data_ptr(), t["x"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                cb = time_launches(lambda t: ok(lib.neox_causal_softmax_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                mf = time_launches(lambda t: ok(lib.neox_masked_softmax_fwd(
+                    t["y"].data_ptr(), t["x"].data_ptr(), mask.data_ptr(), 0.125, 1, B, n, n, 1, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                fb = time_launches(lambda t: ok(lib.neox_masked_softmax_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B * n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                full = B * n * n * 2
+                pct = lambda nbytes, us: round(100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, 1)
+                scan.append({"sk": n, "matrices": B,
+                             "causal_fwd_pct": pct(B * 2 * (tri(n) + n * n), cf), "causal_bwd_pct": pct(B * 2 * (2 * tri(n) + n * n), cb),
+                             "mask_tensor_fwd_pct": pct(2 * full + n * n, mf), "full_row_bwd_pct": pct(3 * full, fb)})
+                del sets, mask
+            result["row_length_scan_pct_of_hbm_peak"] = scan
+            torch.cuda.empty_cache()
         # The reference's own fallback on this GPU, for scale: what FusedScaleMaskSoftmax runs when its
         # predicate fails (always at sk > 2048, e.g. configs[4]) is the unfused torch branch
         # (megatron/model/fused_softmax.py:184-199 with gpt2_attention_mask_func,
