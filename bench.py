@@ -603,6 +603,7 @@ def main():
         if want("models"):
             extra = []
             for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
+                                     (2048, 4, 32, 80, 20), (2048, 4, 32, 80, 80),
                                      (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
                 s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
                 nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4

@@ -196,8 +196,10 @@ int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np);
  * out of place (out_q != q, or out_k != k) the pass-through dims [d_rot, d) are copied
  * from the inputs by the same launch, as the reference's kernels do; pass d = d_rot to
  * have only the rotated span written.  In place the dims >= d_rot keep their values; those
- * that share a 64-byte block with the end of the rotated span may be written back unchanged
- * (whole 64-byte writes are much cheaper for the memory system than partial ones).
+ * that share a 64-byte block with the end of the rotated span (a 32-byte block when the heads
+ * start on 32-byte boundaries only) may be written back unchanged -- whole blocks are much
+ * cheaper for the memory system than partial ones; the block never reaches into the other
+ * tensor of the same call, so q and k may be views into one buffer.
  * k / out_k may both be NULL.
  * Replaces apply_rotary_pos_emb / apply_rotary_pos_emb_torch
  *   megatron/model/positional_embeddings.py:103-126

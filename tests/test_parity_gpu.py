@@ -705,6 +705,25 @@ def test_rotary_offset_and_qkv_views(device, dtype):
     check_rotary(device, 11, 3, 4, 4, 128, 32, dtype, seed=3, offset=2, qkv_view=True)
 
 
+@pytest.mark.parametrize("hn,d_rot,parts", [(48, 40, 2), (48, 24, 2), (48, 40, 3), (80, 20, 3), (80, 40, 2), (112, 28, 3),
+                                            (96, 24, 3), (64, 40, 2)])
+def test_rotary_in_place_on_q_and_k_interleaved_in_one_buffer(device, hn, d_rot, parts):
+    # q and k as views into one [s, b, h, parts * hn] buffer: the kernels write a rotated span back
+    # together with the rest of its 64- or 32-byte block, and that block must never reach into the
+    # other tensor's span, which the same launch rewrites (48-dim heads with 40 rotated dims: the
+    # 64-byte block of q's span end would cover the first 32 bytes of k)
+    s, b, h, dtype = 33, 2, 8, torch.bfloat16
+    for seed in range(3):
+        buf = normal((s, b, h, parts * hn), dtype, device, 70 + seed)
+        before = buf.clone()
+        q, k = buf[..., :hn], buf[..., hn : 2 * hn]
+        cos, sin = (t.to(device) for t in R.rotary_tables(d_rot, s + 1))
+        want_q, want_k = R.partial_rotary(before[..., :hn].float(), before[..., hn : 2 * hn].float(), cos, sin, d_rot, offset=1)
+        apply_rotary_pos_emb_(q, k, cos, sin, 1, d_rot)
+        assert torch.equal(buf[..., :hn], want_q.to(dtype)) and torch.equal(buf[..., hn : 2 * hn], want_k.to(dtype))
+        assert torch.equal(buf[..., 2 * hn :], before[..., 2 * hn :])
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_rotary_half_precision_tables(device, dtype):
     # tables in the dtype of q (the model's usual setting): fp32 arithmetic on the table
