@@ -1,27 +1,35 @@
 #!/usr/bin/env python3
 """Benchmark of the fused softmax / rotary hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table] [--quick] [--only TEXT]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-table] [--quick]
+                    [--only TEXT] [--studies]
 
 A step is one pass of the hot path over one batch of synthetic input with all tensors
 resident in HBM, on the largest single-GPU configuration of BASELINE.json, configs[4]: the
 long-context causal scaled softmax forward + backward on scores [1, 32, 8192, 8192] bf16
 (scale 1/sqrt(128)) plus the full rotary forward + backward on q, k [8192, 1, 32, 128] bf16 --
-four launches.  K steps are timed after W warm-up steps between device synchronisations; the
-JSON line carries
+four launches.  K steps are timed after W warm-up steps between device synchronisations.
+
+The LAST line of stdout is one compact ASCII JSON object (under 6 KB):
 
 * value       -- algorithmic GB/s of the step (bytes of the four launches / step time);
-* min_pct_hbm_peak_over_configs -- the lowest % of HBM peak over every BASELINE shape and op;
 * roofline    -- the step's dominant kernel (the causal backward) alone: algorithmic bytes per
                  launch / mean launch duration of K back-to-back launches between two HIP
                  events on the launch stream, against the 8 TB/s HBM peak; `traffic` is read
                  from the counter summary under profiles/ (it cannot be measured live);
 * cpu_baseline-- the oracle's torch CPU path (forward + autograd backward) timed on
                  this host's cores on 1/32 of the same step;
-* all_configs -- every BASELINE.json shape and op: us per call, GB/s, % of peak and, as part
-                 of the CPU-baseline leg, the oracle's CPU time on a slice scaled to the full
-                 shape with the error of the kernel's output on that slice against it (max
-                 |err|, non-zero masked outputs; bit-equality for rotary).
+* all_configs -- the twelve rows of BASELINE.json's shapes and ops: us per call, GB/s, % of
+                 peak and, as part of the CPU-baseline leg, the oracle's CPU time on a slice
+                 scaled to the full shape with the error of the kernel's output on that slice
+                 against the oracle's fp32 path (forward: the probabilities; backward: autograd
+                 from x; rotary: bit-equality with the fp32 expression rounded once);
+* min_pct_hbm_peak_over_configs -- the lowest % of HBM peak over those rows.
+
+--studies adds the measurements around the table (fused dropout, bias and ALiBi variants, other
+head sizes, ragged lengths, a scan over the row lengths, the unfused torch branches on this GPU,
+the Python modules against the C-ABI, a plain copy) and writes them to
+gpurun_out/bench_studies.json; none of them runs by default and none enters the line.
 
 The oracle is imported by the CPU-baseline leg only (--no-cpu runs never load it); the inputs
 of the measured launches are built without it.
@@ -42,6 +50,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 METRIC = "softmax/rotary fwd+bwd achieved GB/s and % of MI355X HBM peak; µs per call"
+STUDIES_PATH = os.path.join(ROOT, "gpurun_out", "bench_studies.json")
 
 
 def parse():
@@ -55,8 +64,10 @@ def parse():
     ap.add_argument("--quick", action="store_true",
                     help="few launches per table row (for counter-collection runs)")
     ap.add_argument("--only", type=str, default=None,
-                    help="run only the table rows whose name contains this text, or one of several texts "
-                         "separated by commas (profiling aid)")
+                    help="run only the table rows / study sections whose name contains this text, or one of "
+                         "several texts separated by commas (profiling aid)")
+    ap.add_argument("--studies", action="store_true",
+                    help="also run the study sections and write them to gpurun_out/bench_studies.json")
     return ap.parse_args()
 
 
@@ -74,30 +85,26 @@ def measured_traffic(key):
                     kv = dict(p.split("=", 1) for p in parts[2:] if "=" in p)
                     fetched, written = float(kv["fetched_bytes"]), float(kv["written_bytes"])
                     return {"traffic": fetched + written,
-                            "traffic_source": "profiles/hbm_traffic_counters.txt (rocprofv3 --pmc runs of this "
-                                              "script; fetched %.4g B + written %.4g B)" % (fetched, written)}
+                            "traffic_source": "profiles/hbm_traffic_counters.txt (fetched %.4g B + written %.4g B)"
+                                              % (fetched, written)}
     except (OSError, KeyError, ValueError):
         pass
     return {"traffic": None, "traffic_source": "no counter summary for this kernel under profiles/"}
 
 
-def load_probes():
-    """libneox_probes.so: the memory-system probes of this benchmark (plain copy, strided touch,
-    empty kernel).  They are not part of the product library."""
+def load_copy_probe():
+    """libneox_probes.so: a plain copy kernel and an empty kernel with the access shape of the product
+    kernels -- the known-size launch the FETCH_SIZE / WRITE_SIZE counters are calibrated against.
+    Not part of the product library; built by `make -C gpt-neox_amd/csrc probes`."""
     import ctypes
 
     path = os.path.join(ROOT, "gpt-neox_amd", "csrc", "libneox_probes.so")
     if not os.path.exists(path):
-        raise ImportError(f"{path} not found: run `make -C gpt-neox_amd/csrc`")
+        raise ImportError(f"{path} not found: run `make -C gpt-neox_amd/csrc probes`")
     h = ctypes.CDLL(path)
-    vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
     h.neox_probe_copy.restype, h.neox_probe_copy.argtypes = ctypes.c_int, [vp, vp, i64, vp]
     h.neox_probe_empty.restype, h.neox_probe_empty.argtypes = ctypes.c_int, [vp]
-    h.neox_probe_strided.restype = ctypes.c_int
-    h.neox_probe_strided.argtypes = [vp, i64, i32, i32, i64, i32, i32, vp]
-    h.neox_probe_pieces.restype, h.neox_probe_pieces.argtypes = ctypes.c_int, [vp, vp, i64, i32, i32, i32, vp]
-    h.neox_probe_strided_pieces.restype = ctypes.c_int
-    h.neox_probe_strided_pieces.argtypes = [vp, i64, i32, i32, i32, vp]
     return h
 
 
@@ -123,7 +130,6 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     lib = _lib.lib()  # ImportError if the HIP library is not built
-    probes = load_probes()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     stream = torch.cuda.current_stream().cuda_stream
@@ -136,6 +142,12 @@ def main():
     def ok(status):
         if status != 0:
             _lib.check(status)
+
+    def want(name):
+        return args.only is None or any(part in name for part in args.only.split(","))
+
+    def tri(n):
+        return n * (n + 1) // 2
 
     # ------------------------------------------------------------------ workloads
     def masked_sets(b, heads, sq, sk, dtype, seed, nsets):
@@ -220,51 +232,6 @@ def main():
             means.append(e0.elapsed_time(e1) * 1e3 / n_launch)
         return statistics.median(means), min(means)
 
-    def placement_rows():
-        """cfg5 causal forward and backward against where the output lies: the memory is covered with
-        4 GiB tensors, the inputs stay in the first ones and each of the others takes the output in
-        turn.  The times fall into two classes (the 288 GB behave as three regions of 96 GiB; a launch
-        that writes into another region than it reads from is the faster one); reported are the
-        classes' medians and the class of every tensor in allocation order -- a process that starts
-        on an idle device finds the regions in that order, after earlier allocations and frees the
-        driver hands the memory out in another order."""
-        B, n, dt, sc = 32, 8192, torch.bfloat16, 128 ** -0.5
-        tri = n * (n + 1) // 2
-        fwd_bytes, bwd_bytes = B * 2 * (tri + n * n), B * 2 * (2 * tri + n * n)
-        free, total = torch.cuda.mem_get_info()
-        count = int((free - (24 << 30)) // (4 << 30))
-        if count < 8:
-            raise torch.cuda.OutOfMemoryError("not enough free memory to cover the device")
-        t = [torch.empty(B, n, n, device=dev, dtype=dt) for _ in range(count)]
-        x, dy, y = t[0], t[1], t[2]
-        for j in range(0, B, 8):
-            x[j : j + 8].normal_(0.0, 8.0)
-            dy[j : j + 8].normal_()
-        ok(lib.neox_causal_softmax_fwd(y.data_ptr(), x.data_ptr(), sc, B, n, n, code[dt], stream))
-        fwd_us, bwd_us = [], []
-        for out in t[3:]:
-            fwd_us.append(time_launches(lambda _: ok(lib.neox_causal_softmax_fwd(
-                out.data_ptr(), x.data_ptr(), sc, B, n, n, code[dt], stream)), [None], 4, repeats=1, warm=1)[0])
-            bwd_us.append(time_launches(lambda _: ok(lib.neox_causal_softmax_bwd(
-                out.data_ptr(), dy.data_ptr(), y.data_ptr(), sc, B, n, n, code[dt], stream)), [None], 4, repeats=1, warm=1)[0])
-
-        def classes(us, nbytes, what):
-            cut = (min(us) + max(us)) / 2
-            fast = [u for u in us if u < cut]
-            slow = [u for u in us if u >= cut]
-            out = {"outputs_timed": len(us), "spread_pct": round(100 * (max(us) / min(us) - 1), 1)}
-            if out["spread_pct"] < 3.0:  # one class only: every tensor lies alike relative to the inputs
-                out["all"] = row(what, nbytes, statistics.median(us), min(us))
-                return out
-            out["faster"] = dict(row(what, nbytes, statistics.median(fast), min(fast)), outputs=len(fast))
-            out["slower"] = dict(row(what, nbytes, statistics.median(slow), min(slow)), outputs=len(slow))
-            out["class_of_each_output_in_allocation_order"] = "".join("f" if u < cut else "s" for u in us)
-            return out
-
-        return {"device_memory_GiB": round(total / 2**30, 1), "tensor_GiB": 4, "inputs": "the first three tensors allocated",
-                "fwd": classes(fwd_us, fwd_bytes, "cfg5 causal fwd [32,8192,8192] bf16"),
-                "bwd": classes(bwd_us, bwd_bytes, "cfg5 causal bwd [32,8192,8192] bf16")}
-
     def causal_mask(n):
         return torch.ones(n, n, dtype=torch.bool, device=dev).triu_(1).view(1, 1, n, n)
 
@@ -283,9 +250,8 @@ def main():
     # set than its forward launch.
     B5, n5, dt5, sc5 = 32, 8192, torch.bfloat16, 128 ** -0.5
     S5, H5, HN5 = 8192, 32, 128
-    tri5 = n5 * (n5 + 1) // 2
-    cfwd_bytes = B5 * 2 * (tri5 + n5 * n5)
-    cbwd_bytes = B5 * 2 * (2 * tri5 + n5 * n5)
+    cfwd_bytes = B5 * 2 * (tri(n5) + n5 * n5)
+    cbwd_bytes = B5 * 2 * (2 * tri(n5) + n5 * n5)
     rope_bytes = 2 * 2 * S5 * 1 * H5 * HN5 * 2 + 2 * S5 * HN5 * 4
     step_bytes = cfwd_bytes + cbwd_bytes + 2 * rope_bytes
     cset = causal_sets(B5, n5, dt5, 1238, nsets=1, need_bwd=True)[0]
@@ -335,17 +301,16 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
-        "scaling": None,  # one GPU only: every row is independent, more GPUs see a smaller batch
+        "scaling": "weak",  # per-GPU work is fixed: every row is independent, more GPUs see more batches
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16",  # bf16 in HBM; every kernel computes in fp32 and rounds once on the way out
         "data": "synthetic",
         "config": {
-            "workload": "configs[4]: long-context causal scaled softmax fwd+bwd, scores [1,32,8192,8192] "
-                        "bf16 storage, scale 1/sqrt(128), plus full rotary (rotary_pct 1.0) fwd+bwd on "
-                        "q,k [8192,1,32,128] bf16, base 10000, fp32 cos/sin",
+            "workload": "configs[4]: causal scaled softmax fwd+bwd on scores [1,32,8192,8192] bf16, scale "
+                        "1/sqrt(128), plus full rotary fwd+bwd on q,k [8192,1,32,128] bf16, base 10000, fp32 cos/sin",
             "step": "rotary fwd (q+k, one launch) + causal softmax fwd + causal softmax bwd + rotary bwd",
+            "arithmetic": "fp32 from bf16 storage, one rounding to bf16",
             "algorithmic_bytes_per_step": step_bytes,
-            "rotary_buffer_sets": len(rsets),
         },
         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 1),
         "min_pct_hbm_peak_over_configs": None,  # filled in from the per-config table below
@@ -353,7 +318,7 @@ def main():
                         "rotary_fwd": round(rfwd_us, 2), "rotary_bwd": round(rbwd_us, 2)},
         "roofline": {
             "bound": "hbm",
-            "kernel": "softmax_bwd_kernel<BF16, 2 chunks of 512 columns per wave, 8 waves per row, 1 row per block, causal>",
+            "kernel": "softmax_bwd_kernel<BF16, 2 chunks of 512 columns per wave, 8 waves per row, causal>",
             "achieved": round(cbwd_gbps, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -403,9 +368,9 @@ def main():
             "cores": cores,
             "kind": "port",
             "sample": f"1/32 of a step of configs[4]: 1 of the 32 score matrices ([1,1,8192,8192] bf16) "
-                      f"through the oracle's torch softmax path, forward + autograd backward, and {npos} of "
-                      f"the 8192 positions of q,k through its rotary expression, forward + autograd "
-                      f"backward; {reps} repetitions, {cpu_s * 1e3:.1f} ms each",
+                      f"through the oracle's torch softmax path, fwd + autograd bwd, and {npos} of the 8192 "
+                      f"positions of q,k through its rotary expression, fwd + autograd bwd; {reps} "
+                      f"repetitions, {cpu_s * 1e3:.1f} ms each",
             "ms_per_step_scaled_to_full_batch": round(cpu_s * 1e3 * B5, 1),
         }
         del xs, dys, cm, qs, ks
@@ -416,6 +381,7 @@ def main():
     n_elem = b * heads * sq * sk
     fwd_bytes = 2 * n_elem * 2 + b * sq * sk
     bwd_bytes = 3 * n_elem * 2
+
     def cpu_time_us(fn, budget_s=1.5):
         fn()
         reps, t0 = 0, time.perf_counter()
@@ -426,8 +392,11 @@ def main():
 
     def softmax_extras(r, x, y, mask, sc, dt, total, dy=None, dx=None):
         """CPU-baseline leg of a table row: the oracle's CPU time on a slice scaled to the full
-        batch, and the kernels' own output on that slice against the oracle (evaluated on the GPU
-        in fp32).  x, y (, dy, dx): [k, sq, sk] or [k, np, sq, sk] slices; mask broadcastable."""
+        batch, and the kernels' own output on that slice against the oracle's fp32 path (evaluated
+        on the GPU): the probabilities for a forward row; for a backward row autograd from x
+        (`max_abs_err`) and the closed form on the kernel's own rounded probabilities
+        (`err_vs_closed_form`).  x, y (, dy, dx): [k, sq, sk] or [k, np, sq, sk] slices; mask
+        broadcastable."""
         if R is None:
             return r
         k = x.shape[0]
@@ -440,8 +409,11 @@ def main():
         else:
             dy4 = dy if dy.dim() == 4 else dy.unsqueeze(1)
             dx4 = dx if dx.dim() == 4 else dx.unsqueeze(1)
-            r["max_abs_err"] = float((dx4.float() - R.softmax_backward_fp32(dy4, y4, sc)).abs().max())
+            _, auto = R.softmax_autograd_fp32(x4, mask, sc, dy4)
+            r["max_abs_err"] = float((dx4.float() - auto).abs().max())
+            r["err_vs_closed_form"] = float((dx4.float() - R.softmax_backward_fp32(dy4, y4, sc)).abs().max())
             r["masked_nonzero"] = int((dx4[mask.expand_as(dx4)] != 0).sum())
+            del auto
         xc, mc = x4.cpu(), mask.cpu()
         f16 = dt == torch.float16
         if dx is None:
@@ -452,7 +424,7 @@ def main():
             yc = R.forward_torch_softmax(xin, mc, sc, f16, not f16, True)
             us = cpu_time_us(lambda: torch.autograd.grad(yc, xin, gc, retain_graph=True))
         r["cpu_us_per_call"] = round(us * total / k, 1)
-        r["cpu_sample"] = f"{k} of {total} along dim 0, {torch.get_num_threads()} threads, scaled"
+        r["cpu_sample"] = f"{k}/{total} of dim 0"
         return r
 
     def rope_extras(r, S, Bb, H, HN, DR, backward):
@@ -483,22 +455,14 @@ def main():
         else:
             us = cpu_time_us(lambda: R.apply_rotary_pos_emb(qc, kc, cc, sc_))
         r["cpu_us_per_call"] = round(us * S / n, 1)
-        r["cpu_sample"] = f"{n} of {S} positions, {torch.get_num_threads()} threads, scaled"
+        r["cpu_sample"] = f"{n}/{S} positions"
         return r
 
-    # The timed step above is the judged figure; everything below is the per-shape table and the
-    # studies around it.  If one of them stops (a failed check, memory held by someone else), the
-    # line is still printed, with what stopped it.
+    # The timed step above is the judged figure; below it the per-shape table.  If a row stops (a
+    # failed check, memory held by someone else), the line is still printed, with what stopped it.
+    table = []
     try:
         if not args.no_table:
-            table = []
-
-            def want(name):
-                return args.only is None or any(part in name for part in args.only.split(","))
-
-            def tri(n):
-                return n * (n + 1) // 2
-
             # configs[0]: causal fwd, 125M shape
             if want("cfg1"):
                 B, n, dt, sc = 48, 2048, torch.bfloat16, 0.125
@@ -530,38 +494,6 @@ def main():
                 r = row("cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32", nb,
                         *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
                 table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
-                # the same rotation as the attention layer's call receives it (megatron/model/transformer.py:
-                # 826-856): the first 32 dims sliced off as views, new dense tensors returned; its backward
-                # pass works on dense gradients.  Same algorithmic bytes, dense writes.
-                for z in s_:
-                    z["oq"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
-                    z["ok"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
-                    z["ost"] = _lib.strides3(z["oq"])
-
-                def rope_sliced(t, backward):
-                    src_q, src_k, st_in = (t["oq"], t["ok"], t["ost"]) if backward else (t["q"], t["k"], t["st"])
-                    ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), src_q.data_ptr(), src_k.data_ptr(),
-                                           t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, st_in, st_in,
-                                           t["ost"], t["ost"], DR, 0, BF16, F32, backward, stream))
-
-                table.append(row("cfg3 rotary fwd q+k, rotary dims sliced off as views [2048,4,32,:32], dense tensors out", nb,
-                                 *time_launches(lambda t: rope_sliced(t, 0), s_, 200)))
-                table.append(row("cfg3 rotary bwd q+k, dense gradients [2048,4,32,32] in place", nb,
-                                 *time_launches(lambda t: rope_sliced(t, 1), s_, 200)))
-                # the rope_fusion path (megatron/model/transformer.py:844-848): whole heads out of place, the
-                # pass-through dims copied by the same launch; reads and writes all of q and k
-                for z in s_:
-                    z.pop("ok"), z.pop("ost")
-                    z["oq"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
-                    z["ok"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
-
-                def rope_whole(t):
-                    ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
-                                           t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, HN, t["st"], t["st"],
-                                           t["st"], t["st"], DR, 0, BF16, F32, 0, stream))
-
-                table.append(row("cfg3 rotary fwd q+k, whole heads out of place with the pass-through dims copied (rope_fusion)",
-                                 2 * 2 * S * Bb * H * HN * 2 + 2 * S * DR * 4, *time_launches(rope_whole, s_, 200)))
                 del s_
             # configs[3]: 20B shape
             if want("cfg4"):
@@ -601,539 +533,516 @@ def main():
                         *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, 1), s_, 200))
                 table.append(rope_extras(r, S, Bb, H, HN, DR, 1))
                 del s_
-            # rotary at head sizes of other shipped model configurations (in place over whole heads,
-            # q and k in one launch): 20B (96-dim heads, rotary_pct 0.25), a 64-dim-head model at
-            # rotary_pct 0.25, 256-dim heads at 0.25, and full rotary on 96- and 128-dim heads
-            if want("models"):
-                extra = []
-                for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
-                                         (2048, 4, 32, 80, 20), (2048, 4, 32, 80, 80),
-                                         (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
-                    s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
-                    nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-                    for bwd in (0, 1):
-                        r = row(f"rotary {'bwd' if bwd else 'fwd'} q+k [{S},{Bb},{H},{HN}] bf16 d_rot={DR}", nb,
-                                *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, bwd), s_, 200))
-                        extra.append(rope_extras(r, S, Bb, H, HN, DR, bwd))
-                    del s_
-                result["rotary_other_head_sizes"] = extra
-            # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
-            if want("copy"):
-                nbytes = 1 << 30
-                src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
-                dst = torch.empty_like(src)
-                table.append(row("copy 1 GiB (read + write)", 2 * nbytes,
-                                 *time_launches(lambda t: ok(probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(),
-                                                                                   nbytes, stream)), [None], 50)))
-            # softmax + attention dropout in one kernel per pass (the op that follows the softmax in
-            # the model), on the padded, the 20B and the long-context shapes; p = 0.1
-            if want("dropout"):
-                from gpt_neox_amd.fused_kernels import attention_dropout as rng
-
-                extras, p_drop, seed = [], 0.1, 1234
-
-                def drop_extras(r, z, k, mask, sc, fwd):
-                    """Slice [:k] along dim 0: the dropped output against torch's dropout expression
-                    on the kernel's own probabilities and keep pattern (bit-equality), or the
-                    backward against the fp32 closed form (oracle; CPU-baseline leg only)."""
-                    if R is None:
-                        return r
-                    y = z["y"][:k]
-                    keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
-                    if fwd:
-                        r["dropped_bit_equal_to_torch_expression"] = bool(
-                            torch.equal(z["y2"][:k], R.dropout_with_mask(y, keep, p_drop)))
-                        r["kept_fraction"] = round(float(keep.float().mean()), 5)
-                    else:
-                        ref = R.softmax_dropout_backward_fp32(z["dy"][:k], y, keep, p_drop, sc)
-                        r["max_abs_err"] = float((z["dx"][:k].float() - ref).abs().max())
-                        r["masked_nonzero"] = int((z["dx"][:k][mask.expand_as(y)] != 0).sum())
-                    return r
-
-                s_ = masked_sets(b, heads, sq, sk, dtype, 1240, nsets=3)
-                for z in s_:
-                    z["y2"] = torch.empty_like(z["x"])
-
-                def md_fwd(t):
-                    ok(lib.neox_masked_softmax_dropout_fwd(
-                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), None, 0, scale,
-                        p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
-
-                def md_bwd(t):
-                    ok(lib.neox_masked_softmax_dropout_bwd(
-                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0, None,
-                        b * heads * sq, sk, code[dtype], stream))
-
-                z = s_[0]
-                r = row("cfg2 padded fwd + dropout [8,16,1024,1024] fp16", 3 * n_elem * 2 + b * sq * sk,
-                        *time_launches(md_fwd, s_, 100))
-                extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, True))
-                r = row("cfg2 padded bwd + dropout [8,16,1024,1024] fp16", bwd_bytes, *time_launches(md_bwd, s_, 100))
-                extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, False))
-                del s_, z
-                for label, B, n, dt, sc, nl in (("cfg4", 64, 2048, torch.float16, 96 ** -0.5, 100),
-                                                ("cfg5", 32, 8192, torch.bfloat16, 128 ** -0.5, 30)):
-                    torch.cuda.empty_cache()
-                    s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
-                    for z in s_:
-                        z["y2"] = torch.empty_like(z["x"])
-                    cm = causal_mask(n)[0]
-
-                    def cd_fwd(t):
-                        ok(lib.neox_causal_softmax_dropout_fwd(
-                            t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), None, None, 0, sc, p_drop, seed, 0, None,
-                            B, 1, n, n, code[dt], stream))
-
-                    def cd_bwd(t):
-                        ok(lib.neox_causal_softmax_dropout_bwd(
-                            t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
-                            code[dt], stream))
-
-                    z = s_[0]
-                    shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'}"
-                    r = row(f"{label} causal fwd + dropout {shape}", B * 2 * (tri(n) + 2 * n * n),
-                            *time_launches(cd_fwd, s_, nl, warm=5))
-                    extras.append(drop_extras(r, z, 1, cm, sc, True))
-                    r = row(f"{label} causal bwd + dropout {shape}", B * 2 * (2 * tri(n) + n * n),
-                            *time_launches(cd_bwd, s_, nl, warm=5))
-                    extras.append(drop_extras(r, z, 1, cm, sc, False))
-                    del s_, z, cm
-                result["fused_dropout"] = extras
-            # relative-position bias [1, np, sq, sk] read inside the causal softmax (125M shape)
-            if want("bias"):
-                Bb, H, n, dt, sc = 4, 12, 2048, torch.bfloat16, 0.125
-                s_ = causal_sets(Bb * H, n, dt, 1242, nsets=2, need_bwd=False)
-                rpe = (torch.randn(1, H, n, n, device=dev, generator=gen(1243)) * 2).to(dt)
-
-                def cb_fwd(t):
-                    ok(lib.neox_causal_softmax_bias_fwd(t["y"].data_ptr(), t["x"].data_ptr(), rpe.data_ptr(), sc,
-                                                        Bb, H, n, n, 1, code[dt], stream))
-
-                r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
-                        Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
-                z = s_[0]
-                if R is not None:
-                    cm = causal_mask(n)
-                    ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
-                    r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
-                    r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
-                result["fused_bias"] = [r]
-                del s_, z, rpe
-            # evaluation / prefill lengths: rows that are not a multiple of 8 columns long, so that every
-            # row starts at another 2-byte alignment (causal forward, the pass an evaluation runs)
-            if want("ragged"):
-                ragged = []
-                for B, n, dt, nl in ((48, 2047, torch.bfloat16, 100), (96, 1001, torch.float16, 100), (1024, 129, torch.float16, 100)):
-                    sc = 0.125
-                    s_ = causal_sets(B, n, dt, 1245, nsets=2, need_bwd=False)
-                    name = f"causal fwd [{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} (ragged rows)"
-                    r = row(name, B * 2 * (tri(n) + n * n), *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, nl))
-                    ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
-                    del s_
-                result["evaluation_lengths"] = ragged
-            # Every kernel family over the row lengths, the shape boundaries of the dispatcher included (one
-            # length at and one just above each power of two): % of the HBM peak by algorithmic bytes, fp16,
-            # about 600 MB per tensor, three buffer sets.  Causal rows of a few columns read whole 64-byte
-            # sectors where the algorithmic count has half a row, so their figures stop at 55-60 %.
-            if want("scan") and not args.quick:
-                scan = []
-                for n in (64, 128, 129, 256, 257, 320, 512, 520, 768, 1024, 1032, 1280, 1536, 2048, 2056, 3072, 4096, 4104,
-                          6144, 8192, 8200, 12288, 16384):
-                    B = max(2, int(600e6 // (n * n * 2)))  # at least two matrices: 0.6-1.1 GB per tensor
-                    sets = []
-                    for _ in range(3):
-                        x = torch.empty(B, n, n, device=dev, dtype=torch.float16).normal_(0.0, 8.0)
-                        sets.append(dict(x=x, y=torch.empty_like(x), dy=torch.empty_like(x).normal_(), dx=torch.empty_like(x)))
-                    mask = (torch.rand(1, 1, n, n, device=dev) < 0.2).to(torch.uint8)
-                    f16 = code[torch.float16]
-                    cf = time_launches(lambda t: ok(lib.neox_causal_softmax_fwd(
-                        t["y"].data_ptr(), t["x"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-                    cb = time_launches(lambda t: ok(lib.neox_causal_softmax_bwd(
-                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-                    mf = time_launches(lambda t: ok(lib.neox_masked_softmax_fwd(
-                        t["y"].data_ptr(), t["x"].data_ptr(), mask.data_ptr(), 0.125, 1, B, n, n, 1, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-                    fb = time_launches(lambda t: ok(lib.neox_masked_softmax_bwd(
-                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B * n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-                    full = B * n * n * 2
-                    pct = lambda nbytes, us: round(100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, 1)
-                    scan.append({"sk": n, "matrices": B,
-                                 "causal_fwd_pct": pct(B * 2 * (tri(n) + n * n), cf), "causal_bwd_pct": pct(B * 2 * (2 * tri(n) + n * n), cb),
-                                 "mask_tensor_fwd_pct": pct(2 * full + n * n, mf), "full_row_bwd_pct": pct(3 * full, fb)})
-                    del sets, mask
-                result["row_length_scan_pct_of_hbm_peak"] = scan
-                torch.cuda.empty_cache()
-            # The reference's own fallback on this GPU, for scale: what FusedScaleMaskSoftmax runs when its
-            # predicate fails (always at sk > 2048, e.g. configs[4]) is the unfused torch branch
-            # (megatron/model/fused_softmax.py:184-199 with gpt2_attention_mask_func,
-            # megatron/model/gpt2_model.py:49-57), and the unfused rotary is the torch expression with the
-            # caller's slice and concatenate (megatron/model/transformer.py:826-860).  Both are timed
-            # here through this package's copies of those branches; the fused figure beside each is the
-            # sum of the kernels the fused modules launch for the same work.
-            if want("unfused"):
-                from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
-                from gpt_neox_amd.positional_embeddings import _rotary_torch
-
-                def mask_func(scores, mask_):
-                    return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
-
-                def timed(fn, n, warm=3):
-                    m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
-                    return m
-
-                fused_us = {r["op"]: r["us_per_call"] for r in table}
-                unfused = []
-
-                def softmax_row(label, shape, dt, sc, mask_, keys, n):
-                    mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, SoftmaxFusionTypes.none,
-                                                mask_func, True, sc)
-                    x = (torch.randn(shape, device=dev, generator=gen(77)) * 8).to(dt)
-                    with torch.no_grad():
-                        f_us = timed(lambda: mod(x, mask_), n)
-                    xg = x.clone().requires_grad_(True)
-                    g = torch.randn(shape, device=dev, generator=gen(78)).to(dt)
-
-                    def fb():
-                        mod(xg, mask_).backward(g)
-                        xg.grad = None
-
-                    fb_us = timed(fb, n)
-                    r = {"op": label + ": unfused torch branch", "fwd_us": round(f_us, 1), "fwd_bwd_us": round(fb_us, 1)}
-                    have = [fused_us.get(k) for k in keys]
-                    if have[0] is not None:
-                        r["fused_fwd_us"] = have[0]
-                        r["fwd_speedup"] = round(f_us / have[0], 1)
-                        if len(have) > 1 and have[1] is not None:
-                            r["fused_fwd_bwd_us"] = round(have[0] + have[1], 2)
-                            r["fwd_bwd_speedup"] = round(fb_us / (have[0] + have[1]), 1)
-                    unfused.append(r)
-
-                if not args.quick:
-                    lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(79))
-                    pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
-                    softmax_row("cfg2 padded [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale, pad,
-                                ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 20)
-                    softmax_row("cfg4 causal [1,64,2048,2048] fp16", (1, 64, 2048, 2048), torch.float16, 96 ** -0.5, causal_mask(2048),
-                                ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 20)
-                    torch.cuda.empty_cache()
-                    softmax_row("cfg5 causal [1,32,8192,8192] bf16", (1, 32, 8192, 8192), torch.bfloat16, 128 ** -0.5, causal_mask(8192),
-                                ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 5)
-                    torch.cuda.empty_cache()
-                    # partial rotary as the attention layer does it: slice, rotate, concatenate (forward)
-                    S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
-                    t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1246, nsets=1)[0]
-                    cos4 = t["cos"].view(S, 1, 1, DR).bfloat16()
-                    sin4 = t["sin"].view(S, 1, 1, DR).bfloat16()
-
-                    def layer_rotary():
-                        q_rot, q_pass = t["q"][..., :DR], t["q"][..., DR:]
-                        k_rot, k_pass = t["k"][..., :DR], t["k"][..., DR:]
-                        q2, k2 = _rotary_torch(q_rot, k_rot, cos4, sin4, 0)
-                        return torch.cat((q2, q_pass), dim=-1), torch.cat((k2, k_pass), dim=-1)
-
-                    with torch.no_grad():
-                        r_us = timed(layer_rotary, 50)
-                    r = {"op": "cfg3 partial rotary q+k [2048,4,32,128] bf16: slice + torch expression + cat",
-                         "fwd_us": round(r_us, 1)}
-                    have = fused_us.get("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32")
-                    if have is not None:
-                        r["fused_fwd_us"] = have
-                        r["fwd_speedup"] = round(r_us / have, 1)
-                    unfused.append(r)
-                    del t
-                result["unfused_reference_branches_on_this_gpu"] = unfused
-            # What the memory pattern of the in-place partial rotary costs by itself (cfg3: the first 64
-            # of every 256 bytes of q and k, 134 MB, loaded and stored back), probed with several launch
-            # shapes and split into its streams, next to dense patterns that move the same useful bytes
-            # or the same HBM traffic (whole 128-byte lines are fetched: 128 B read + 64 B written per
-            # span).  `bytes` counts the bytes a row's accesses ask for.
-            if want("pattern"):
-                pr = []
-                n_spans = 2 * 2048 * 4 * 32
-                bufs = [torch.empty(n_spans * 256, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(10)]
-
-                def strided(ld, st_, stride, threads=256, in_flight=4, spans=n_spans):
-                    return lambda t: ok(probes.neox_probe_strided(t.data_ptr(), spans, ld, st_, stride, threads,
-                                                                  in_flight, stream))
-
-                def prow(name, nbytes, fn):
-                    pr.append(row("pattern probe: " + name, nbytes, *time_launches(fn, bufs, 200)))
-
-                u = n_spans * 64
-                prow("64 of every 256 B, load + store back (cfg3's accesses), 256-thread blocks, 4 in flight", 2 * u,
-                     strided(64, 64, 256))
-                prow("the same, 1024-thread blocks", 2 * u, strided(64, 64, 256, 1024, 4))
-                prow("the same, 256-thread blocks, 8 in flight (half as many blocks)", 2 * u, strided(64, 64, 256, 256, 8))
-                prow("the same, 1024-thread blocks, 8 in flight", 2 * u, strided(64, 64, 256, 1024, 8))
-                prow("64 of every 256 B stored, the whole 128-byte line requested by the loads", 3 * u, strided(128, 64, 256))
-                prow("64 of every 256 B, load only", u, strided(64, 0, 256))
-                prow("64 of every 256 B, store only", u, strided(0, 64, 256))
-                prow("128 of every 256 B, load + store back (whole lines, half of the pages)", 4 * u, strided(128, 128, 256))
-                prow("the same useful bytes contiguous (33.5 MB loaded and stored back)", 2 * u,
-                     strided(4096, 4096, 4096, spans=u // 4096))
-                prow("the same HBM traffic contiguous (67 MB of lines loaded, half of each stored back)", 3 * u,
-                     strided(128, 64, 128))
-                pr.append(row("empty kernel, back-to-back launches", 0,
-                              *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200)))
-                # the same pattern by 4 KiB pieces, one piece per wave access, with the pieces of a block
-                # consecutive or 8 apart (every XCD on its own piece residue: the order the kernels use)
-                for per_wave in (1, 2):
-                    for order, oname in ((0, "consecutive pieces"), (1, "pieces 8 apart (XCD-aware)")):
-                        prow(f"64 of every 256 B, load + store back, one 4 KiB piece per wave access, {per_wave} per wave, {oname}",
-                             2 * u, lambda t, pw=per_wave, od=order: ok(probes.neox_probe_strided_pieces(
-                                 t.data_ptr(), n_spans * 256, 0, pw, od, stream)))
-                for op, opname in ((1, "load only"), (2, "store only")):
-                    for order, oname in ((0, "consecutive pieces"), (1, "pieces 8 apart (XCD-aware)")):
-                        prow(f"64 of every 256 B, {opname}, one 4 KiB piece per wave access, 1 per wave, {oname}", u,
-                             lambda t, o=op, od=order: ok(probes.neox_probe_strided_pieces(t.data_ptr(), n_spans * 256, o, 1, od, stream)))
-                result["memory_pattern_probes"] = pr
-                del bufs
-                # Dense streams of 1 GiB in 4 KiB pieces against the block -> piece order: workgroups go to the
-                # 8 XCDs in turn, so "8 apart" keeps every XCD on one piece residue (mod 8), "consecutive"
-                # gives it 2 or 4 residues, "rotating" all 8.
-                xp = []
-                big = [torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(2)]
-                for op, opname, moved in ((0, "write", 1 << 30), (1, "read", 1 << 30), (2, "copy", 2 << 30)):
-                    for per_block, order, oname in ((1, 0, "1 piece per block, in order"), (1, 2, "1 piece per block, rotating over the XCDs"),
-                                                    (4, 0, "4 consecutive pieces per block"), (4, 1, "4 pieces per block, 8 apart")):
-                        xp.append(row(f"{opname} 1 GiB: {oname}", moved, *time_launches(
-                            lambda t, o=op, pb=per_block, od=order: ok(probes.neox_probe_pieces(
-                                big[0].data_ptr(), big[1].data_ptr(), 1 << 30, o, pb, od, stream)), [None], 30)))
-                del big
-                # the same copy over 4 GiB per tensor (the size of the long-context score tensors): the
-                # consecutive-pieces order loses more there, the XCD-aware one does not
-                torch.cuda.empty_cache()
-                big = [torch.empty(4 << 30, dtype=torch.uint8, device=dev) for _ in range(2)]
-                big[1].random_(0, 255)
-                for per_block, order, oname in ((4, 0, "4 consecutive pieces per block"), (4, 1, "4 pieces per block, 8 apart")):
-                    xp.append(row(f"copy 4 GiB: {oname}", 8 << 30, *time_launches(
-                        lambda t, pb=per_block, od=order: ok(probes.neox_probe_pieces(
-                            big[0].data_ptr(), big[1].data_ptr(), 4 << 30, 2, pb, od, stream)), [None], 10, warm=3)))
-                result["xcd_order_probes"] = xp
-                del big
-                torch.cuda.empty_cache()
-                # cfg3 forward replayed from a HIP graph of 20 launches over distinct buffer sets: the
-                # kernel's time without the host's launch path between consecutive launches
-                S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
-                s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1247, nsets=10)
-                side = torch.cuda.Stream()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.stream(side):
-                    stream_side = side.cuda_stream
-
-                    def rope_on_side(t):
-                        ok(lib.neox_rope_apply(t["q"].data_ptr(), t["k"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
-                                               t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, t["st"], t["st"],
-                                               t["st"], t["st"], DR, 0, BF16, F32, 0, stream_side))
-
-                    rope_on_side(s_[0])
-                    side.synchronize()
-                    with torch.cuda.graph(graph, stream=side):
-                        for i in range(20):
-                            rope_on_side(s_[i % 10])
-                torch.cuda.synchronize()
-                nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-                med, best = time_launches(lambda t: graph.replay(), [None], 20, warm=3)
-                result["cfg3_from_a_hip_graph"] = row("cfg3 rotary fwd q+k, 20 launches per graph replay", nb, med / 20, best / 20)
-                del s_, graph
-            if want("placement") and not args.quick:
-                # Placement of the tensors over the memory: the long-context kernels run 5-6 % faster when a
-                # launch writes into another third of the 288 GB than it reads from (see placement_rows).
-                try:
-                    result["placement_over_the_memory"] = placement_rows()
-                except torch.cuda.OutOfMemoryError as e:  # memory held by someone else: the section is left out
-                    result["placement_over_the_memory"] = {"skipped": str(e).split("\n")[0]}
-                torch.cuda.empty_cache()
-            # The drop-in where it is dropped in: the Python modules the attention layer calls
-            # (megatron/model/transformer.py:534 FusedScaleMaskSoftmax.forward, :850-856
-            # apply_rotary_pos_emb, :844-848 fused_apply_rotary_pos_emb_cached) -- module -> autograd
-            # Function -> ctypes -> C-ABI -> kernel.  Per row: us per call of back-to-back calls
-            # (HIP events, as above: the GPU-side cost when the host keeps ahead), the C-ABI figure of the
-            # same work from the table, and the host's own time per call (wall clock of calls on a
-            # tiny input of the same kind, where the kernel is negligible).
-            if want("module"):
-                from gpt_neox_amd.fused_rope import fused_apply_rotary_pos_emb_cached
-                from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
-                from gpt_neox_amd.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_qkv_
-
-                def mask_fill(scores, mask_):
-                    return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
-
-                abi_us = {r["op"]: r["us_per_call"] for r in table}
-                mrows = []
-
-                def events_us(fn, n, warm=3):
-                    m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
-                    return m
-
-                def host_us(fn, n=2000):
-                    for _ in range(50):
-                        fn()
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
-                    for _ in range(n):
-                        fn()
-                    dt = time.perf_counter() - t0
-                    torch.cuda.synchronize()
-                    return dt / n * 1e6
-
-                def mrow(name, f_us, fb_us, host_f, host_fb, keys):
-                    r = {"op": name, "module_fwd_us": round(f_us, 2), "host_fwd_us": round(host_f, 2)}
-                    if fb_us is not None:
-                        r["module_fwd_bwd_us"] = round(fb_us, 2)
-                        r["host_fwd_bwd_us"] = round(host_fb, 2)
-                    have = [abi_us.get(k) for k in keys]
-                    if have and have[0] is not None:
-                        r["c_abi_fwd_us"] = have[0]
-                        if len(have) > 1 and have[1] is not None:
-                            r["c_abi_fwd_bwd_us"] = round(have[0] + have[1], 2)
-                    mrows.append(r)
-
-                def softmax_module_row(name, shape, dt, sc, fusion, mask_, keys, n, with_bwd=True):
-                    mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, fusion, mask_fill, True, sc)
-                    x = (torch.randn(shape[0], shape[1], shape[2], shape[3], device=dev, generator=gen(81)) * 8).to(dt) \
-                        if shape[0] * shape[1] * shape[2] * shape[3] < 2 ** 30 else None
-                    if x is None:  # chunked: no full-size fp32 temporary
-                        x = torch.empty(shape, device=dev, dtype=dt)
-                        for j in range(0, shape[1], 8):
-                            x[:, j : j + 8] = (torch.randn(x[:, j : j + 8].shape, device=dev, generator=gen(81 + j)) * 8).to(dt)
-                    mod(x[:1, :1], mask_[:1])  # the mask's verdict is decided before the timed calls
-                    with torch.no_grad():
-                        f_us = events_us(lambda: mod(x, mask_), n)
-                    fb_us = host_fb = None
-                    tiny = x[:1, :1, :16, :16].contiguous()
-                    tmask = mask_[:1, :, :16, :16].contiguous()
-                    mod(tiny, tmask)
-                    with torch.no_grad():
-                        host_f = host_us(lambda: mod(tiny, tmask))
-                    if with_bwd:
-                        xg = x.requires_grad_(True)
-                        g = torch.empty_like(x).normal_()
-
-                        def fb():
-                            mod(xg, mask_).backward(g)
-                            xg.grad = None
-
-                        fb_us = events_us(fb, n)
-                        tg = tiny.clone().requires_grad_(True)
-                        gg = torch.ones_like(tiny)
-
-                        def tiny_fb():
-                            mod(tg, tmask).backward(gg)
-                            tg.grad = None
-
-                        host_fb = host_us(tiny_fb)
-                    mrow(name, f_us, fb_us, host_f, host_fb, keys)
-
-                softmax_module_row("cfg1 FusedScaleMaskSoftmax(upper_triang) [4,12,2048,2048] bf16", (4, 12, 2048, 2048),
-                                   torch.bfloat16, 0.125, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
-                                   ["cfg1 causal fwd [48,2048,2048] bf16"], 50, with_bwd=False)
-                lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(82))
-                pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
-                softmax_module_row("cfg2 FusedScaleMaskSoftmax(general) [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale,
-                                   SoftmaxFusionTypes.general, pad,
-                                   ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 50)
-                softmax_module_row("cfg4 FusedScaleMaskSoftmax(upper_triang) [1,64,2048,2048] fp16", (1, 64, 2048, 2048),
-                                   torch.float16, 96 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
-                                   ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 50)
-                torch.cuda.empty_cache()
-                if not args.quick:
-                    softmax_module_row("cfg5 FusedScaleMaskSoftmax(upper_triang) [1,32,8192,8192] bf16", (1, 32, 8192, 8192),
-                                       torch.bfloat16, 128 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(8192),
-                                       ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 10)
-                    torch.cuda.empty_cache()
-                # a mask the module has not seen: the device-side comparison with the plain triangle and,
-                # with causal_mask_check="verify", the wait for it (paid once per new mask tensor)
-                fresh_rows = {}
-                for mode in ("verify", "lazy", "trust"):
-                    mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, mask_fill, True, 0.125,
-                                                causal_mask_check=mode)
-                    x = (torch.randn(1, 1, 8192, 8192, device=dev, generator=gen(83)) * 8).bfloat16()
-                    big = causal_mask(8192)
-                    mod(x, big)
-                    torch.cuda.synchronize()
-                    walls = []
-                    for _ in range(5):
-                        fresh = big.clone()
-                        torch.cuda.synchronize()
-                        t0 = time.perf_counter()
-                        mod(x, fresh)
-                        t1 = time.perf_counter()
-                        torch.cuda.synchronize()
-                        walls.append(((t1 - t0) * 1e6, (time.perf_counter() - t0) * 1e6))
-                    fresh_rows[mode] = {"host_returns_after_us": round(statistics.median(w[0] for w in walls), 1),
-                                        "gpu_done_after_us": round(statistics.median(w[1] for w in walls), 1)}
-                    del x, big
-                result["module_call_with_a_fresh_causal_mask_1x1x8192x8192"] = fresh_rows
-
-                # rotary through the modules: cfg3 (partial) and cfg5 (full)
-                for label, S, Bb, H, HN, DR, keys in (
-                        ("cfg3", 2048, 4, 32, 128, 32, ["cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32",
-                                                        "cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32"]),
-                        ("cfg5", 8192, 1, 32, 128, 128, ["cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128",
-                                                         "cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128"])):
-                    sets_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1250, nsets=6)
-                    cos4, sin4 = sets_[0]["cos"].view(S, 1, 1, DR), sets_[0]["sin"].view(S, 1, 1, DR)
-                    it = [0]
-
-                    def nxt():
-                        it[0] += 1
-                        return sets_[it[0] % 6]
-
-                    def sliced():  # what the attention layer does: slice, rotate (new tensors), caller concatenates
-                        t = nxt()
-                        return apply_rotary_pos_emb(t["q"][..., :DR], t["k"][..., :DR], cos4, sin4)
-
-                    def fused_rope_path():  # rope_fusion: one call per tensor, pass-through dims copied in the kernel
-                        t = nxt()
-                        return fused_apply_rotary_pos_emb_cached(t["q"], cos4, sin4), fused_apply_rotary_pos_emb_cached(t["k"], cos4, sin4)
-
-                    tq = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
-                    tk = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
-                    tc, ts_ = cos4[:4].contiguous(), sin4[:4].contiguous()
-                    with torch.no_grad():
-                        f_us = events_us(sliced, 200)
-                        hf = host_us(lambda: apply_rotary_pos_emb(tq[..., :DR], tk[..., :DR], tc, ts_))
-                        mrow(f"{label} apply_rotary_pos_emb(q[..., :{DR}], k[..., :{DR}], cos, sin) [{S},{Bb},{H},{HN}] bf16",
-                             f_us, None, hf, None, keys[:1])
-                        f_us = events_us(fused_rope_path, 200)
-                        hf = host_us(lambda: fused_apply_rotary_pos_emb_cached(tq, tc, ts_))
-                        mrow(f"{label} fused_apply_rotary_pos_emb_cached(q) + (k): whole heads out of place "
-                             f"[{S},{Bb},{H},{HN}] bf16 d2={DR}; host figure per call", f_us, None, hf, None, [])
-                    # in place on the fused QKV projection [s, b, np, 3*hn]: q and k thirds rotated, no copies
-                    mixed = [torch.randn(S, Bb, H, 3 * HN, device=dev, generator=gen(1251 + i)).bfloat16() for i in range(4)]
-                    tmixed = torch.randn(4, 1, 2, 3 * HN, device=dev).bfloat16()
-                    with torch.no_grad():
-                        def qkv_in_place():
-                            it[0] += 1
-                            return apply_rotary_pos_emb_qkv_(mixed[it[0] % 4], cos4, sin4, 0, DR)
-
-                        f_us = events_us(qkv_in_place, 200)
-                        hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
-                    mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
-                    del sets_, mixed
-                # for scale: what the host spends on torch's own smallest differentiable step
-                tx = torch.randn(16, 16, device=dev, dtype=torch.float16, requires_grad=True)
-                tgg = torch.ones_like(tx)
-
-                def torch_floor():
-                    (tx * 2.0).backward(tgg)
-                    tx.grad = None
-
-                with torch.no_grad():
-                    floor_f = host_us(lambda: tx * 2.0)
-                mrows.append({"op": "torch's own floor on this host: y = x * 2 (forward), then y.backward(g)",
-                              "host_fwd_us": round(floor_f, 2), "host_fwd_bwd_us": round(host_us(torch_floor), 2)})
-                result["module_api"] = mrows
             result["all_configs"] = table
-            pcts = [r["pct_hbm_peak"] for r in table if not r["op"].startswith("copy")]
+            pcts = [r["pct_hbm_peak"] for r in table]
             if pcts:
                 result["min_pct_hbm_peak_over_configs"] = min(pcts)
                 result["min_pct_hbm_peak_row"] = next(r["op"] for r in table if r["pct_hbm_peak"] == min(pcts))
     except Exception as e:
-        result["table_stopped_by"] = f"{type(e).__name__}: {e}"[:400]
-        result.setdefault("all_configs", locals().get("table", []))
+        result["table_stopped_by"] = f"{type(e).__name__}: {e}"[:200]
+        result.setdefault("all_configs", table)
 
-    print(json.dumps(result), flush=True)
+    # ------------------------------------------------------------------ studies (opt-in; own file)
+    if args.studies:
+        ctx = dict(locals())
+        try:
+            studies = run_studies(ctx)
+        except Exception as e:  # the line below is printed whatever happens here
+            studies = {"stopped_by": f"{type(e).__name__}: {e}"[:400]}
+        try:
+            os.makedirs(os.path.dirname(STUDIES_PATH), exist_ok=True)
+            with open(STUDIES_PATH, "w") as f:
+                json.dump(studies, f, indent=1)
+            result["studies_file"] = os.path.relpath(STUDIES_PATH, ROOT)
+        except OSError as e:
+            result["studies_file"] = f"not written: {e}"[:120]
+
+    print(json.dumps(result, allow_nan=False), flush=True)
+
+
+def run_studies(c):
+    """The measurements around the BASELINE table; returns a dict that main() writes to
+    gpurun_out/bench_studies.json.  `c` holds main()'s helpers and the table's rows."""
+    import torch
+
+    from gpt_neox_amd import _lib
+
+    args, lib, dev, stream, code, R = c["args"], c["lib"], c["dev"], c["stream"], c["code"], c["R"]
+    gen, ok, want, tri, row = c["gen"], c["ok"], c["want"], c["tri"], c["row"]
+    time_launches, causal_sets, masked_sets, rope_sets = c["time_launches"], c["causal_sets"], c["masked_sets"], c["rope_sets"]
+    causal_fwd, rope_apply, causal_mask = c["causal_fwd"], c["rope_apply"], c["causal_mask"]
+    softmax_extras, rope_extras, table = c["softmax_extras"], c["rope_extras"], c["table"]
+    b, heads, sq, sk, dtype, scale = c["b"], c["heads"], c["sq"], c["sk"], c["dtype"], c["scale"]
+    n_elem, bwd_bytes = c["n_elem"], c["bwd_bytes"]
+    BF16, F32 = _lib.NEOX_BF16, _lib.NEOX_F32
+    out = {"all_configs": table}
+
+    # configs[2] as the attention layer's call receives it, and the rope_fusion path
+    if want("cfg3"):
+        S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+        s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1236, nsets=10)
+        nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+        rows = []
+        # the first 32 dims sliced off as views, new dense tensors returned (megatron/model/transformer.py:
+        # 826-856); its backward pass works on dense gradients.  Same algorithmic bytes, dense writes.
+        for z in s_:
+            z["oq"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+            z["ok"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+            z["ost"] = _lib.strides3(z["oq"])
+
+        def rope_sliced(t, backward):
+            src_q, src_k, st_in = (t["oq"], t["ok"], t["ost"]) if backward else (t["q"], t["k"], t["st"])
+            ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), src_q.data_ptr(), src_k.data_ptr(),
+                                   t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, st_in, st_in,
+                                   t["ost"], t["ost"], DR, 0, BF16, F32, backward, stream))
+
+        rows.append(row("cfg3 rotary fwd q+k, rotary dims sliced off as views [2048,4,32,:32], dense tensors out", nb,
+                        *time_launches(lambda t: rope_sliced(t, 0), s_, 200)))
+        rows.append(row("cfg3 rotary bwd q+k, dense gradients [2048,4,32,32] in place", nb,
+                        *time_launches(lambda t: rope_sliced(t, 1), s_, 200)))
+        # the rope_fusion path (megatron/model/transformer.py:844-848): whole heads out of place, the
+        # pass-through dims copied by the same launch; reads and writes all of q and k
+        for z in s_:
+            z.pop("ok"), z.pop("ost")
+            z["oq"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+            z["ok"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+
+        def rope_whole(t):
+            ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
+                                   t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, HN, t["st"], t["st"],
+                                   t["st"], t["st"], DR, 0, BF16, F32, 0, stream))
+
+        rows.append(row("cfg3 rotary fwd q+k, whole heads out of place with the pass-through dims copied (rope_fusion)",
+                        2 * 2 * S * Bb * H * HN * 2 + 2 * S * DR * 4, *time_launches(rope_whole, s_, 200)))
+        out["partial_rotary_other_call_shapes"] = rows
+        del s_
+    # rotary at head sizes of other shipped model configurations (in place over whole heads,
+    # q and k in one launch): 20B (96-dim heads, rotary_pct 0.25), a 64-dim-head model at
+    # rotary_pct 0.25, 256-dim heads at 0.25, and full rotary on 96- and 128-dim heads
+    if want("models"):
+        extra = []
+        for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
+                                 (2048, 4, 32, 80, 20), (2048, 4, 32, 80, 80),
+                                 (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
+            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
+            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+            for bwd in (0, 1):
+                r = row(f"rotary {'bwd' if bwd else 'fwd'} q+k [{S},{Bb},{H},{HN}] bf16 d_rot={DR}", nb,
+                        *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, bwd), s_, 200))
+                extra.append(rope_extras(r, S, Bb, H, HN, DR, bwd))
+            del s_
+        out["rotary_other_head_sizes"] = extra
+    # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
+    if want("copy"):
+        try:
+            probes = load_copy_probe()
+            nbytes = 1 << 30
+            src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+            dst = torch.empty_like(src)
+            out["copy"] = [row("copy 1 GiB (read + write)", 2 * nbytes,
+                               *time_launches(lambda t: ok(probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(),
+                                                                                 nbytes, stream)), [None], 50)),
+                           row("empty kernel, back-to-back launches", 0,
+                               *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200))]
+            del src, dst
+        except ImportError as e:
+            out["copy"] = {"skipped": str(e)}
+    # softmax + attention dropout in one kernel per pass (the op that follows the softmax in
+    # the model), on the padded, the 20B and the long-context shapes; p = 0.1
+    if want("dropout"):
+        from gpt_neox_amd.fused_kernels import attention_dropout as rng
+
+        extras, p_drop, seed = [], 0.1, 1234
+
+        def drop_extras(r, z, k, mask, sc, fwd):
+            """Slice [:k] along dim 0: the dropped output against torch's dropout expression
+            on the kernel's own probabilities and keep pattern (bit-equality), or the
+            backward against the fp32 closed form (oracle; CPU-baseline leg only)."""
+            if R is None:
+                return r
+            y = z["y"][:k]
+            keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
+            if fwd:
+                r["dropped_bit_equal_to_torch_expression"] = bool(
+                    torch.equal(z["y2"][:k], R.dropout_with_mask(y, keep, p_drop)))
+                r["kept_fraction"] = round(float(keep.float().mean()), 5)
+            else:
+                ref = R.softmax_dropout_backward_fp32(z["dy"][:k], y, keep, p_drop, sc)
+                r["max_abs_err"] = float((z["dx"][:k].float() - ref).abs().max())
+                r["masked_nonzero"] = int((z["dx"][:k][mask.expand_as(y)] != 0).sum())
+            return r
+
+        s_ = masked_sets(b, heads, sq, sk, dtype, 1240, nsets=3)
+        for z in s_:
+            z["y2"] = torch.empty_like(z["x"])
+
+        def md_fwd(t):
+            ok(lib.neox_masked_softmax_dropout_fwd(
+                t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), None, 0, scale,
+                p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
+
+        def md_bwd(t):
+            ok(lib.neox_masked_softmax_dropout_bwd(
+                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0, None,
+                b * heads * sq, sk, code[dtype], stream))
+
+        z = s_[0]
+        r = row("cfg2 padded fwd + dropout [8,16,1024,1024] fp16", 3 * n_elem * 2 + b * sq * sk,
+                *time_launches(md_fwd, s_, 100))
+        extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, True))
+        r = row("cfg2 padded bwd + dropout [8,16,1024,1024] fp16", bwd_bytes, *time_launches(md_bwd, s_, 100))
+        extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, False))
+        del s_, z
+        for label, B, n, dt, sc, nl in (("cfg4", 64, 2048, torch.float16, 96 ** -0.5, 100),
+                                        ("cfg5", 32, 8192, torch.bfloat16, 128 ** -0.5, 30)):
+            torch.cuda.empty_cache()
+            s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
+            for z in s_:
+                z["y2"] = torch.empty_like(z["x"])
+            cm = causal_mask(n)[0]
+
+            def cd_fwd(t):
+                ok(lib.neox_causal_softmax_dropout_fwd(
+                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), None, None, 0, sc, p_drop, seed, 0, None,
+                    B, 1, n, n, code[dt], stream))
+
+            def cd_bwd(t):
+                ok(lib.neox_causal_softmax_dropout_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
+                    code[dt], stream))
+
+            z = s_[0]
+            shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'}"
+            r = row(f"{label} causal fwd + dropout {shape}", B * 2 * (tri(n) + 2 * n * n),
+                    *time_launches(cd_fwd, s_, nl, warm=5))
+            extras.append(drop_extras(r, z, 1, cm, sc, True))
+            r = row(f"{label} causal bwd + dropout {shape}", B * 2 * (2 * tri(n) + n * n),
+                    *time_launches(cd_bwd, s_, nl, warm=5))
+            extras.append(drop_extras(r, z, 1, cm, sc, False))
+            del s_, z, cm
+        out["fused_dropout"] = extras
+    # relative-position bias [1, np, sq, sk] read inside the causal softmax (125M shape)
+    if want("bias"):
+        Bb, H, n, dt, sc = 4, 12, 2048, torch.bfloat16, 0.125
+        s_ = causal_sets(Bb * H, n, dt, 1242, nsets=2, need_bwd=False)
+        rpe = (torch.randn(1, H, n, n, device=dev, generator=gen(1243)) * 2).to(dt)
+
+        def cb_fwd(t):
+            ok(lib.neox_causal_softmax_bias_fwd(t["y"].data_ptr(), t["x"].data_ptr(), rpe.data_ptr(), sc,
+                                                Bb, H, n, n, 1, code[dt], stream))
+
+        r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
+                Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
+        z = s_[0]
+        if R is not None:
+            cm = causal_mask(n)
+            ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
+            r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
+            r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
+        out["fused_bias"] = [r]
+        del s_, z, rpe
+    # evaluation / prefill lengths: rows that are not a multiple of 8 columns long, so that every
+    # row starts at another 2-byte alignment (causal forward, the pass an evaluation runs)
+    if want("ragged"):
+        ragged = []
+        for B, n, dt, nl in ((48, 2047, torch.bfloat16, 100), (96, 1001, torch.float16, 100), (1024, 129, torch.float16, 100)):
+            sc = 0.125
+            s_ = causal_sets(B, n, dt, 1245, nsets=2, need_bwd=False)
+            name = f"causal fwd [{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} (ragged rows)"
+            r = row(name, B * 2 * (tri(n) + n * n), *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, nl))
+            ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
+            del s_
+        out["evaluation_lengths"] = ragged
+    # Every kernel family over the row lengths, the shape boundaries of the dispatcher included (one
+    # length at and one just above each power of two): % of the HBM peak by algorithmic bytes, fp16,
+    # about 600 MB per tensor, three buffer sets.  Causal rows of a few columns read whole 64-byte
+    # sectors where the algorithmic count has half a row, so their figures stop at 55-60 %.
+    if want("scan") and not args.quick:
+        scan = []
+        for n in (64, 128, 129, 256, 257, 320, 512, 520, 768, 1024, 1032, 1280, 1536, 2048, 2056, 3072, 4096, 4104,
+                  6144, 8192, 8200, 12288, 16384):
+            B = max(2, int(600e6 // (n * n * 2)))  # at least two matrices: 0.6-1.1 GB per tensor
+            sets = []
+            for _ in range(3):
+                x = torch.empty(B, n, n, device=dev, dtype=torch.float16).normal_(0.0, 8.0)
+                sets.append(dict(x=x, y=torch.empty_like(x), dy=torch.empty_like(x).normal_(), dx=torch.empty_like(x)))
+            mask = (torch.rand(1, 1, n, n, device=dev) < 0.2).to(torch.uint8)
+            f16 = code[torch.float16]
+            cf = time_launches(lambda t: ok(lib.neox_causal_softmax_fwd(
+                t["y"].data_ptr(), t["x"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+            cb = time_launches(lambda t: ok(lib.neox_causal_softmax_bwd(
+                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+            mf = time_launches(lambda t: ok(lib.neox_masked_softmax_fwd(
+                t["y"].data_ptr(), t["x"].data_ptr(), mask.data_ptr(), 0.125, 1, B, n, n, 1, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+            fb = time_launches(lambda t: ok(lib.neox_masked_softmax_bwd(
+                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B * n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+            full = B * n * n * 2
+            pct = lambda nbytes, us: round(100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, 1)
+            scan.append({"sk": n, "matrices": B,
+                         "causal_fwd_pct": pct(B * 2 * (tri(n) + n * n), cf), "causal_bwd_pct": pct(B * 2 * (2 * tri(n) + n * n), cb),
+                         "mask_tensor_fwd_pct": pct(2 * full + n * n, mf), "full_row_bwd_pct": pct(3 * full, fb)})
+            del sets, mask
+        out["row_length_scan_pct_of_hbm_peak"] = scan
+        torch.cuda.empty_cache()
+    # The reference's own fallback on this GPU, for scale: what FusedScaleMaskSoftmax runs when its
+    # predicate fails (always at sk > 2048, e.g. configs[4]) is the unfused torch branch
+    # (megatron/model/fused_softmax.py:184-199 with gpt2_attention_mask_func,
+    # megatron/model/gpt2_model.py:49-57), and the unfused rotary is the torch expression with the
+    # caller's slice and concatenate (megatron/model/transformer.py:826-860).  Both are timed
+    # here through this package's copies of those branches; the fused figure beside each is the
+    # sum of the kernels the fused modules launch for the same work.
+    if want("unfused") and not args.quick:
+        from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+        from gpt_neox_amd.positional_embeddings import _rotary_torch
+
+        def mask_func(scores, mask_):
+            return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+
+        def timed(fn, n, warm=3):
+            m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+            return m
+
+        fused_us = {r["op"]: r["us_per_call"] for r in table}
+        unfused = []
+
+        def softmax_row(label, shape, dt, sc, mask_, keys, n):
+            mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, SoftmaxFusionTypes.none,
+                                        mask_func, True, sc)
+            x = (torch.randn(shape, device=dev, generator=gen(77)) * 8).to(dt)
+            with torch.no_grad():
+                f_us = timed(lambda: mod(x, mask_), n)
+            xg = x.clone().requires_grad_(True)
+            g = torch.randn(shape, device=dev, generator=gen(78)).to(dt)
+
+            def fb():
+                mod(xg, mask_).backward(g)
+                xg.grad = None
+
+            fb_us = timed(fb, n)
+            r = {"op": label + ": unfused torch branch", "fwd_us": round(f_us, 1), "fwd_bwd_us": round(fb_us, 1)}
+            have = [fused_us.get(k) for k in keys]
+            if have[0] is not None:
+                r["fused_fwd_us"] = have[0]
+                r["fwd_speedup"] = round(f_us / have[0], 1)
+                if len(have) > 1 and have[1] is not None:
+                    r["fused_fwd_bwd_us"] = round(have[0] + have[1], 2)
+                    r["fwd_bwd_speedup"] = round(fb_us / (have[0] + have[1]), 1)
+            unfused.append(r)
+
+        lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(79))
+        pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+        softmax_row("cfg2 padded [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale, pad,
+                    ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 20)
+        softmax_row("cfg4 causal [1,64,2048,2048] fp16", (1, 64, 2048, 2048), torch.float16, 96 ** -0.5, causal_mask(2048),
+                    ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 20)
+        torch.cuda.empty_cache()
+        softmax_row("cfg5 causal [1,32,8192,8192] bf16", (1, 32, 8192, 8192), torch.bfloat16, 128 ** -0.5, causal_mask(8192),
+                    ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 5)
+        torch.cuda.empty_cache()
+        # partial rotary as the attention layer does it: slice, rotate, concatenate (forward)
+        S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+        t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1246, nsets=1)[0]
+        cos4 = t["cos"].view(S, 1, 1, DR).bfloat16()
+        sin4 = t["sin"].view(S, 1, 1, DR).bfloat16()
+
+        def layer_rotary():
+            q_rot, q_pass = t["q"][..., :DR], t["q"][..., DR:]
+            k_rot, k_pass = t["k"][..., :DR], t["k"][..., DR:]
+            q2, k2 = _rotary_torch(q_rot, k_rot, cos4, sin4, 0)
+            return torch.cat((q2, q_pass), dim=-1), torch.cat((k2, k_pass), dim=-1)
+
+        with torch.no_grad():
+            r_us = timed(layer_rotary, 50)
+        r = {"op": "cfg3 partial rotary q+k [2048,4,32,128] bf16: slice + torch expression + cat",
+             "fwd_us": round(r_us, 1)}
+        have = fused_us.get("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32")
+        if have is not None:
+            r["fused_fwd_us"] = have
+            r["fwd_speedup"] = round(r_us / have, 1)
+        unfused.append(r)
+        del t
+        out["unfused_reference_branches_on_this_gpu"] = unfused
+    # The drop-in where it is dropped in: the Python modules the attention layer calls
+    # (megatron/model/transformer.py:534 FusedScaleMaskSoftmax.forward, :850-856
+    # apply_rotary_pos_emb, :844-848 fused_apply_rotary_pos_emb_cached) -- module -> autograd
+    # Function -> ctypes -> C-ABI -> kernel.  Per row: us per call of back-to-back calls
+    # (HIP events, as above: the GPU-side cost when the host keeps ahead), the C-ABI figure of the
+    # same work from the table, and the host's own time per call (wall clock of calls on a
+    # tiny input of the same kind, where the kernel is negligible).
+    if want("module"):
+        from gpt_neox_amd.fused_rope import fused_apply_rotary_pos_emb_cached
+        from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+        from gpt_neox_amd.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_qkv_
+
+        def mask_fill(scores, mask_):
+            return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+
+        abi_us = {r["op"]: r["us_per_call"] for r in table}
+        mrows = []
+
+        def events_us(fn, n, warm=3):
+            m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+            return m
+
+        def host_us(fn, n=2000):
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            dt = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            return dt / n * 1e6
+
+        def mrow(name, f_us, fb_us, host_f, host_fb, keys):
+            r = {"op": name, "module_fwd_us": round(f_us, 2), "host_fwd_us": round(host_f, 2)}
+            if fb_us is not None:
+                r["module_fwd_bwd_us"] = round(fb_us, 2)
+                r["host_fwd_bwd_us"] = round(host_fb, 2)
+            have = [abi_us.get(k) for k in keys]
+            if have and have[0] is not None:
+                r["c_abi_fwd_us"] = have[0]
+                if len(have) > 1 and have[1] is not None:
+                    r["c_abi_fwd_bwd_us"] = round(have[0] + have[1], 2)
+            mrows.append(r)
+
+        def softmax_module_row(name, shape, dt, sc, fusion, mask_, keys, n, with_bwd=True):
+            mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, fusion, mask_fill, True, sc)
+            x = torch.empty(shape, device=dev, dtype=dt)
+            for j in range(0, shape[1], 8):  # chunked: no full-size fp32 temporary
+                x[:, j : j + 8] = (torch.randn(x[:, j : j + 8].shape, device=dev, generator=gen(81 + j)) * 8).to(dt)
+            mod(x[:1, :1], mask_[:1])  # the mask's verdict is decided before the timed calls
+            torch.cuda.synchronize()
+            with torch.no_grad():
+                f_us = events_us(lambda: mod(x, mask_), n)
+            fb_us = host_fb = None
+            tiny = x[:1, :1, :16, :16].contiguous()
+            tmask = mask_[:1, :, :16, :16].contiguous()
+            mod(tiny, tmask)
+            with torch.no_grad():
+                host_f = host_us(lambda: mod(tiny, tmask))
+            if with_bwd:
+                xg = x.requires_grad_(True)
+                g = torch.empty_like(x).normal_()
+
+                def fb():
+                    mod(xg, mask_).backward(g)
+                    xg.grad = None
+
+                fb_us = events_us(fb, n)
+                tg = tiny.clone().requires_grad_(True)
+                gg = torch.ones_like(tiny)
+
+                def tiny_fb():
+                    mod(tg, tmask).backward(gg)
+                    tg.grad = None
+
+                host_fb = host_us(tiny_fb)
+            mrow(name, f_us, fb_us, host_f, host_fb, keys)
+
+        softmax_module_row("cfg1 FusedScaleMaskSoftmax(upper_triang) [4,12,2048,2048] bf16", (4, 12, 2048, 2048),
+                           torch.bfloat16, 0.125, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                           ["cfg1 causal fwd [48,2048,2048] bf16"], 50, with_bwd=False)
+        lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(82))
+        pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+        softmax_module_row("cfg2 FusedScaleMaskSoftmax(general) [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale,
+                           SoftmaxFusionTypes.general, pad,
+                           ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 50)
+        softmax_module_row("cfg4 FusedScaleMaskSoftmax(upper_triang) [1,64,2048,2048] fp16", (1, 64, 2048, 2048),
+                           torch.float16, 96 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                           ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 50)
+        torch.cuda.empty_cache()
+        if not args.quick:
+            softmax_module_row("cfg5 FusedScaleMaskSoftmax(upper_triang) [1,32,8192,8192] bf16", (1, 32, 8192, 8192),
+                               torch.bfloat16, 128 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(8192),
+                               ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 10)
+            torch.cuda.empty_cache()
+        # a mask the module has not seen (GPT-NeoX builds one per micro-batch): host time until the
+        # call returns and time until the GPU is done, for the default check and the two others
+        fresh_rows = {}
+        for mode in (None, "verify", "lazy", "trust"):
+            kw = {} if mode is None else {"causal_mask_check": mode}
+            mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, mask_fill, True, 0.125, **kw)
+            x = (torch.randn(1, 1, 8192, 8192, device=dev, generator=gen(83)) * 8).bfloat16()
+            big = causal_mask(8192)
+            mod(x, big)
+            torch.cuda.synchronize()
+            walls = []
+            for _ in range(5):
+                fresh = big.clone()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                mod(x, fresh)
+                t1 = time.perf_counter()
+                torch.cuda.synchronize()
+                walls.append(((t1 - t0) * 1e6, (time.perf_counter() - t0) * 1e6))
+            fresh_rows["default (%s)" % mod.causal_mask_check if mode is None else mode] = {
+                "host_returns_after_us": round(statistics.median(w[0] for w in walls), 1),
+                "gpu_done_after_us": round(statistics.median(w[1] for w in walls), 1)}
+            del x, big
+        out["module_call_with_a_fresh_causal_mask_1x1x8192x8192"] = fresh_rows
+
+        # rotary through the modules: cfg3 (partial) and cfg5 (full)
+        for label, S, Bb, H, HN, DR, keys in (
+                ("cfg3", 2048, 4, 32, 128, 32, ["cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32",
+                                                "cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32"]),
+                ("cfg5", 8192, 1, 32, 128, 128, ["cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128",
+                                                 "cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128"])):
+            sets_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1250, nsets=6)
+            cos4, sin4 = sets_[0]["cos"].view(S, 1, 1, DR), sets_[0]["sin"].view(S, 1, 1, DR)
+            it = [0]
+
+            def nxt():
+                it[0] += 1
+                return sets_[it[0] % 6]
+
+            def sliced():  # what the attention layer does: slice, rotate (new tensors), caller concatenates
+                t = nxt()
+                return apply_rotary_pos_emb(t["q"][..., :DR], t["k"][..., :DR], cos4, sin4)
+
+            def fused_rope_path():  # rope_fusion: one call per tensor, pass-through dims copied in the kernel
+                t = nxt()
+                return fused_apply_rotary_pos_emb_cached(t["q"], cos4, sin4), fused_apply_rotary_pos_emb_cached(t["k"], cos4, sin4)
+
+            tq = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+            tk = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+            tc, ts_ = cos4[:4].contiguous(), sin4[:4].contiguous()
+            with torch.no_grad():
+                f_us = events_us(sliced, 200)
+                hf = host_us(lambda: apply_rotary_pos_emb(tq[..., :DR], tk[..., :DR], tc, ts_))
+                mrow(f"{label} apply_rotary_pos_emb(q[..., :{DR}], k[..., :{DR}], cos, sin) [{S},{Bb},{H},{HN}] bf16",
+                     f_us, None, hf, None, keys[:1])
+                f_us = events_us(fused_rope_path, 200)
+                hf = host_us(lambda: fused_apply_rotary_pos_emb_cached(tq, tc, ts_))
+                mrow(f"{label} fused_apply_rotary_pos_emb_cached(q) + (k): whole heads out of place "
+                     f"[{S},{Bb},{H},{HN}] bf16 d2={DR}; host figure per call", f_us, None, hf, None, [])
+            # in place on the fused QKV projection [s, b, np, 3*hn]: q and k thirds rotated, no copies
+            mixed = [torch.randn(S, Bb, H, 3 * HN, device=dev, generator=gen(1251 + i)).bfloat16() for i in range(4)]
+            tmixed = torch.randn(4, 1, 2, 3 * HN, device=dev).bfloat16()
+            with torch.no_grad():
+                def qkv_in_place():
+                    it[0] += 1
+                    return apply_rotary_pos_emb_qkv_(mixed[it[0] % 4], cos4, sin4, 0, DR)
+
+                f_us = events_us(qkv_in_place, 200)
+                hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
+            mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
+            del sets_, mixed
+        # for scale: what the host spends on torch's own smallest differentiable step
+        tx = torch.randn(16, 16, device=dev, dtype=torch.float16, requires_grad=True)
+        tgg = torch.ones_like(tx)
+
+        def torch_floor():
+            (tx * 2.0).backward(tgg)
+            tx.grad = None
+
+        with torch.no_grad():
+            floor_f = host_us(lambda: tx * 2.0)
+        mrows.append({"op": "torch's own floor on this host: y = x * 2 (forward), then y.backward(g)",
+                      "host_fwd_us": round(floor_f, 2), "host_fwd_bwd_us": round(host_us(torch_floor), 2)})
+        out["module_api"] = mrows
+    return out
 
 
 if __name__ == "__main__":

@@ -78,9 +78,10 @@ _lock = threading.Lock()
 _lib = None
 
 
-def build(verbose=False):
-    """Compile ``libneox_fused.so`` for gfx950 with hipcc (works without a GPU)."""
-    cmd = ["make", "-C", _CSRC, "-j4", "-B"]
+def build(verbose=False, targets=("all",)):
+    """Compile ``libneox_fused.so`` for gfx950 with hipcc (works without a GPU).  ``targets``:
+    make targets; ``"probes"`` is the benchmark's copy kernel, a library of its own."""
+    cmd = ["make", "-C", _CSRC, "-j4", "-B", *targets]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         print(res.stdout)

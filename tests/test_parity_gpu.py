@@ -1445,53 +1445,6 @@ def test_one_lane_rows_at_any_alignment(device, offset):
                    R.softmax_dropout_backward_fp32(g, probs.masked_fill(causal, 0), keep, 0.25, 0.5)) <= 2 * TOL[dtype]
 
 
-def test_measurement_aids_copy_and_strided_touch(device):
-    # the benchmark's probes (their own library, not part of the product ABI) leave memory as the
-    # measurements assume: the copy copies, every strided variant stores back what it loaded
-    import bench
-
-    probes = bench.load_probes()
-    stream = torch.cuda.current_stream().cuda_stream
-    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=device)
-    dst = torch.zeros_like(src)
-    assert probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(), src.numel() - 16, stream) == 0
-    assert torch.equal(dst[:-16], src[:-16]) and (dst[-16:] == 0).all()
-    before = src.clone()
-    for threads in (256, 1024):
-        for in_flight in (4, 8):
-            for load, store in ((64, 64), (64, 0), (128, 64), (128, 128)):
-                assert probes.neox_probe_strided(src.data_ptr(), 4096, load, store, 256, threads, in_flight, stream) == 0
-            assert probes.neox_probe_strided(src.data_ptr(), 1, 4096, 4096, 4096, threads, in_flight, stream) == 0
-    assert probes.neox_probe_empty(stream) == 0
-    assert torch.equal(src, before)
-    assert probes.neox_probe_strided(src.data_ptr(), 4096, 0, 64, 256, 256, 4, stream) == 0  # store only
-    torch.cuda.synchronize()
-    # the probes by 4 KiB pieces: copies copy whatever the block -> piece order, the strided ones
-    # store back what they loaded
-    for n_pieces, orders in ((37, (0, 1)), (40, (0, 1, 2))):
-        buf = torch.randint(0, 255, (n_pieces * 4096,), dtype=torch.uint8, device=device)
-        for per_block in (1, 2, 4):
-            for order in orders:
-                out = torch.zeros_like(buf)
-                assert probes.neox_probe_pieces(out.data_ptr(), buf.data_ptr(), buf.numel(), 2, per_block, order, stream) == 0
-                assert torch.equal(out, buf), (n_pieces, per_block, order)
-                assert probes.neox_probe_pieces(out.data_ptr(), buf.data_ptr(), buf.numel(), 1, per_block, order, stream) == 0
-    buf = torch.randint(0, 255, (37 * 4096,), dtype=torch.uint8, device=device)
-    assert probes.neox_probe_pieces(buf.data_ptr(), buf.data_ptr(), buf.numel(), 2, 1, 2, stream) == -3
-    keep = buf.clone()
-    for per_wave in (1, 2, 4):
-        for order in (0, 1):
-            assert probes.neox_probe_strided_pieces(buf.data_ptr(), buf.numel(), 0, per_wave, order, stream) == 0
-            assert probes.neox_probe_strided_pieces(buf.data_ptr(), buf.numel(), 1, per_wave, order, stream) == 0
-    assert torch.equal(buf, keep)
-    assert probes.neox_probe_strided_pieces(buf.data_ptr(), buf.numel(), 2, 1, 1, stream) == 0  # zeros into the spans
-    v = buf.view(-1, 256)
-    assert (v[:, :64] == 0).all() and torch.equal(v[:, 64:], keep.view(-1, 256)[:, 64:])
-    assert probes.neox_probe_pieces(buf.data_ptr(), buf.data_ptr(), 4095, 0, 1, 0, stream) == -3
-    assert probes.neox_probe_strided(src.data_ptr(), 4096, 24, 64, 256, 256, 4, stream) == -3
-    assert probes.neox_probe_strided(src.data_ptr(), 4096, 64, 64, 256, 512, 4, stream) == -3
-
-
 def test_mask_and_bias_tensors_beyond_4_gib(device):
     # short rows whose mask / bias tensor no longer fits a 32-bit buffer: the several-rows-per-wave
     # kernels step aside for the row kernels, which address every row through its own buffer
