@@ -26,8 +26,8 @@ The LAST line of stdout is one compact ASCII JSON object (under 6 KB):
                  from x; rotary: bit-equality with the fp32 expression rounded once);
 * min_pct_hbm_peak_over_configs -- the lowest % of HBM peak over those rows.
 
---studies adds the measurements around the table (fused dropout, bias and ALiBi variants, other
-head sizes, ragged lengths, a scan over the row lengths, the unfused torch branches on this GPU,
+--studies adds the measurements around the table (fused dropout, bias and ALiBi variants, sliding-window
+masks, other head sizes, ragged lengths, a scan over the row lengths, the unfused torch branches on this GPU,
 the Python modules against the C-ABI, a plain copy) and writes them to
 gpurun_out/bench_studies.json; none of them runs by default and none enters the line.
 
@@ -577,213 +577,308 @@ def run_studies(c):
     BF16, F32 = _lib.NEOX_BF16, _lib.NEOX_F32
     out = {"all_configs": table}
 
+    class section:
+        """A study section: if it stops (a failed launch, memory held by someone else), the others still run."""
+
+        def __init__(self, name):
+            self.name = name
+
+        def __enter__(self):
+            return self
+
+        def __exit__(self, kind, value, tb):
+            if kind is None or not issubclass(kind, Exception):
+                return False
+            out.setdefault("stopped_sections", {})[self.name] = f"{kind.__name__}: {value}"[:300]
+            torch.cuda.empty_cache()
+            return True
+
     # configs[2] as the attention layer's call receives it, and the rope_fusion path
     if want("cfg3"):
-        S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
-        s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1236, nsets=10)
-        nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-        rows = []
-        # the first 32 dims sliced off as views, new dense tensors returned (megatron/model/transformer.py:
-        # 826-856); its backward pass works on dense gradients.  Same algorithmic bytes, dense writes.
-        for z in s_:
-            z["oq"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
-            z["ok"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
-            z["ost"] = _lib.strides3(z["oq"])
+        with section("cfg3"):
+            S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1236, nsets=10)
+            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+            rows = []
+            # the first 32 dims sliced off as views, new dense tensors returned (megatron/model/transformer.py:
+            # 826-856); its backward pass works on dense gradients.  Same algorithmic bytes, dense writes.
+            for z in s_:
+                z["oq"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+                z["ok"] = torch.empty(S, Bb, H, DR, device=dev, dtype=torch.bfloat16)
+                z["ost"] = _lib.strides3(z["oq"])
 
-        def rope_sliced(t, backward):
-            src_q, src_k, st_in = (t["oq"], t["ok"], t["ost"]) if backward else (t["q"], t["k"], t["st"])
-            ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), src_q.data_ptr(), src_k.data_ptr(),
-                                   t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, st_in, st_in,
-                                   t["ost"], t["ost"], DR, 0, BF16, F32, backward, stream))
+            def rope_sliced(t, backward):
+                src_q, src_k, st_in = (t["oq"], t["ok"], t["ost"]) if backward else (t["q"], t["k"], t["st"])
+                ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), src_q.data_ptr(), src_k.data_ptr(),
+                                       t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, DR, st_in, st_in,
+                                       t["ost"], t["ost"], DR, 0, BF16, F32, backward, stream))
 
-        rows.append(row("cfg3 rotary fwd q+k, rotary dims sliced off as views [2048,4,32,:32], dense tensors out", nb,
-                        *time_launches(lambda t: rope_sliced(t, 0), s_, 200)))
-        rows.append(row("cfg3 rotary bwd q+k, dense gradients [2048,4,32,32] in place", nb,
-                        *time_launches(lambda t: rope_sliced(t, 1), s_, 200)))
-        # the rope_fusion path (megatron/model/transformer.py:844-848): whole heads out of place, the
-        # pass-through dims copied by the same launch; reads and writes all of q and k
-        for z in s_:
-            z.pop("ok"), z.pop("ost")
-            z["oq"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
-            z["ok"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+            rows.append(row("cfg3 rotary fwd q+k, rotary dims sliced off as views [2048,4,32,:32], dense tensors out", nb,
+                            *time_launches(lambda t: rope_sliced(t, 0), s_, 200)))
+            rows.append(row("cfg3 rotary bwd q+k, dense gradients [2048,4,32,32] in place", nb,
+                            *time_launches(lambda t: rope_sliced(t, 1), s_, 200)))
+            # the rope_fusion path (megatron/model/transformer.py:844-848): whole heads out of place, the
+            # pass-through dims copied by the same launch; reads and writes all of q and k
+            for z in s_:
+                z.pop("ok"), z.pop("ost")
+                z["oq"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
+                z["ok"] = torch.empty(S, Bb, H, HN, device=dev, dtype=torch.bfloat16)
 
-        def rope_whole(t):
-            ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
-                                   t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, HN, t["st"], t["st"],
-                                   t["st"], t["st"], DR, 0, BF16, F32, 0, stream))
+            def rope_whole(t):
+                ok(lib.neox_rope_apply(t["oq"].data_ptr(), t["ok"].data_ptr(), t["q"].data_ptr(), t["k"].data_ptr(),
+                                       t["cos"].data_ptr(), t["sin"].data_ptr(), S, Bb, H, H, DR, HN, t["st"], t["st"],
+                                       t["st"], t["st"], DR, 0, BF16, F32, 0, stream))
 
-        rows.append(row("cfg3 rotary fwd q+k, whole heads out of place with the pass-through dims copied (rope_fusion)",
-                        2 * 2 * S * Bb * H * HN * 2 + 2 * S * DR * 4, *time_launches(rope_whole, s_, 200)))
-        out["partial_rotary_other_call_shapes"] = rows
-        del s_
+            rows.append(row("cfg3 rotary fwd q+k, whole heads out of place with the pass-through dims copied (rope_fusion)",
+                            2 * 2 * S * Bb * H * HN * 2 + 2 * S * DR * 4, *time_launches(rope_whole, s_, 200)))
+            out["partial_rotary_other_call_shapes"] = rows
+            del s_
     # rotary at head sizes of other shipped model configurations (in place over whole heads,
     # q and k in one launch): 20B (96-dim heads, rotary_pct 0.25), a 64-dim-head model at
     # rotary_pct 0.25, 256-dim heads at 0.25, and full rotary on 96- and 128-dim heads
     if want("models"):
-        extra = []
-        for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
-                                 (2048, 4, 32, 80, 20), (2048, 4, 32, 80, 80),
-                                 (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
-            s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
-            nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
-            for bwd in (0, 1):
-                r = row(f"rotary {'bwd' if bwd else 'fwd'} q+k [{S},{Bb},{H},{HN}] bf16 d_rot={DR}", nb,
-                        *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, bwd), s_, 200))
-                extra.append(rope_extras(r, S, Bb, H, HN, DR, bwd))
-            del s_
-        out["rotary_other_head_sizes"] = extra
+        with section("models"):
+            extra = []
+            for S, Bb, H, HN, DR in ((2048, 4, 64, 96, 24), (2048, 8, 12, 64, 16), (2048, 4, 16, 256, 64),
+                                     (2048, 4, 32, 80, 20), (2048, 4, 32, 80, 80),
+                                     (2048, 4, 64, 96, 96), (2048, 4, 40, 128, 128)):
+                s_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1244, nsets=8)
+                nb = 2 * 2 * S * Bb * H * DR * 2 + 2 * S * DR * 4
+                for bwd in (0, 1):
+                    r = row(f"rotary {'bwd' if bwd else 'fwd'} q+k [{S},{Bb},{H},{HN}] bf16 d_rot={DR}", nb,
+                            *time_launches(lambda t: rope_apply(t, S, Bb, H, DR, torch.bfloat16, bwd), s_, 200))
+                    extra.append(rope_extras(r, S, Bb, H, HN, DR, bwd))
+                del s_
+            out["rotary_other_head_sizes"] = extra
     # plain copy of 1 GiB with the same access shape: what this HBM sustains for read+write
     if want("copy"):
-        try:
-            probes = load_copy_probe()
-            nbytes = 1 << 30
-            src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
-            dst = torch.empty_like(src)
-            out["copy"] = [row("copy 1 GiB (read + write)", 2 * nbytes,
-                               *time_launches(lambda t: ok(probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(),
-                                                                                 nbytes, stream)), [None], 50)),
-                           row("empty kernel, back-to-back launches", 0,
-                               *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200))]
-            del src, dst
-        except ImportError as e:
-            out["copy"] = {"skipped": str(e)}
+        with section("copy"):
+            try:
+                probes = load_copy_probe()
+                nbytes = 1 << 30
+                src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+                dst = torch.empty_like(src)
+                out["copy"] = [row("copy 1 GiB (read + write)", 2 * nbytes,
+                                   *time_launches(lambda t: ok(probes.neox_probe_copy(dst.data_ptr(), src.data_ptr(),
+                                                                                     nbytes, stream)), [None], 50)),
+                               row("empty kernel, back-to-back launches", 0,
+                                   *time_launches(lambda t: ok(probes.neox_probe_empty(stream)), [None], 200))]
+                del src, dst
+            except ImportError as e:
+                out["copy"] = {"skipped": str(e)}
     # softmax + attention dropout in one kernel per pass (the op that follows the softmax in
     # the model), on the padded, the 20B and the long-context shapes; p = 0.1
     if want("dropout"):
-        from gpt_neox_amd.fused_kernels import attention_dropout as rng
+        with section("dropout"):
+            from gpt_neox_amd.fused_kernels import attention_dropout as rng
 
-        extras, p_drop, seed = [], 0.1, 1234
+            extras, p_drop, seed = [], 0.1, 1234
 
-        def drop_extras(r, z, k, mask, sc, fwd):
-            """Slice [:k] along dim 0: the dropped output against torch's dropout expression
-            on the kernel's own probabilities and keep pattern (bit-equality), or the
-            backward against the fp32 closed form (oracle; CPU-baseline leg only)."""
-            if R is None:
+            def drop_extras(r, z, k, mask, sc, fwd):
+                """Slice [:k] along dim 0: the dropped output against torch's dropout expression
+                on the kernel's own probabilities and keep pattern (bit-equality), or the
+                backward against the fp32 closed form (oracle; CPU-baseline leg only)."""
+                if R is None:
+                    return r
+                y = z["y"][:k]
+                keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
+                if fwd:
+                    r["dropped_bit_equal_to_torch_expression"] = bool(
+                        torch.equal(z["y2"][:k], R.dropout_with_mask(y, keep, p_drop)))
+                    r["kept_fraction"] = round(float(keep.float().mean()), 5)
+                else:
+                    ref = R.softmax_dropout_backward_fp32(z["dy"][:k], y, keep, p_drop, sc)
+                    r["max_abs_err"] = float((z["dx"][:k].float() - ref).abs().max())
+                    r["masked_nonzero"] = int((z["dx"][:k][mask.expand_as(y)] != 0).sum())
                 return r
-            y = z["y"][:k]
-            keep = rng.keep_mask(y.numel(), p_drop, seed, 0, dev).view(y.shape)
-            if fwd:
-                r["dropped_bit_equal_to_torch_expression"] = bool(
-                    torch.equal(z["y2"][:k], R.dropout_with_mask(y, keep, p_drop)))
-                r["kept_fraction"] = round(float(keep.float().mean()), 5)
-            else:
-                ref = R.softmax_dropout_backward_fp32(z["dy"][:k], y, keep, p_drop, sc)
-                r["max_abs_err"] = float((z["dx"][:k].float() - ref).abs().max())
-                r["masked_nonzero"] = int((z["dx"][:k][mask.expand_as(y)] != 0).sum())
-            return r
 
-        s_ = masked_sets(b, heads, sq, sk, dtype, 1240, nsets=3)
-        for z in s_:
-            z["y2"] = torch.empty_like(z["x"])
-
-        def md_fwd(t):
-            ok(lib.neox_masked_softmax_dropout_fwd(
-                t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), None, 0, scale,
-                p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
-
-        def md_bwd(t):
-            ok(lib.neox_masked_softmax_dropout_bwd(
-                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0, None,
-                b * heads * sq, sk, code[dtype], stream))
-
-        z = s_[0]
-        r = row("cfg2 padded fwd + dropout [8,16,1024,1024] fp16", 3 * n_elem * 2 + b * sq * sk,
-                *time_launches(md_fwd, s_, 100))
-        extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, True))
-        r = row("cfg2 padded bwd + dropout [8,16,1024,1024] fp16", bwd_bytes, *time_launches(md_bwd, s_, 100))
-        extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, False))
-        del s_, z
-        for label, B, n, dt, sc, nl in (("cfg4", 64, 2048, torch.float16, 96 ** -0.5, 100),
-                                        ("cfg5", 32, 8192, torch.bfloat16, 128 ** -0.5, 30)):
-            torch.cuda.empty_cache()
-            s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
+            s_ = masked_sets(b, heads, sq, sk, dtype, 1240, nsets=3)
             for z in s_:
                 z["y2"] = torch.empty_like(z["x"])
-            cm = causal_mask(n)[0]
 
-            def cd_fwd(t):
-                ok(lib.neox_causal_softmax_dropout_fwd(
-                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), None, None, 0, sc, p_drop, seed, 0, None,
-                    B, 1, n, n, code[dt], stream))
+            def md_fwd(t):
+                ok(lib.neox_masked_softmax_dropout_fwd(
+                    t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), t["mask"].data_ptr(), None, None, 0, scale,
+                    p_drop, seed, 0, None, b, heads, sq, sk, b, code[dtype], stream))
 
-            def cd_bwd(t):
-                ok(lib.neox_causal_softmax_dropout_bwd(
-                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
-                    code[dt], stream))
+            def md_bwd(t):
+                ok(lib.neox_masked_softmax_dropout_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), scale, p_drop, seed, 0, None,
+                    b * heads * sq, sk, code[dtype], stream))
 
             z = s_[0]
-            shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'}"
-            r = row(f"{label} causal fwd + dropout {shape}", B * 2 * (tri(n) + 2 * n * n),
-                    *time_launches(cd_fwd, s_, nl, warm=5))
-            extras.append(drop_extras(r, z, 1, cm, sc, True))
-            r = row(f"{label} causal bwd + dropout {shape}", B * 2 * (2 * tri(n) + n * n),
-                    *time_launches(cd_bwd, s_, nl, warm=5))
-            extras.append(drop_extras(r, z, 1, cm, sc, False))
-            del s_, z, cm
-        out["fused_dropout"] = extras
+            r = row("cfg2 padded fwd + dropout [8,16,1024,1024] fp16", 3 * n_elem * 2 + b * sq * sk,
+                    *time_launches(md_fwd, s_, 100))
+            extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, True))
+            r = row("cfg2 padded bwd + dropout [8,16,1024,1024] fp16", bwd_bytes, *time_launches(md_bwd, s_, 100))
+            extras.append(drop_extras(r, z, 1, z["mask"][:1], scale, False))
+            del s_, z
+            for label, B, n, dt, sc, nl in (("cfg4", 64, 2048, torch.float16, 96 ** -0.5, 100),
+                                            ("cfg5", 32, 8192, torch.bfloat16, 128 ** -0.5, 30)):
+                torch.cuda.empty_cache()
+                s_ = causal_sets(B, n, dt, 1241, nsets=1 if n > 4096 else 2, need_bwd=True)
+                for z in s_:
+                    z["y2"] = torch.empty_like(z["x"])
+                cm = causal_mask(n)[0]
+
+                def cd_fwd(t):
+                    ok(lib.neox_causal_softmax_dropout_fwd(
+                        t["y2"].data_ptr(), t["y"].data_ptr(), t["x"].data_ptr(), None, None, 0, sc, p_drop, seed, 0, None,
+                        B, 1, n, n, code[dt], stream))
+
+                def cd_bwd(t):
+                    ok(lib.neox_causal_softmax_dropout_bwd(
+                        t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, p_drop, seed, 0, None, B, n, n,
+                        code[dt], stream))
+
+                z = s_[0]
+                shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'}"
+                r = row(f"{label} causal fwd + dropout {shape}", B * 2 * (tri(n) + 2 * n * n),
+                        *time_launches(cd_fwd, s_, nl, warm=5))
+                extras.append(drop_extras(r, z, 1, cm, sc, True))
+                r = row(f"{label} causal bwd + dropout {shape}", B * 2 * (2 * tri(n) + n * n),
+                        *time_launches(cd_bwd, s_, nl, warm=5))
+                extras.append(drop_extras(r, z, 1, cm, sc, False))
+                del s_, z, cm
+            out["fused_dropout"] = extras
     # relative-position bias [1, np, sq, sk] read inside the causal softmax (125M shape)
     if want("bias"):
-        Bb, H, n, dt, sc = 4, 12, 2048, torch.bfloat16, 0.125
-        s_ = causal_sets(Bb * H, n, dt, 1242, nsets=2, need_bwd=False)
-        rpe = (torch.randn(1, H, n, n, device=dev, generator=gen(1243)) * 2).to(dt)
+        with section("bias"):
+            Bb, H, n, dt, sc = 4, 12, 2048, torch.bfloat16, 0.125
+            s_ = causal_sets(Bb * H, n, dt, 1242, nsets=2, need_bwd=False)
+            rpe = (torch.randn(1, H, n, n, device=dev, generator=gen(1243)) * 2).to(dt)
 
-        def cb_fwd(t):
-            ok(lib.neox_causal_softmax_bias_fwd(t["y"].data_ptr(), t["x"].data_ptr(), rpe.data_ptr(), sc,
-                                                Bb, H, n, n, 1, code[dt], stream))
+            def cb_fwd(t):
+                ok(lib.neox_causal_softmax_bias_fwd(t["y"].data_ptr(), t["x"].data_ptr(), rpe.data_ptr(), None, sc,
+                                                    Bb, H, n, n, 1, code[dt], stream))
 
-        r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
-                Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
-        z = s_[0]
-        if R is not None:
-            cm = causal_mask(n)
-            ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
-            r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
-            r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
-        out["fused_bias"] = [r]
-        del s_, z, rpe
+            r = row("cfg1 causal fwd + bias tensor [4,12,2048,2048] bf16, bias [1,12,2048,2048]",
+                    Bb * H * 2 * (tri(n) + n * n) + H * 2 * tri(n), *time_launches(cb_fwd, s_, 100))
+            z = s_[0]
+            if R is not None:
+                cm = causal_mask(n)
+                ref = R.softmax_fp32(z["x"][:2].float().unsqueeze(0) + rpe[:, :2].float(), cm, sc)
+                r["max_abs_err"] = float((z["y"][:2].float().unsqueeze(0) - ref).abs().max())
+                r["masked_nonzero"] = int((z["y"][:2].unsqueeze(0)[cm.expand(1, 2, n, n)] != 0).sum())
+            out["fused_bias"] = [r]
+            del s_, z, rpe
+    # causal softmax under a sliding window (megatron/utils.py:67-80; the Mistral 7B configuration trains
+    # 8192 tokens with a window of 4096): the band kernels read no mask and no score outside the band.
+    # Algorithmic bytes: the band read once (twice in the backward pass: gradient and probabilities),
+    # the dense output written -- band = sum over the rows of min(i, w) + 1 elements.  Beside them the
+    # mask-tensor kernels on the same mask (what serves such a mask without the band kernels), timed
+    # and priced by the same bytes.
+    if want("window"):
+        with section("window"):
+            rows_w = []
+            for B, n, w, dt, nl in ((32, 8192, 4096, torch.bfloat16, 30), (64, 2048, 1024, torch.float16, 100),
+                                    (8, 16384, 4096, torch.bfloat16, 30)):
+                torch.cuda.empty_cache()
+                sc = 0.125
+                s_ = causal_sets(B, n, dt, 1260, nsets=1 if n > 4096 else 2, need_bwd=True)
+                band = (w + 1) * (w + 2) // 2 + (n - 1 - w) * (w + 1)
+                shape = f"[{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} window {w}"
+
+                def wf(t):
+                    ok(lib.neox_sliding_window_softmax_fwd(t["y"].data_ptr(), t["x"].data_ptr(), sc, B, n, n, w, code[dt], stream))
+
+                def wb(t):
+                    ok(lib.neox_sliding_window_softmax_bwd(t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), sc, B, n, n, w,
+                                                           code[dt], stream))
+
+                r = row(f"sliding-window causal fwd {shape}", B * 2 * (band + n * n), *time_launches(wf, s_, nl, warm=5))
+                z = s_[0]
+                wmask = None
+                if R is not None:
+                    wmask = R.get_attn_mask(n, dev, sliding_window_width=w)
+                    k = 1
+                    ref, auto = R.softmax_autograd_fp32(z["x"][:k].unsqueeze(1), wmask, sc, z["dy"][:k].unsqueeze(1))
+                    r["max_abs_err"] = float((z["y"][:k].unsqueeze(1).float() - ref).abs().max())
+                    r["masked_nonzero"] = int((z["y"][:k].unsqueeze(1)[wmask.expand(k, 1, n, n)] != 0).sum())
+                rows_w.append(r)
+                r = row(f"sliding-window causal bwd {shape}", B * 2 * (2 * band + n * n), *time_launches(wb, s_, nl, warm=5))
+                if R is not None:
+                    r["max_abs_err"] = float((z["dx"][:k].unsqueeze(1).float() - auto).abs().max())
+                    r["masked_nonzero"] = int((z["dx"][:k].unsqueeze(1)[wmask.expand(k, 1, n, n)] != 0).sum())
+                    del ref, auto
+                rows_w.append(r)
+                m8 = (wmask if wmask is not None else
+                      (torch.ones(n, n, dtype=torch.bool, device=dev).triu_(1) | torch.ones(n, n, dtype=torch.bool, device=dev).tril_(-w - 1)).view(1, 1, n, n))
+
+                def mf(t):
+                    ok(lib.neox_masked_softmax_fwd(t["y"].data_ptr(), t["x"].data_ptr(), m8.data_ptr(), sc, 1, B, n, n, 1, code[dt], stream))
+
+                rows_w.append(row(f"the same mask as a tensor, mask-tensor fwd {shape}", B * 2 * (band + n * n),
+                                  *time_launches(mf, s_, nl, warm=5)))
+                del s_, z, m8, wmask
+            out["sliding_window"] = rows_w
+    # ALiBi slopes folded into the kernels: causal (BLOOM-style training shape) and with a mask tensor
+    if want("alibi"):
+        with section("alibi"):
+            Bb, H, n, dt, sc = 4, 16, 2048, torch.bfloat16, 0.125
+            s_ = causal_sets(Bb * H, n, dt, 1270, nsets=2, need_bwd=False)
+            slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], device=dev)
+            pad = (torch.arange(n, device=dev)[None, None, None, :] >= torch.tensor([1500, 2048, 1024, 2000], device=dev)[:, None, None, None])
+            pad = pad.expand(Bb, 1, n, n).contiguous()
+
+            def ca(t):
+                ok(lib.neox_causal_softmax_alibi_fwd(t["y"].data_ptr(), t["x"].data_ptr(), slopes.data_ptr(), sc, Bb, H, n, n,
+                                                     code[dt], stream))
+
+            def ma(t):
+                ok(lib.neox_masked_softmax_alibi_fwd(t["y"].data_ptr(), t["x"].data_ptr(), pad.data_ptr(), slopes.data_ptr(), sc,
+                                                     Bb, H, n, n, Bb, code[dt], stream))
+
+            out["fused_alibi"] = [
+                row("causal fwd + ALiBi [4,16,2048,2048] bf16", Bb * H * 2 * (tri(n) + n * n), *time_launches(ca, s_, 100)),
+                row("mask-tensor fwd + ALiBi [4,16,2048,2048] bf16, padding mask [4,1,2048,2048]",
+                    Bb * H * 2 * 2 * n * n + Bb * n * n, *time_launches(ma, s_, 100))]
+            del s_
     # evaluation / prefill lengths: rows that are not a multiple of 8 columns long, so that every
     # row starts at another 2-byte alignment (causal forward, the pass an evaluation runs)
     if want("ragged"):
-        ragged = []
-        for B, n, dt, nl in ((48, 2047, torch.bfloat16, 100), (96, 1001, torch.float16, 100), (1024, 129, torch.float16, 100)):
-            sc = 0.125
-            s_ = causal_sets(B, n, dt, 1245, nsets=2, need_bwd=False)
-            name = f"causal fwd [{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} (ragged rows)"
-            r = row(name, B * 2 * (tri(n) + n * n), *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, nl))
-            ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
-            del s_
-        out["evaluation_lengths"] = ragged
+        with section("ragged"):
+            ragged = []
+            for B, n, dt, nl in ((48, 2047, torch.bfloat16, 100), (96, 1001, torch.float16, 100), (1024, 129, torch.float16, 100)):
+                sc = 0.125
+                s_ = causal_sets(B, n, dt, 1245, nsets=2, need_bwd=False)
+                name = f"causal fwd [{B},{n},{n}] {'fp16' if dt == torch.float16 else 'bf16'} (ragged rows)"
+                r = row(name, B * 2 * (tri(n) + n * n), *time_launches(lambda t: causal_fwd(t, B, n, dt, sc), s_, nl))
+                ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
+                del s_
+            out["evaluation_lengths"] = ragged
     # Every kernel family over the row lengths, the shape boundaries of the dispatcher included (one
     # length at and one just above each power of two): % of the HBM peak by algorithmic bytes, fp16,
     # about 600 MB per tensor, three buffer sets.  Causal rows of a few columns read whole 64-byte
     # sectors where the algorithmic count has half a row, so their figures stop at 55-60 %.
     if want("scan") and not args.quick:
-        scan = []
-        for n in (64, 128, 129, 256, 257, 320, 512, 520, 768, 1024, 1032, 1280, 1536, 2048, 2056, 3072, 4096, 4104,
-                  6144, 8192, 8200, 12288, 16384):
-            B = max(2, int(600e6 // (n * n * 2)))  # at least two matrices: 0.6-1.1 GB per tensor
-            sets = []
-            for _ in range(3):
-                x = torch.empty(B, n, n, device=dev, dtype=torch.float16).normal_(0.0, 8.0)
-                sets.append(dict(x=x, y=torch.empty_like(x), dy=torch.empty_like(x).normal_(), dx=torch.empty_like(x)))
-            mask = (torch.rand(1, 1, n, n, device=dev) < 0.2).to(torch.uint8)
-            f16 = code[torch.float16]
-            cf = time_launches(lambda t: ok(lib.neox_causal_softmax_fwd(
-                t["y"].data_ptr(), t["x"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-            cb = time_launches(lambda t: ok(lib.neox_causal_softmax_bwd(
-                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-            mf = time_launches(lambda t: ok(lib.neox_masked_softmax_fwd(
-                t["y"].data_ptr(), t["x"].data_ptr(), mask.data_ptr(), 0.125, 1, B, n, n, 1, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-            fb = time_launches(lambda t: ok(lib.neox_masked_softmax_bwd(
-                t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B * n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
-            full = B * n * n * 2
-            pct = lambda nbytes, us: round(100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, 1)
-            scan.append({"sk": n, "matrices": B,
-                         "causal_fwd_pct": pct(B * 2 * (tri(n) + n * n), cf), "causal_bwd_pct": pct(B * 2 * (2 * tri(n) + n * n), cb),
-                         "mask_tensor_fwd_pct": pct(2 * full + n * n, mf), "full_row_bwd_pct": pct(3 * full, fb)})
-            del sets, mask
-        out["row_length_scan_pct_of_hbm_peak"] = scan
-        torch.cuda.empty_cache()
+        with section("scan"):
+            scan = []
+            for n in (64, 128, 129, 256, 257, 320, 512, 520, 768, 1024, 1032, 1280, 1536, 2048, 2056, 3072, 4096, 4104,
+                      6144, 8192, 8200, 12288, 16384):
+                B = max(2, int(600e6 // (n * n * 2)))  # at least two matrices: 0.6-1.1 GB per tensor
+                sets = []
+                for _ in range(3):
+                    x = torch.empty(B, n, n, device=dev, dtype=torch.float16).normal_(0.0, 8.0)
+                    sets.append(dict(x=x, y=torch.empty_like(x), dy=torch.empty_like(x).normal_(), dx=torch.empty_like(x)))
+                mask = (torch.rand(1, 1, n, n, device=dev) < 0.2).to(torch.uint8)
+                f16 = code[torch.float16]
+                cf = time_launches(lambda t: ok(lib.neox_causal_softmax_fwd(
+                    t["y"].data_ptr(), t["x"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                cb = time_launches(lambda t: ok(lib.neox_causal_softmax_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B, n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                mf = time_launches(lambda t: ok(lib.neox_masked_softmax_fwd(
+                    t["y"].data_ptr(), t["x"].data_ptr(), mask.data_ptr(), 0.125, 1, B, n, n, 1, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                fb = time_launches(lambda t: ok(lib.neox_masked_softmax_bwd(
+                    t["dx"].data_ptr(), t["dy"].data_ptr(), t["y"].data_ptr(), 0.125, B * n, n, f16, stream)), sets, 20, repeats=3, warm=5)[0]
+                full = B * n * n * 2
+                pct = lambda nbytes, us: round(100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, 1)
+                scan.append({"sk": n, "matrices": B,
+                             "causal_fwd_pct": pct(B * 2 * (tri(n) + n * n), cf), "causal_bwd_pct": pct(B * 2 * (2 * tri(n) + n * n), cb),
+                             "mask_tensor_fwd_pct": pct(2 * full + n * n, mf), "full_row_bwd_pct": pct(3 * full, fb)})
+                del sets, mask
+            out["row_length_scan_pct_of_hbm_peak"] = scan
+            torch.cuda.empty_cache()
     # The reference's own fallback on this GPU, for scale: what FusedScaleMaskSoftmax runs when its
     # predicate fails (always at sk > 2048, e.g. configs[4]) is the unfused torch branch
     # (megatron/model/fused_softmax.py:184-199 with gpt2_attention_mask_func,
@@ -792,76 +887,77 @@ def run_studies(c):
     # here through this package's copies of those branches; the fused figure beside each is the
     # sum of the kernels the fused modules launch for the same work.
     if want("unfused") and not args.quick:
-        from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
-        from gpt_neox_amd.positional_embeddings import _rotary_torch
+        with section("unfused"):
+            from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+            from gpt_neox_amd.positional_embeddings import _rotary_torch
 
-        def mask_func(scores, mask_):
-            return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+            def mask_func(scores, mask_):
+                return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
 
-        def timed(fn, n, warm=3):
-            m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
-            return m
+            def timed(fn, n, warm=3):
+                m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+                return m
 
-        fused_us = {r["op"]: r["us_per_call"] for r in table}
-        unfused = []
+            fused_us = {r["op"]: r["us_per_call"] for r in table}
+            unfused = []
 
-        def softmax_row(label, shape, dt, sc, mask_, keys, n):
-            mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, SoftmaxFusionTypes.none,
-                                        mask_func, True, sc)
-            x = (torch.randn(shape, device=dev, generator=gen(77)) * 8).to(dt)
+            def softmax_row(label, shape, dt, sc, mask_, keys, n):
+                mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, SoftmaxFusionTypes.none,
+                                            mask_func, True, sc)
+                x = (torch.randn(shape, device=dev, generator=gen(77)) * 8).to(dt)
+                with torch.no_grad():
+                    f_us = timed(lambda: mod(x, mask_), n)
+                xg = x.clone().requires_grad_(True)
+                g = torch.randn(shape, device=dev, generator=gen(78)).to(dt)
+
+                def fb():
+                    mod(xg, mask_).backward(g)
+                    xg.grad = None
+
+                fb_us = timed(fb, n)
+                r = {"op": label + ": unfused torch branch", "fwd_us": round(f_us, 1), "fwd_bwd_us": round(fb_us, 1)}
+                have = [fused_us.get(k) for k in keys]
+                if have[0] is not None:
+                    r["fused_fwd_us"] = have[0]
+                    r["fwd_speedup"] = round(f_us / have[0], 1)
+                    if len(have) > 1 and have[1] is not None:
+                        r["fused_fwd_bwd_us"] = round(have[0] + have[1], 2)
+                        r["fwd_bwd_speedup"] = round(fb_us / (have[0] + have[1]), 1)
+                unfused.append(r)
+
+            lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(79))
+            pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+            softmax_row("cfg2 padded [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale, pad,
+                        ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 20)
+            softmax_row("cfg4 causal [1,64,2048,2048] fp16", (1, 64, 2048, 2048), torch.float16, 96 ** -0.5, causal_mask(2048),
+                        ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 20)
+            torch.cuda.empty_cache()
+            softmax_row("cfg5 causal [1,32,8192,8192] bf16", (1, 32, 8192, 8192), torch.bfloat16, 128 ** -0.5, causal_mask(8192),
+                        ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 5)
+            torch.cuda.empty_cache()
+            # partial rotary as the attention layer does it: slice, rotate, concatenate (forward)
+            S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
+            t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1246, nsets=1)[0]
+            cos4 = t["cos"].view(S, 1, 1, DR).bfloat16()
+            sin4 = t["sin"].view(S, 1, 1, DR).bfloat16()
+
+            def layer_rotary():
+                q_rot, q_pass = t["q"][..., :DR], t["q"][..., DR:]
+                k_rot, k_pass = t["k"][..., :DR], t["k"][..., DR:]
+                q2, k2 = _rotary_torch(q_rot, k_rot, cos4, sin4, 0)
+                return torch.cat((q2, q_pass), dim=-1), torch.cat((k2, k_pass), dim=-1)
+
             with torch.no_grad():
-                f_us = timed(lambda: mod(x, mask_), n)
-            xg = x.clone().requires_grad_(True)
-            g = torch.randn(shape, device=dev, generator=gen(78)).to(dt)
-
-            def fb():
-                mod(xg, mask_).backward(g)
-                xg.grad = None
-
-            fb_us = timed(fb, n)
-            r = {"op": label + ": unfused torch branch", "fwd_us": round(f_us, 1), "fwd_bwd_us": round(fb_us, 1)}
-            have = [fused_us.get(k) for k in keys]
-            if have[0] is not None:
-                r["fused_fwd_us"] = have[0]
-                r["fwd_speedup"] = round(f_us / have[0], 1)
-                if len(have) > 1 and have[1] is not None:
-                    r["fused_fwd_bwd_us"] = round(have[0] + have[1], 2)
-                    r["fwd_bwd_speedup"] = round(fb_us / (have[0] + have[1]), 1)
+                r_us = timed(layer_rotary, 50)
+            r = {"op": "cfg3 partial rotary q+k [2048,4,32,128] bf16: slice + torch expression + cat",
+                 "fwd_us": round(r_us, 1)}
+            have = fused_us.get("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32")
+            if have is not None:
+                r["fused_fwd_us"] = have
+                r["fwd_speedup"] = round(r_us / have, 1)
             unfused.append(r)
-
-        lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(79))
-        pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
-        softmax_row("cfg2 padded [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale, pad,
-                    ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 20)
-        softmax_row("cfg4 causal [1,64,2048,2048] fp16", (1, 64, 2048, 2048), torch.float16, 96 ** -0.5, causal_mask(2048),
-                    ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 20)
-        torch.cuda.empty_cache()
-        softmax_row("cfg5 causal [1,32,8192,8192] bf16", (1, 32, 8192, 8192), torch.bfloat16, 128 ** -0.5, causal_mask(8192),
-                    ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 5)
-        torch.cuda.empty_cache()
-        # partial rotary as the attention layer does it: slice, rotate, concatenate (forward)
-        S, Bb, H, HN, DR = 2048, 4, 32, 128, 32
-        t = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1246, nsets=1)[0]
-        cos4 = t["cos"].view(S, 1, 1, DR).bfloat16()
-        sin4 = t["sin"].view(S, 1, 1, DR).bfloat16()
-
-        def layer_rotary():
-            q_rot, q_pass = t["q"][..., :DR], t["q"][..., DR:]
-            k_rot, k_pass = t["k"][..., :DR], t["k"][..., DR:]
-            q2, k2 = _rotary_torch(q_rot, k_rot, cos4, sin4, 0)
-            return torch.cat((q2, q_pass), dim=-1), torch.cat((k2, k_pass), dim=-1)
-
-        with torch.no_grad():
-            r_us = timed(layer_rotary, 50)
-        r = {"op": "cfg3 partial rotary q+k [2048,4,32,128] bf16: slice + torch expression + cat",
-             "fwd_us": round(r_us, 1)}
-        have = fused_us.get("cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32")
-        if have is not None:
-            r["fused_fwd_us"] = have
-            r["fwd_speedup"] = round(r_us / have, 1)
-        unfused.append(r)
-        del t
-        out["unfused_reference_branches_on_this_gpu"] = unfused
+            del t
+            out["unfused_reference_branches_on_this_gpu"] = unfused
     # The drop-in where it is dropped in: the Python modules the attention layer calls
     # (megatron/model/transformer.py:534 FusedScaleMaskSoftmax.forward, :850-856
     # apply_rotary_pos_emb, :844-848 fused_apply_rotary_pos_emb_cached) -- module -> autograd
@@ -870,178 +966,178 @@ def run_studies(c):
     # same work from the table, and the host's own time per call (wall clock of calls on a
     # tiny input of the same kind, where the kernel is negligible).
     if want("module"):
-        from gpt_neox_amd.fused_rope import fused_apply_rotary_pos_emb_cached
-        from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
-        from gpt_neox_amd.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_qkv_
+        with section("module"):
+            from gpt_neox_amd.fused_rope import fused_apply_rotary_pos_emb_cached
+            from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, SoftmaxFusionTypes
+            from gpt_neox_amd.positional_embeddings import apply_rotary_pos_emb, apply_rotary_pos_emb_qkv_
 
-        def mask_fill(scores, mask_):
-            return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
+            def mask_fill(scores, mask_):
+                return scores.masked_fill_(mask_, torch.finfo(scores.dtype).min)
 
-        abi_us = {r["op"]: r["us_per_call"] for r in table}
-        mrows = []
+            abi_us = {r["op"]: r["us_per_call"] for r in table}
+            mrows = []
 
-        def events_us(fn, n, warm=3):
-            m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
-            return m
+            def events_us(fn, n, warm=3):
+                m, _ = time_launches(lambda _t: fn(), [None], n, repeats=3, warm=warm)
+                return m
 
-        def host_us(fn, n=2000):
-            for _ in range(50):
-                fn()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(n):
-                fn()
-            dt = time.perf_counter() - t0
-            torch.cuda.synchronize()
-            return dt / n * 1e6
-
-        def mrow(name, f_us, fb_us, host_f, host_fb, keys):
-            r = {"op": name, "module_fwd_us": round(f_us, 2), "host_fwd_us": round(host_f, 2)}
-            if fb_us is not None:
-                r["module_fwd_bwd_us"] = round(fb_us, 2)
-                r["host_fwd_bwd_us"] = round(host_fb, 2)
-            have = [abi_us.get(k) for k in keys]
-            if have and have[0] is not None:
-                r["c_abi_fwd_us"] = have[0]
-                if len(have) > 1 and have[1] is not None:
-                    r["c_abi_fwd_bwd_us"] = round(have[0] + have[1], 2)
-            mrows.append(r)
-
-        def softmax_module_row(name, shape, dt, sc, fusion, mask_, keys, n, with_bwd=True):
-            mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, fusion, mask_fill, True, sc)
-            x = torch.empty(shape, device=dev, dtype=dt)
-            for j in range(0, shape[1], 8):  # chunked: no full-size fp32 temporary
-                x[:, j : j + 8] = (torch.randn(x[:, j : j + 8].shape, device=dev, generator=gen(81 + j)) * 8).to(dt)
-            mod(x[:1, :1], mask_[:1])  # the mask's verdict is decided before the timed calls
-            torch.cuda.synchronize()
-            with torch.no_grad():
-                f_us = events_us(lambda: mod(x, mask_), n)
-            fb_us = host_fb = None
-            tiny = x[:1, :1, :16, :16].contiguous()
-            tmask = mask_[:1, :, :16, :16].contiguous()
-            mod(tiny, tmask)
-            with torch.no_grad():
-                host_f = host_us(lambda: mod(tiny, tmask))
-            if with_bwd:
-                xg = x.requires_grad_(True)
-                g = torch.empty_like(x).normal_()
-
-                def fb():
-                    mod(xg, mask_).backward(g)
-                    xg.grad = None
-
-                fb_us = events_us(fb, n)
-                tg = tiny.clone().requires_grad_(True)
-                gg = torch.ones_like(tiny)
-
-                def tiny_fb():
-                    mod(tg, tmask).backward(gg)
-                    tg.grad = None
-
-                host_fb = host_us(tiny_fb)
-            mrow(name, f_us, fb_us, host_f, host_fb, keys)
-
-        softmax_module_row("cfg1 FusedScaleMaskSoftmax(upper_triang) [4,12,2048,2048] bf16", (4, 12, 2048, 2048),
-                           torch.bfloat16, 0.125, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
-                           ["cfg1 causal fwd [48,2048,2048] bf16"], 50, with_bwd=False)
-        lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(82))
-        pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
-        softmax_module_row("cfg2 FusedScaleMaskSoftmax(general) [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale,
-                           SoftmaxFusionTypes.general, pad,
-                           ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 50)
-        softmax_module_row("cfg4 FusedScaleMaskSoftmax(upper_triang) [1,64,2048,2048] fp16", (1, 64, 2048, 2048),
-                           torch.float16, 96 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
-                           ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 50)
-        torch.cuda.empty_cache()
-        if not args.quick:
-            softmax_module_row("cfg5 FusedScaleMaskSoftmax(upper_triang) [1,32,8192,8192] bf16", (1, 32, 8192, 8192),
-                               torch.bfloat16, 128 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(8192),
-                               ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 10)
-            torch.cuda.empty_cache()
-        # a mask the module has not seen (GPT-NeoX builds one per micro-batch): host time until the
-        # call returns and time until the GPU is done, for the default check and the two others
-        fresh_rows = {}
-        for mode in (None, "verify", "lazy", "trust"):
-            kw = {} if mode is None else {"causal_mask_check": mode}
-            mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, mask_fill, True, 0.125, **kw)
-            x = (torch.randn(1, 1, 8192, 8192, device=dev, generator=gen(83)) * 8).bfloat16()
-            big = causal_mask(8192)
-            mod(x, big)
-            torch.cuda.synchronize()
-            walls = []
-            for _ in range(5):
-                fresh = big.clone()
+            def host_us(fn, n=2000):
+                for _ in range(50):
+                    fn()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
-                mod(x, fresh)
-                t1 = time.perf_counter()
+                for _ in range(n):
+                    fn()
+                dt = time.perf_counter() - t0
                 torch.cuda.synchronize()
-                walls.append(((t1 - t0) * 1e6, (time.perf_counter() - t0) * 1e6))
-            fresh_rows["default (%s)" % mod.causal_mask_check if mode is None else mode] = {
-                "host_returns_after_us": round(statistics.median(w[0] for w in walls), 1),
-                "gpu_done_after_us": round(statistics.median(w[1] for w in walls), 1)}
-            del x, big
-        out["module_call_with_a_fresh_causal_mask_1x1x8192x8192"] = fresh_rows
+                return dt / n * 1e6
 
-        # rotary through the modules: cfg3 (partial) and cfg5 (full)
-        for label, S, Bb, H, HN, DR, keys in (
-                ("cfg3", 2048, 4, 32, 128, 32, ["cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32",
-                                                "cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32"]),
-                ("cfg5", 8192, 1, 32, 128, 128, ["cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128",
-                                                 "cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128"])):
-            sets_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1250, nsets=6)
-            cos4, sin4 = sets_[0]["cos"].view(S, 1, 1, DR), sets_[0]["sin"].view(S, 1, 1, DR)
-            it = [0]
+            def mrow(name, f_us, fb_us, host_f, host_fb, keys):
+                r = {"op": name, "module_fwd_us": round(f_us, 2), "host_fwd_us": round(host_f, 2)}
+                if fb_us is not None:
+                    r["module_fwd_bwd_us"] = round(fb_us, 2)
+                    r["host_fwd_bwd_us"] = round(host_fb, 2)
+                have = [abi_us.get(k) for k in keys]
+                if have and have[0] is not None:
+                    r["c_abi_fwd_us"] = have[0]
+                    if len(have) > 1 and have[1] is not None:
+                        r["c_abi_fwd_bwd_us"] = round(have[0] + have[1], 2)
+                mrows.append(r)
 
-            def nxt():
-                it[0] += 1
-                return sets_[it[0] % 6]
+            def softmax_module_row(name, shape, dt, sc, fusion, mask_, keys, n, with_bwd=True):
+                mod = FusedScaleMaskSoftmax(dt == torch.float16, dt == torch.bfloat16, fusion, mask_fill, True, sc)
+                x = torch.empty(shape, device=dev, dtype=dt)
+                for j in range(0, shape[1], 8):  # chunked: no full-size fp32 temporary
+                    x[:, j : j + 8] = (torch.randn(x[:, j : j + 8].shape, device=dev, generator=gen(81 + j)) * 8).to(dt)
+                mod(x[:1, :1], mask_[:1])  # the mask's verdict is decided before the timed calls
+                torch.cuda.synchronize()
+                with torch.no_grad():
+                    f_us = events_us(lambda: mod(x, mask_), n)
+                fb_us = host_fb = None
+                tiny = x[:1, :1, :16, :16].contiguous()
+                tmask = mask_[:1, :, :16, :16].contiguous()
+                mod(tiny, tmask)
+                with torch.no_grad():
+                    host_f = host_us(lambda: mod(tiny, tmask))
+                if with_bwd:
+                    xg = x.requires_grad_(True)
+                    g = torch.empty_like(x).normal_()
 
-            def sliced():  # what the attention layer does: slice, rotate (new tensors), caller concatenates
-                t = nxt()
-                return apply_rotary_pos_emb(t["q"][..., :DR], t["k"][..., :DR], cos4, sin4)
+                    def fb():
+                        # (autograd.grad: inside a model the scores are no leaf either; .backward() into a
+                        # leaf would add AccumulateGrad's copy of the gradient, 0.1 ms at these sizes)
+                        torch.autograd.grad(mod(xg, mask_), xg, g)
 
-            def fused_rope_path():  # rope_fusion: one call per tensor, pass-through dims copied in the kernel
-                t = nxt()
-                return fused_apply_rotary_pos_emb_cached(t["q"], cos4, sin4), fused_apply_rotary_pos_emb_cached(t["k"], cos4, sin4)
+                    fb_us = events_us(fb, n)
+                    tg = tiny.clone().requires_grad_(True)
+                    gg = torch.ones_like(tiny)
 
-            tq = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
-            tk = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
-            tc, ts_ = cos4[:4].contiguous(), sin4[:4].contiguous()
-            with torch.no_grad():
-                f_us = events_us(sliced, 200)
-                hf = host_us(lambda: apply_rotary_pos_emb(tq[..., :DR], tk[..., :DR], tc, ts_))
-                mrow(f"{label} apply_rotary_pos_emb(q[..., :{DR}], k[..., :{DR}], cos, sin) [{S},{Bb},{H},{HN}] bf16",
-                     f_us, None, hf, None, keys[:1])
-                f_us = events_us(fused_rope_path, 200)
-                hf = host_us(lambda: fused_apply_rotary_pos_emb_cached(tq, tc, ts_))
-                mrow(f"{label} fused_apply_rotary_pos_emb_cached(q) + (k): whole heads out of place "
-                     f"[{S},{Bb},{H},{HN}] bf16 d2={DR}; host figure per call", f_us, None, hf, None, [])
-            # in place on the fused QKV projection [s, b, np, 3*hn]: q and k thirds rotated, no copies
-            mixed = [torch.randn(S, Bb, H, 3 * HN, device=dev, generator=gen(1251 + i)).bfloat16() for i in range(4)]
-            tmixed = torch.randn(4, 1, 2, 3 * HN, device=dev).bfloat16()
-            with torch.no_grad():
-                def qkv_in_place():
+                    def tiny_fb():
+                        torch.autograd.grad(mod(tg, tmask), tg, gg)
+
+                    host_fb = host_us(tiny_fb)
+                mrow(name, f_us, fb_us, host_f, host_fb, keys)
+
+            softmax_module_row("cfg1 FusedScaleMaskSoftmax(upper_triang) [4,12,2048,2048] bf16", (4, 12, 2048, 2048),
+                               torch.bfloat16, 0.125, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                               ["cfg1 causal fwd [48,2048,2048] bf16"], 50, with_bwd=False)
+            lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(82))
+            pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+            softmax_module_row("cfg2 FusedScaleMaskSoftmax(general) [8,16,1024,1024] fp16", (b, heads, sq, sk), dtype, scale,
+                               SoftmaxFusionTypes.general, pad,
+                               ["cfg2 padded fwd [8,16,1024,1024] fp16", "cfg2 padded bwd [8,16,1024,1024] fp16"], 50)
+            softmax_module_row("cfg4 FusedScaleMaskSoftmax(upper_triang) [1,64,2048,2048] fp16", (1, 64, 2048, 2048),
+                               torch.float16, 96 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(2048),
+                               ["cfg4 causal fwd [64,2048,2048] fp16", "cfg4 causal bwd [64,2048,2048] fp16"], 50)
+            torch.cuda.empty_cache()
+            if not args.quick:
+                softmax_module_row("cfg5 FusedScaleMaskSoftmax(upper_triang) [1,32,8192,8192] bf16", (1, 32, 8192, 8192),
+                                   torch.bfloat16, 128 ** -0.5, SoftmaxFusionTypes.upper_triang, causal_mask(8192),
+                                   ["cfg5 causal fwd [32,8192,8192] bf16", "cfg5 causal bwd [32,8192,8192] bf16"], 10)
+                torch.cuda.empty_cache()
+            # a mask the module has not seen (GPT-NeoX builds one per micro-batch): host time until the
+            # call returns and time until the GPU is done, for the default check and the two others
+            fresh_rows = {}
+            for mode in (None, "verify", "lazy", "trust"):
+                kw = {} if mode is None else {"causal_mask_check": mode}
+                mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.upper_triang, mask_fill, True, 0.125, **kw)
+                x = (torch.randn(1, 1, 8192, 8192, device=dev, generator=gen(83)) * 8).bfloat16()
+                big = causal_mask(8192)
+                mod(x, big)
+                torch.cuda.synchronize()
+                walls = []
+                for _ in range(5):
+                    fresh = big.clone()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    mod(x, fresh)
+                    t1 = time.perf_counter()
+                    torch.cuda.synchronize()
+                    walls.append(((t1 - t0) * 1e6, (time.perf_counter() - t0) * 1e6))
+                fresh_rows["default (%s)" % mod.causal_mask_check if mode is None else mode] = {
+                    "host_returns_after_us": round(statistics.median(w[0] for w in walls), 1),
+                    "gpu_done_after_us": round(statistics.median(w[1] for w in walls), 1)}
+                del x, big
+            out["module_call_with_a_fresh_causal_mask_1x1x8192x8192"] = fresh_rows
+
+            # rotary through the modules: cfg3 (partial) and cfg5 (full)
+            for label, S, Bb, H, HN, DR, keys in (
+                    ("cfg3", 2048, 4, 32, 128, 32, ["cfg3 rotary fwd q+k [2048,4,32,128] bf16 d_rot=32",
+                                                    "cfg3 rotary bwd q+k [2048,4,32,128] bf16 d_rot=32"]),
+                    ("cfg5", 8192, 1, 32, 128, 128, ["cfg5 rotary fwd q+k [8192,1,32,128] bf16 d_rot=128",
+                                                     "cfg5 rotary bwd q+k [8192,1,32,128] bf16 d_rot=128"])):
+                sets_ = rope_sets(S, Bb, H, HN, DR, torch.bfloat16, 1250, nsets=6)
+                cos4, sin4 = sets_[0]["cos"].view(S, 1, 1, DR), sets_[0]["sin"].view(S, 1, 1, DR)
+                it = [0]
+
+                def nxt():
                     it[0] += 1
-                    return apply_rotary_pos_emb_qkv_(mixed[it[0] % 4], cos4, sin4, 0, DR)
+                    return sets_[it[0] % 6]
 
-                f_us = events_us(qkv_in_place, 200)
-                hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
-            mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
-            del sets_, mixed
-        # for scale: what the host spends on torch's own smallest differentiable step
-        tx = torch.randn(16, 16, device=dev, dtype=torch.float16, requires_grad=True)
-        tgg = torch.ones_like(tx)
+                def sliced():  # what the attention layer does: slice, rotate (new tensors), caller concatenates
+                    t = nxt()
+                    return apply_rotary_pos_emb(t["q"][..., :DR], t["k"][..., :DR], cos4, sin4)
 
-        def torch_floor():
-            (tx * 2.0).backward(tgg)
-            tx.grad = None
+                def fused_rope_path():  # rope_fusion: one call per tensor, pass-through dims copied in the kernel
+                    t = nxt()
+                    return fused_apply_rotary_pos_emb_cached(t["q"], cos4, sin4), fused_apply_rotary_pos_emb_cached(t["k"], cos4, sin4)
 
-        with torch.no_grad():
-            floor_f = host_us(lambda: tx * 2.0)
-        mrows.append({"op": "torch's own floor on this host: y = x * 2 (forward), then y.backward(g)",
-                      "host_fwd_us": round(floor_f, 2), "host_fwd_bwd_us": round(host_us(torch_floor), 2)})
-        out["module_api"] = mrows
+                tq = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+                tk = torch.randn(4, 1, 2, HN, device=dev).bfloat16()
+                tc, ts_ = cos4[:4].contiguous(), sin4[:4].contiguous()
+                with torch.no_grad():
+                    f_us = events_us(sliced, 200)
+                    hf = host_us(lambda: apply_rotary_pos_emb(tq[..., :DR], tk[..., :DR], tc, ts_))
+                    mrow(f"{label} apply_rotary_pos_emb(q[..., :{DR}], k[..., :{DR}], cos, sin) [{S},{Bb},{H},{HN}] bf16",
+                         f_us, None, hf, None, keys[:1])
+                    f_us = events_us(fused_rope_path, 200)
+                    hf = host_us(lambda: fused_apply_rotary_pos_emb_cached(tq, tc, ts_))
+                    mrow(f"{label} fused_apply_rotary_pos_emb_cached(q) + (k): whole heads out of place "
+                         f"[{S},{Bb},{H},{HN}] bf16 d2={DR}; host figure per call", f_us, None, hf, None, [])
+                # in place on the fused QKV projection [s, b, np, 3*hn]: q and k thirds rotated, no copies
+                mixed = [torch.randn(S, Bb, H, 3 * HN, device=dev, generator=gen(1251 + i)).bfloat16() for i in range(4)]
+                tmixed = torch.randn(4, 1, 2, 3 * HN, device=dev).bfloat16()
+                with torch.no_grad():
+                    def qkv_in_place():
+                        it[0] += 1
+                        return apply_rotary_pos_emb_qkv_(mixed[it[0] % 4], cos4, sin4, 0, DR)
+
+                    f_us = events_us(qkv_in_place, 200)
+                    hf = host_us(lambda: apply_rotary_pos_emb_qkv_(tmixed, tc, ts_, 0, DR))
+                mrow(f"{label} apply_rotary_pos_emb_qkv_(mixed [{S},{Bb},{H},{3 * HN}]) in place, d_rot={DR}", f_us, None, hf, None, keys[:1])
+                del sets_, mixed
+            # for scale: what the host spends on torch's own smallest differentiable step
+            tx = torch.randn(16, 16, device=dev, dtype=torch.float16, requires_grad=True)
+            tgg = torch.ones_like(tx)
+
+            def torch_floor():
+                torch.autograd.grad(tx * 2.0, tx, tgg)
+
+            with torch.no_grad():
+                floor_f = host_us(lambda: tx * 2.0)
+            mrows.append({"op": "torch's own floor on this host: y = x * 2 (forward), then autograd.grad(y, x, g)",
+                          "host_fwd_us": round(floor_f, 2), "host_fwd_bwd_us": round(host_us(torch_floor), 2)})
+            out["module_api"] = mrows
     return out
 
 

@@ -14,7 +14,7 @@ import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(_CSRC, "libneox_fused.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 NEOX_F16, NEOX_BF16, NEOX_F32 = 0, 1, 2
 _DTYPE_CODE = {torch.float16: NEOX_F16, torch.bfloat16: NEOX_BF16, torch.float32: NEOX_F32}
@@ -38,13 +38,19 @@ SIGNATURES = {
         [_vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
     "neox_masked_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _vp]),
+    "neox_masked_softmax_alibi_fwd": (
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
+    ),
     "neox_causal_softmax_bias_fwd": (
-        ctypes.c_int, [_vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
+        ctypes.c_int, [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     ),
     "neox_masked_softmax_bias_fwd": (
         ctypes.c_int,
-        [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+        [_vp, _vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
     ),
+    "neox_sliding_window_softmax_fwd": (ctypes.c_int, [_vp, _vp, _f32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "neox_sliding_window_softmax_bwd": (ctypes.c_int, [_vp, _vp, _vp, _f32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "neox_mask_classify": (ctypes.c_int, [_vp, _vp, _i32, _i32, _i32, _vp]),
     "neox_causal_softmax_dropout_fwd": (
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _vp],
@@ -54,7 +60,7 @@ SIGNATURES = {
     ),
     "neox_masked_softmax_dropout_fwd": (
         ctypes.c_int,
-        [_vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
          _vp],
     ),
     "neox_masked_softmax_dropout_bwd": (
@@ -81,7 +87,7 @@ _lib = None
 def build(verbose=False, targets=("all",)):
     """Compile ``libneox_fused.so`` for gfx950 with hipcc (works without a GPU).  ``targets``:
     make targets; ``"probes"`` is the benchmark's copy kernel, a library of its own."""
-    cmd = ["make", "-C", _CSRC, "-j4", "-B", *targets]
+    cmd = ["make", "-C", _CSRC, "-j8", "-B", *targets]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         print(res.stdout)

@@ -68,12 +68,11 @@ static int make_dropout(DropoutArgs& d, float p, uint64_t seed, uint64_t offset,
 // `status`; nothing here touches the GPU.  The 16-bit tensors given to the constructor
 // also decide whether 128-bit accesses are legal (`vec_ok`).
 struct SoftmaxCall {
-    typedef hipError_t (*Launcher)(const SoftmaxArgs&, Mask, int, bool, hipStream_t);
-
     const char* what;
     int dtype;
     int status = NEOX_OK;
     bool vec_ok = true;
+    int features = 0;  // kAlibi | kBias | kDropout, by what the call brings along
     SoftmaxArgs a{};
 
     SoftmaxCall(const char* name, int dtype_code, std::initializer_list<const void*> tensors,
@@ -141,6 +140,7 @@ struct SoftmaxCall {
         a.bias = t;
         a.bias_rows = (bias_b == 1 && b != 1) ? (uint32_t)((int64_t)np * a.sq) : 0u;
         a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
+        features |= kBias;
     }
     // ALiBi slopes, fp32 [np]
     void alibi(const float* slopes, int np) {
@@ -151,9 +151,11 @@ struct SoftmaxCall {
         }
         a.slopes = slopes;
         a.np = (uint32_t)np;
+        features |= kAlibi;
     }
     void dropout(float p, uint64_t seed, uint64_t offset, const uint64_t* device_state) {
         if (!status) status = make_dropout(a.drop, p, seed, offset, device_state, what);
+        features |= kDropout;
     }
     void second_output(void* y_drop, const void* y) {
         if (status) return;
@@ -172,12 +174,15 @@ struct SoftmaxCall {
         a.in1 = y;
         a.scale = scale;
     }
-    // `ragged`, if given, serves rows that rule out aligned 128-bit accesses; without it (or
-    // outside its range of row lengths) those go to `fn`'s element-wise kernels.
-    int launch(Launcher fn, Mask m, void* stream, Launcher ragged = nullptr) const {
+    // The translation unit of the call's feature set; rows that rule out aligned 128-bit accesses
+    // go to its kRagged twin, and outside that twin's range of row lengths to the element-wise kernels.
+    int launch(bool backward, Mask m, void* stream) const {
         const bool vec = vec_ok && a.sk % kVec == 0;
-        if (!vec && ragged != nullptr && a.sk >= kVec && a.sk < kMaxRegisterRow) fn = ragged;
-        return check_launch(fn(a, m, dtype, vec, (hipStream_t)stream), what);
+        int flags = backward ? (features & kDropout) : features;
+        if (!vec && a.sk >= kVec && a.sk < kMaxRegisterRow) flags |= kRagged;
+        const hipError_t e = backward ? launch_softmax_bwd(flags, a, m, dtype, vec, (hipStream_t)stream)
+                                      : launch_softmax_fwd(flags, a, m, dtype, vec, (hipStream_t)stream);
+        return check_launch(e, what);
     }
 
   private:
@@ -204,6 +209,26 @@ __global__ __launch_bounds__(256) void keep_mask_kernel(uint8_t* keep, DropoutAr
     const uint32_t bits = keep_bits8(resolve(d), group);
     for (int k = 0; k < 8; ++k)
         if (group * 8 + k < n) keep[group * 8 + k] = (bits >> k) & 1u;
+}
+
+hipError_t launch_softmax_fwd(int flags, const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok, hipStream_t stream) {
+    switch (flags) {
+#define NEOX_CASE(F) \
+    case F: return launch_softmax_fwd_flags<F>(a, mask, dtype, vec_ok, stream);
+        NEOX_FWD_FEATURE_SETS(NEOX_CASE)
+#undef NEOX_CASE
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_softmax_bwd(int flags, const SoftmaxArgs& a, Mask mask, int dtype, bool vec_ok, hipStream_t stream) {
+    switch (flags) {
+#define NEOX_CASE(F) \
+    case F: return launch_softmax_bwd_flags<F>(a, mask, dtype, vec_ok, stream);
+        NEOX_BWD_FEATURE_SETS(NEOX_CASE)
+#undef NEOX_CASE
+    }
+    return hipErrorInvalidValue;
 }
 
 }  // namespace neox
@@ -236,7 +261,7 @@ int neox_causal_softmax_fwd(void* y, const void* x, float scale, int64_t batches
     c.causal_rows(batches, sq, sk);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
+    return c.launch(false, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, float scale, int32_t b,
@@ -246,7 +271,7 @@ int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, f
     c.alibi(slopes, np);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
+    return c.launch(false, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
@@ -255,7 +280,7 @@ int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     c.causal_rows(batches, sq, sk);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_bwd, Mask::Causal, stream, launch_softmax_ragged_bwd);
+    return c.launch(true, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
@@ -266,7 +291,7 @@ int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float s
     c.mask(mask, b, np, mask_b);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_fwd, Mask::Bytes, stream, launch_softmax_ragged_fwd);
+    return c.launch(false, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t rows,
@@ -275,31 +300,46 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     c.plain_rows(rows, sk);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_bwd, Mask::None, stream, launch_softmax_ragged_bwd);
+    return c.launch(true, Mask::None, stream);
 }
 
-int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
-                                 int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
-                                 void* stream) {
+int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, const float* alibi_slopes,
+                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t bias_b,
+                                 int32_t dtype, void* stream) {
     SoftmaxCall c("neox_causal_softmax_bias_fwd", dtype, {y, x}, bias);
     c.head_rows(b, np, sq, sk);
     c.bias(bias, b, np, bias_b);
+    if (alibi_slopes) c.alibi(alibi_slopes, np);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_bias_fwd, Mask::Causal, stream, launch_softmax_ragged_fwd);
+    return c.launch(false, Mask::Causal, stream);
+}
+
+int neox_masked_softmax_alibi_fwd(void* y, const void* x, const uint8_t* mask, const float* slopes, float scale,
+                                  int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b, int32_t dtype,
+                                  void* stream) {
+    if (!slopes) return fail(NEOX_ERR_NULL_POINTER, "neox_masked_softmax_alibi_fwd: null tensor pointer");
+    SoftmaxCall c("neox_masked_softmax_alibi_fwd", dtype, {y, x}, mask);
+    c.head_rows(b, np, sq, sk);
+    c.mask(mask, b, np, mask_b);
+    c.alibi(slopes, np);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(false, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
-                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
-                                 int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream) {
+                                 const float* alibi_slopes, float scale, int32_t b, int32_t np, int32_t sq,
+                                 int32_t sk, int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream) {
     if (!bias) return fail(NEOX_ERR_NULL_POINTER, "neox_masked_softmax_bias_fwd: null tensor pointer");
     SoftmaxCall c("neox_masked_softmax_bias_fwd", dtype, {y, x}, mask);
     c.head_rows(b, np, sq, sk);
     c.mask(mask, b, np, mask_b);
     c.bias(bias, b, np, bias_b);
+    if (alibi_slopes) c.alibi(alibi_slopes, np);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_bias_fwd, Mask::Bytes, stream, launch_softmax_ragged_fwd);
+    return c.launch(false, Mask::Bytes, stream);
 }
 
 int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const float* alibi_slopes,
@@ -307,10 +347,7 @@ int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const 
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
                                     int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t dtype,
                                     void* stream) {
-    static const char* what = "neox_causal_softmax_dropout_fwd";
-    if (alibi_slopes && bias)
-        return fail(NEOX_ERR_BAD_SHAPE, "%s: give ALiBi slopes or a bias tensor, not both", what);
-    SoftmaxCall c(what, dtype, {y_drop, y, x});
+    SoftmaxCall c("neox_causal_softmax_dropout_fwd", dtype, {y_drop, y, x});
     c.second_output(y_drop, y);
     c.head_rows(b, np, sq, sk);
     if (alibi_slopes) c.alibi(alibi_slopes, np);
@@ -318,7 +355,7 @@ int neox_causal_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const 
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_dropout_fwd, Mask::Causal, stream, launch_softmax_ragged_dropout_fwd);
+    return c.launch(false, Mask::Causal, stream);
 }
 
 int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
@@ -330,11 +367,11 @@ int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_dropout_bwd, Mask::Causal, stream, launch_softmax_ragged_dropout_bwd);
+    return c.launch(true, Mask::Causal, stream);
 }
 
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    const void* bias, int32_t bias_b, float scale, float p,
+                                    const float* alibi_slopes, const void* bias, int32_t bias_b, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
                                     int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream) {
@@ -342,11 +379,12 @@ int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const 
     c.second_output(y_drop, y);
     c.head_rows(b, np, sq, sk);
     c.mask(mask, b, np, mask_b);
+    if (alibi_slopes) c.alibi(alibi_slopes, np);
     if (bias) c.bias(bias, b, np, bias_b);
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.forward(y, x, scale);
-    return c.launch(launch_softmax_dropout_fwd, Mask::Bytes, stream, launch_softmax_ragged_dropout_fwd);
+    return c.launch(false, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, float scale, float p,
@@ -358,7 +396,7 @@ int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
     c.dropout(p, seed, offset, device_state);
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
-    return c.launch(launch_softmax_dropout_bwd, Mask::None, stream, launch_softmax_ragged_dropout_bwd);
+    return c.launch(true, Mask::None, stream);
 }
 
 int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset,
@@ -372,6 +410,49 @@ int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offse
     hipLaunchKernelGGL(keep_mask_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, keep, d, (uint64_t)n);
     return check_launch(hipGetLastError(), what);
+}
+
+// aligned rows of 513 .. kMaxRegisterRow columns: what the sliding-window kernels take
+static int check_window_call(const SoftmaxCall& c, int32_t sq, int32_t sk, int32_t window) {
+    if (sq != sk) return fail(NEOX_ERR_BAD_SHAPE, "%s: sq=%d and sk=%d must be equal", c.what, sq, sk);
+    if (window < 0) return fail(NEOX_ERR_BAD_SHAPE, "%s: window=%d is negative", c.what, window);
+    if (sk <= kChunk || sk > kMaxRegisterRow || sk % kVec != 0)
+        return fail(NEOX_ERR_BAD_SHAPE, "%s: sk=%d must be a multiple of %d in (%d, %d]", c.what, sk, kVec, kChunk,
+                    kMaxRegisterRow);
+    if (!c.vec_ok) return fail(NEOX_ERR_MISALIGNED, "%s: the tensors must be 16-byte aligned", c.what);
+    return NEOX_OK;
+}
+
+int neox_sliding_window_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int32_t sq, int32_t sk,
+                                    int32_t window, int32_t dtype, void* stream) {
+    SoftmaxCall c("neox_sliding_window_softmax_fwd", dtype, {y, x});
+    c.causal_rows(batches, sq, sk);
+    if (c.status) return c.status;
+    if (int e = check_window_call(c, sq, sk, window)) return e;
+    c.forward(y, x, scale);
+    c.a.window = window;
+    return check_launch(launch_softmax_band_fwd(c.a, dtype, true, (hipStream_t)stream), c.what);
+}
+
+int neox_sliding_window_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
+                                    int32_t sq, int32_t sk, int32_t window, int32_t dtype, void* stream) {
+    SoftmaxCall c("neox_sliding_window_softmax_bwd", dtype, {dx, dy, y});
+    c.causal_rows(batches, sq, sk);
+    if (c.status) return c.status;
+    if (int e = check_window_call(c, sq, sk, window)) return e;
+    c.backward(dx, dy, y, scale);
+    c.a.window = window;
+    return check_launch(launch_softmax_band_bwd(c.a, dtype, true, (hipStream_t)stream), c.what);
+}
+
+int neox_mask_classify(int32_t* record, const uint8_t* mask, int32_t mask_b, int32_t sq, int32_t sk, void* stream) {
+    static const char* what = "neox_mask_classify";
+    if (!record || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
+    if (mask_b < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: mask_b=%d must be >= 1", what, mask_b);
+    if (int e = check_rows((int64_t)mask_b * (sq < 1 ? 0 : sq), sq, sk, what)) return e;
+    if (sq != sk) return fail(NEOX_ERR_BAD_SHAPE, "%s: sq=%d and sk=%d must be equal", what, sq, sk);
+    if (!aligned(record, 4)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+    return check_launch(launch_mask_classify(record, mask, (uint32_t)mask_b * (uint32_t)sq, sq, sk, (hipStream_t)stream), what);
 }
 
 int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np) {
@@ -427,6 +508,19 @@ static int rope_apply(const char* what, void* out_q, void* out_k, const void* q,
     if (has_k) {
         if (int e = check_rope_strides(k_strides, what, "k")) return e;
         if (int e = check_rope_strides(out_k_strides, what, "out_k")) return e;
+    }
+    // the d leading dims of a head must not reach into the next head: the pass-through copy and the
+    // padded write-back both move whole heads' worth of dims
+    auto heads_apart = [&](const int64_t* st, int h, const char* name) {
+        if (h > 1 && st[2] < d)
+            return fail(NEOX_ERR_BAD_STRIDE, "%s: %s head stride %lld is smaller than d=%d", what, name, (long long)st[2], d);
+        return (int)NEOX_OK;
+    };
+    if (int e = heads_apart(q_strides, h_q, "q")) return e;
+    if (int e = heads_apart(out_q_strides, h_q, "out_q")) return e;
+    if (has_k) {
+        if (int e = heads_apart(k_strides, h_k, "k")) return e;
+        if (int e = heads_apart(out_k_strides, h_k, "out_k")) return e;
     }
     const int cs_size = (angles || cs_dtype == NEOX_F32) ? 4 : 2;
     if (!aligned(q, 2) || !aligned(out_q, 2) || (has_k && (!aligned(k, 2) || !aligned(out_k, 2))) ||

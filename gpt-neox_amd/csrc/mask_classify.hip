@@ -1,0 +1,89 @@
+// Recognises causal attention masks on the device, so that a caller holding only the mask tensor can
+// choose the kernel that never reads it.  The masks in question are the ones
+// megatron/utils.py:67-80 (get_attn_mask) builds: row i hides every key j > i and, with a sliding
+// window of width w, every key j < i - w as well.
+//
+// One wave per mask row finds the number of visible keys, the first and the last one.  The row fits
+// the pattern if the visible keys are the contiguous run [lo, i]; the rows then have to agree on one
+// w with lo = max(0, i - w): a row with lo > 0 fixes w = i - lo, a row with lo = 0 only says w >= i.
+// The wave's first lane folds its row into the four-word record the host reads afterwards.
+#include <limits.h>
+
+#include "internal.hpp"
+
+namespace neox {
+
+// record[0]: 1 if some row does not fit the pattern; [1], [2]: smallest and largest i - lo over the rows
+// with lo > 0 (INT_MAX and -1 without such a row); [3]: largest i over the rows with lo = 0 (-1 if none).
+__global__ void mask_classify_init_kernel(int32_t* record) {
+    if (threadIdx.x == 0) {
+        record[0] = 0;
+        record[1] = INT_MAX;
+        record[2] = -1;
+        record[3] = -1;
+    }
+}
+
+template <bool WIDE>
+__global__ __launch_bounds__(256) void mask_classify_kernel(int32_t* record, const uint8_t* mask, uint32_t rows,
+                                                            int sq, int sk) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= rows) return;  // wave-uniform
+    const int i = (int)(row % (uint32_t)sq);
+    const uint8_t* m = mask + (size_t)row * sk;
+    int count = 0, first = INT_MAX, last = -1;
+    if constexpr (WIDE) {  // sk % 8 == 0 and the tensor 8-byte aligned
+        for (int c = lane * 8; c < sk; c += kWave * 8) {
+            const uint64_t v = *reinterpret_cast<const uint64_t*>(m + c);
+            if (v == 0) {
+                count += 8;
+                first = min(first, c);
+                last = c + 7;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (((v >> (8 * k)) & 0xffu) == 0) {
+                        ++count;
+                        first = min(first, c + k);
+                        last = c + k;
+                    }
+                }
+            }
+        }
+    } else {
+        for (int c = lane; c < sk; c += kWave) {
+            if (m[c] == 0) {
+                ++count;
+                first = min(first, c);
+                last = c;
+            }
+        }
+    }
+#pragma unroll
+    for (int step = 1; step < kWave; step <<= 1) {
+        count += __shfl_xor(count, step);
+        first = min(first, __shfl_xor(first, step));
+        last = max(last, __shfl_xor(last, step));
+    }
+    if (lane != 0) return;
+    if (count == 0 || last != i || count != last - first + 1) {
+        atomicOr(record, 1);
+    } else if (first > 0) {
+        atomicMin(record + 1, i - first);
+        atomicMax(record + 2, i - first);
+    } else {
+        atomicMax(record + 3, i);
+    }
+}
+
+hipError_t launch_mask_classify(int32_t* record, const uint8_t* mask, uint32_t rows, int sq, int sk, hipStream_t st) {
+    hipLaunchKernelGGL(mask_classify_init_kernel, dim3(1), dim3(64), 0, st, record);
+    const dim3 grid((rows + 3) / 4), block(256);
+    const bool wide = sk % 8 == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
+    if (wide) hipLaunchKernelGGL((mask_classify_kernel<true>), grid, block, 0, st, record, mask, rows, sq, sk);
+    else hipLaunchKernelGGL((mask_classify_kernel<false>), grid, block, 0, st, record, mask, rows, sq, sk);
+    return hipGetLastError();
+}
+
+}  // namespace neox

@@ -22,6 +22,7 @@
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
 //   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768)
 //                  the same packed and one- to sixteen-wave row kernels with the kRagged flag
+//   sliding window (kBand) the one- to sixteen-wave row kernels, aligned rows of 513-32768 columns
 //   anything else  element-wise kernels (ragged rows outside that range, rows beyond 81408
 //                  columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
 #pragma once
@@ -33,21 +34,10 @@
 
 namespace neox {
 
-// Forward features selected at run time on top of a translation unit's EXTRA flags: the
-// ALiBi slopes (causal kernels) and, in the dropout and ragged units, a bias tensor.  `launch`
-// is called with the resulting flag set as a compile-time constant.
-template <Mask M, bool BWD, int EXTRA, typename Launch>
-static hipError_t with_runtime_flags(const SoftmaxArgs& a, Launch&& launch) {
-    if constexpr (!BWD && (EXTRA & kBias) == 0) {
-        if constexpr (M == Mask::Causal) {
-            if (a.slopes != nullptr) return launch(std::integral_constant<int, EXTRA | kAlibi>{});
-        }
-        if constexpr ((EXTRA & (kDropout | kRagged)) != 0) {
-            if (a.bias != nullptr) return launch(std::integral_constant<int, EXTRA | kBias>{});
-        }
-    }
-    return launch(std::integral_constant<int, EXTRA>{});
-}
+// EXTRA is the feature set of a translation unit -- any combination of kAlibi, kBias, kDropout and
+// kRagged for the forward pass, of kDropout and kRagged for the backward pass, or kBand alone -- and
+// every kernel of the unit is compiled for exactly that set: the caller picks the unit by what the
+// call brings along (slopes, a bias tensor, a dropout probability, unaligned rows).
 
 // Switches the XCD-aware block -> unit mapping on (see xcd_slot) when the work units of a block
 // -- `units` of them, `unit_bytes` each, consecutive in memory -- tile 4 KiB pieces exactly and
@@ -73,15 +63,13 @@ static hipError_t launch_shape(const SoftmaxArgs& a0, hipStream_t st) {
     const dim3 grid((a0.rows + RPB - 1) / RPB);
     const dim3 block(kWave * WPR * RPB);
     const SoftmaxArgs a = with_xcd_mapping(a0, (uint64_t)a0.sk * 2, RPB, grid.x);
-    return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
-        constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
-        if constexpr (BWD) {
-            hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
-        } else {
-            hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
-        }
-        return hipGetLastError();
-    });
+    constexpr int FLAGS = kDefaultFlags | EXTRA;
+    if constexpr (BWD) {
+        hipLaunchKernelGGL((softmax_bwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
+    } else {
+        hipLaunchKernelGGL((softmax_fwd_kernel<T, NCH, WPR, RPB, M, FLAGS>), grid, block, 0, st, a);
+    }
+    return hipGetLastError();
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA>
@@ -104,15 +92,13 @@ static hipError_t launch_packed_shape(const SoftmaxArgs& a0, hipStream_t st) {
     // several chunks per lane group: two loads per store, and the order measured 0-2 % slower there.
     const uint64_t unit_bytes = (BWD && C > 1) ? 0 : (uint64_t)Packed<G, R>::kRowsPerWave * a0.sk * 2;
     const SoftmaxArgs a = with_xcd_mapping(a0, unit_bytes, 4, grid.x);
-    return with_runtime_flags<M, BWD, EXTRA>(a, [&](auto extra) {
-        constexpr int FLAGS = kDefaultFlags | decltype(extra)::value;
-        if constexpr (BWD) {
-            hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
-        } else {
-            hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
-        }
-        return hipGetLastError();
-    });
+    constexpr int FLAGS = kDefaultFlags | EXTRA;
+    if constexpr (BWD) {
+        hipLaunchKernelGGL((softmax_bwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((softmax_fwd_packed_kernel<T, G, M, FLAGS, R, C>), grid, dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
 }
 
 template <typename T, Mask M, bool BWD, int EXTRA, int G>
@@ -147,14 +133,10 @@ static hipError_t dispatch_packed(const SoftmaxArgs& a, hipStream_t st) {
 // kernel, which forms a 64-bit address per row.  (The backward pass reads neither.)
 template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_short_rows(const SoftmaxArgs& a, hipStream_t st) {
-    constexpr bool side_tensor = !BWD && (M == Mask::Bytes || (EXTRA & (kBias | kDropout | kRagged)) != 0);
+    constexpr bool side_tensor = !BWD && (M == Mask::Bytes || (EXTRA & kBias) != 0);
     if constexpr (side_tensor) {
         const bool fits32 = (M != Mask::Bytes || a.mask_bytes != 0) && (a.bias == nullptr || a.bias_bytes != 0);
-        if (!fits32) {
-            // only a bias tensor brings a causal call here
-            constexpr int WITH = (M == Mask::Causal) ? (EXTRA | kBias) : EXTRA;
-            return launch_shape<T, M, BWD, WITH, 1, 1, 4>(a, st);
-        }
+        if (!fits32) return launch_shape<T, M, BWD, EXTRA, 1, 1, 4>(a, st);
     }
     return dispatch_packed<T, M, BWD, EXTRA>(a, st);
 }
@@ -168,7 +150,7 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
         // beyond the register budget: the row is staged in LDS (plain kernels only), in half
         // of a CU's LDS when it fits there
         if constexpr (EXTRA == 0) {
-            if (a.sk <= kMaxLdsRow && a.slopes == nullptr) {
+            if (a.sk <= kMaxLdsRow) {
                 const bool half = a.sk <= kMaxLdsHalfRow;
                 const dim3 grid(a.rows), block(kLdsThreads);
                 if constexpr (BWD) {
@@ -216,7 +198,10 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
 template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     int chunks = (a.sk + kChunk - 1) / kChunk;
-    if constexpr ((EXTRA & kRagged) != 0) {
+    if constexpr ((EXTRA & kBand) != 0) {
+        // sliding-window rows: the row kernels below only (aligned rows of two chunks or more)
+        if (!vec_ok || chunks < 2 || a.sk > kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+    } else if constexpr ((EXTRA & kRagged) != 0) {
         // rows at any alignment: the packed kernels up to 512 columns, the row kernels below beyond
         if (a.sk < kVec || a.sk >= kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
         if (chunks > 1) {
@@ -261,6 +246,13 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
     if (chunks <= 32) return launch_shape<T, M, BWD, EXTRA, 2, 16, 1>(a, st);
     if (chunks <= 48) return launch_shape<T, M, BWD, EXTRA, 3, 16, 1>(a, st);
     return launch_shape<T, M, BWD, EXTRA, 4, 16, 1>(a, st);
+}
+
+// Sliding-window causal softmax (EXTRA = kBand): causal rows only.
+template <bool BWD>
+static hipError_t dispatch_band(const SoftmaxArgs& a, int dtype, bool vec_ok, hipStream_t st) {
+    return dtype == NEOX_F16 ? dispatch_rows<F16, Mask::Causal, BWD, kBand>(a, vec_ok, st)
+                             : dispatch_rows<BF16, Mask::Causal, BWD, kBand>(a, vec_ok, st);
 }
 
 template <bool BWD, int EXTRA = 0>

@@ -47,6 +47,7 @@ struct SoftmaxArgs {
     // by the launchers: work units (rows, or the rows of a wave) per 4 KiB piece, 0 = units in order
     uint32_t units_per_piece;
     uint32_t affine_blocks;        // leading blocks that take part: a multiple of 8
+    int32_t window;                // kBand kernels: row i sees the keys max(0, i - window) .. i
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -55,7 +56,11 @@ enum class Mask { Causal, Bytes, None };
 // Compile-time switches of the kernels (FLAGS): two memory hints and three optional features.
 constexpr int kNtLoad = 1;   // non-temporal hint on the streaming loads
 constexpr int kNtStore = 2;  // non-temporal hint on the streaming stores
-constexpr int kAlibi = 4;    // causal forward adds the ALiBi bias -slope[head]*(i - j) to the scores
+// Forward adds the ALiBi bias slope[head] * min(j - i', 0) to the scores, i' = i + sk - sq the key
+// position of query row i (the last row of a decode step sees itself: the reference's AliBi module,
+// megatron/model/positional_embeddings.py:210-257, has sq == sk or sq == 1).  Under the causal mask
+// only j <= i is evaluated, where the minimum is the difference itself.
+constexpr int kAlibi = 4;
 // Attention dropout fused in.  Forward: besides y (kept for the backward pass) the kernel
 // stores dropout(y) = keep ? round(y)*1/(1-p) : 0 to out2.  Backward: the incoming gradient is
 // the gradient of dropout(y); the kernel regenerates the keep pattern and uses
@@ -78,6 +83,12 @@ constexpr int kBias = 16;
 // positions [sh, len + sh).  With kDropout a lane's 8 columns straddle two Philox groups (the
 // pattern is a function of the row-major element index).
 constexpr int kRagged = 32;
+// Sliding-window causal rows (Mask::Causal row kernels only): row i sees the keys lo .. i with
+// lo = max(0, i - window) -- the mask megatron/utils.py:67-80 builds for sliding_window_width.  The
+// row's buffer starts at the 128-bit access that holds key lo, accesses in front of it are given an
+// out-of-range offset, and chunks that lie wholly in front of the band are neither read nor
+// computed (wave-uniform branch), like those above the diagonal; their zeros are still stored.
+constexpr int kBand = 64;
 constexpr int kDefaultFlags = kNtLoad | kNtStore;
 constexpr uint32_t kOutOfRange = 0xFFFFFFFFu;  // a byte offset no buffer contains
 
@@ -140,6 +151,18 @@ __device__ __forceinline__ void ragged_head_store(rsrc_t r, const u32x4& o, bool
 __device__ __forceinline__ u32x2 ragged_head_mask(rsrc_t rm, bool first_lane) {
     const u32x2 m = buf_ld64(rm, first_lane ? 0u : kOutOfRange, 0);
     return u32x2{m.x << 8, (m.y << 8) | (m.x >> 24)};
+}
+
+// ALiBi: distance term of key `j` for the query at key position `ipos`, as a float.  Under the causal
+// mask only j <= ipos is ever used.
+template <Mask MASK>
+__device__ __forceinline__ float alibi_distance(int j, int ipos) {
+    return (float)((MASK == Mask::Causal) ? j - ipos : min(j - ipos, 0));
+}
+// Key position of query row i: the causal kernels align the triangle at the top left (j <= i).
+template <Mask MASK>
+__device__ __forceinline__ int alibi_row_position(uint32_t i, const SoftmaxArgs& a) {
+    return (MASK == Mask::Causal) ? (int)i : (int)i + a.sk - a.sq;
 }
 
 // Row of the bias tensor that belongs to score row `row`
@@ -239,6 +262,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
+    constexpr bool kBnd = (FLAGS & kBand) != 0;
+    static_assert(!kBnd || (MASK == Mask::Causal && (FLAGS & (kRagged | kAlibi | kBias | kDropout)) == 0),
+                  "the sliding window comes with the plain causal row kernels only");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave in block
@@ -257,9 +283,14 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     const bool first_lane = head && lane == 0;      // its first access would begin in front of the row
     DropoutArgs drop = a.drop;
     if constexpr ((FLAGS & kDropout) != 0) drop = resolve(drop);
-    // ALiBi: scale*(x + slope*(j - i)) = x*scale + slope2*(j - i), slope2 wave-uniform
+    // ALiBi: scale*(x + slope*(j - i')) = x*scale + slope2*(j - i'), slope2 wave-uniform
     float slope2 = 0.f;
     if constexpr ((FLAGS & kAlibi) != 0) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
+    const int ipos = alibi_row_position<MASK>(pos.i, a);
+    // kBand: first visible key of the row, and the start of the 128-bit access that holds it
+    int lo = 0;
+    if constexpr (kBnd) lo = max((int)pos.i - a.window, 0);
+    const int lo8 = lo & ~(kVec - 1);
     u32x4 raw[NCH];
     u32x4 rawb[NCH];  // kBias
     u32x2 mk[NCH];
@@ -271,8 +302,11 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         const uint32_t row_bytes = (uint32_t)(kRag ? pos.len : (pos.len + kVec - 1) & ~(kVec - 1)) * 2u;
         const rsrc_t rx = make_rsrc(x, row_bytes);
 #pragma unroll
-        for (int c = 0; c < NCH; ++c)
-            raw[c] = buf_ld128<kLdNt>(rx, (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2, 0);
+        for (int c = 0; c < NCH; ++c) {
+            uint32_t off = (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2;
+            if constexpr (kBnd) off = ((int)off < lo8 * 2) ? kOutOfRange : off;  // in front of the band: nothing fetched
+            raw[c] = buf_ld128<kLdNt>(rx, off, 0);
+        }
         if constexpr (kRag) {
             tail_x = ragged_tail16(rx, pos.len, sh);
             if (head) raw[0] |= ragged_head_load(rx, first_lane);
@@ -313,7 +347,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;  // first position of the chunk (wave-uniform)
-            if (c0 < plen) {
+            if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 const int col = c0 + lane * kVec - sh;  // first column of the lane, -1 in front of the row
                 if constexpr (kRag) {
                     if (c0 + kChunk >= plen) {  // the chunk that holds the row end
@@ -331,6 +365,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 }
                 // no lane of the wave crosses the row end (or holds the position in front of the row)
                 bool plain = (c0 + kChunk <= plen) && !(head && c == 0);
+                if constexpr (kBnd) plain = plain && c0 >= lo;
                 if constexpr (MASK == Mask::Bytes) {
                     plain = plain && (__builtin_amdgcn_ballot_w64((mk[c].x | mk[c].y) != 0) == 0);
                 }
@@ -338,7 +373,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     bias[k] = 0.f;
-                    if constexpr ((FLAGS & kAlibi) != 0) bias[k] = slope2 * (float)(col + k - (int)pos.i);
+                    if constexpr ((FLAGS & kAlibi) != 0) bias[k] = slope2 * alibi_distance<MASK>(col + k, ipos);
                 }
                 if (plain) {
 #pragma unroll
@@ -351,6 +386,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                     for (int k = 0; k < 8; ++k) {
                         bool keep = (col + k) < len;
                         if constexpr (kRag) keep = keep && (col + k) >= 0;
+                        if constexpr (kBnd) keep = keep && (col + k) >= lo;
                         if constexpr (MASK == Mask::Bytes) {
                             const uint32_t w = (k < 4) ? mk[c].x : mk[c].y;
                             keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
@@ -369,7 +405,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
-            if (c0 < plen) {
+            if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     v[c][k] = fast_exp2(v[c][k] - mx);
@@ -409,7 +445,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             o[c] = u32x4{0, 0, 0, 0};
-            if (c0 < plen) {
+            if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) v[c][k] *= inv;
                 o[c] = pack8<T>(v[c]);
@@ -450,6 +486,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     __shared__ float red_sum[WPR * RPB];
     constexpr bool kLdNt = (FLAGS & kNtLoad) != 0, kStNt = (FLAGS & kNtStore) != 0;
     constexpr bool kRag = (FLAGS & kRagged) != 0;
+    constexpr bool kBnd = (FLAGS & kBand) != 0;
+    static_assert(!kBnd || (MASK == Mask::Causal && (FLAGS & (kRagged | kDropout)) == 0),
+                  "the sliding window comes with the plain causal row kernels only");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -457,6 +496,10 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     const int wir = wib % WPR;
     const int sk = a.sk;
     const RowPos pos = locate<MASK>(xcd_slot(blockIdx.x, rib, RPB, a), a);
+    // kBand: first visible key of the row, and the start of the 128-bit access that holds it
+    int lo = 0;
+    if constexpr (kBnd) lo = max((int)pos.i - a.window, 0);
+    const int lo8 = lo & ~(kVec - 1);
     // kRagged: the row lies one position later on the lanes when it starts on an odd element; the
     // position in front of it stays zero in both tensors and is never stored
     int sh = 0;
@@ -474,7 +517,8 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const uint32_t off = (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2;
+            uint32_t off = (c == 0 && first_lane) ? kOutOfRange : voff + c * WPR * kChunk * 2;
+            if constexpr (kBnd) off = ((int)off < lo8 * 2) ? kOutOfRange : off;  // in front of the band: nothing fetched
             rg[c] = buf_ld128<kLdNt>(bg, off, 0);
             rp[c] = buf_ld128<kLdNt>(by, off, 0);
         }
@@ -499,7 +543,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             kb[c] = 0xffu;
-            if (c0 < plen) {
+            if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 const int col = c0 + lane * kVec - sh;  // first column of the lane
                 if constexpr (kRag) {
                     if (c0 + kChunk >= plen) {  // the chunk that holds the row end
@@ -521,6 +565,13 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                     for (int k = 0; k < 8; ++k)
                         if ((col + k) >= len) gv[k] = pv[k] = 0.f;
                 }
+                if constexpr (kBnd) {
+                    if (c0 < lo) {  // the lane holding the first visible key has loaded the columns in front of it
+#pragma unroll
+                        for (int k = 0; k < 8; ++k)
+                            if ((col + k) < lo) gv[k] = pv[k] = 0.f;
+                    }
+                }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) dot = fmaf(gv[k], pv[k], dot);
             }
@@ -534,7 +585,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         for (int c = 0; c < NCH; ++c) {
             const int c0 = (wir + WPR * c) * kChunk;
             u32x4 o = u32x4{0, 0, 0, 0};
-            if (c0 < plen) {
+            if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 float gv[8], pv[8];
                 unpack8<T>(rg[c], gv);
                 unpack8<T>(rp[c], pv);
@@ -544,6 +595,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
                     if constexpr ((FLAGS & kDropout) != 0) gv[k] = ((kb[c] >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                     gv[k] = a.scale * (pv[k] * (gv[k] - dot));
                     if ((c0 + kChunk > plen) && (col + k) >= len) gv[k] = 0.f;
+                    if constexpr (kBnd) {
+                        if (c0 < lo && (col + k) < lo) gv[k] = 0.f;
+                    }
                 }
                 o = pack8<T>(gv);
             }
@@ -662,7 +716,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
         const uint32_t i = wrap_row(i0 + lr, (uint32_t)a.sq);
         len[p] = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
         if (lr >= rows_here) len[p] = 0;
-        ipos[p] = (int)i;
+        ipos[p] = alibi_row_position<MASK>(i, a);
         slope2[p] = 0.f;
         if constexpr ((FLAGS & kAlibi) != 0) {
             const uint32_t safe_row = lr < rows_here ? row : row0;
@@ -706,7 +760,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
                     keep = keep && (((w >> (8 * (k & 3))) & 0xffu) == 0);
                 }
                 float bias = 0.f;
-                if constexpr ((FLAGS & kAlibi) != 0) bias = slope2[p] * (float)(col + k - ipos[p]);
+                if constexpr ((FLAGS & kAlibi) != 0) bias = slope2[p] * alibi_distance<MASK>(col + k, ipos[p]);
                 v[c][k] = keep ? fmaf(v[c][k], a.scale, bias) : ninf;
                 mx = fmaxf(mx, v[c][k]);
             }
@@ -1135,16 +1189,16 @@ __global__ __launch_bounds__(kGenericThreads) void softmax_fwd_generic_kernel(So
         mrow = a.mask + ((size_t)mb * a.sq + i) * sk;
     }
     const float ninf = -__builtin_inff();
-    // ALiBi (causal only): slopes given -> scores get slope*(j - i) before the scale
-    const float slope2 = (MASK == Mask::Causal && a.slopes != nullptr)
-                             ? a.slopes[(row / (uint32_t)a.sq) % a.np] * a.scale : 0.f;
+    // ALiBi: slopes given -> scores get slope * min(j - i', 0) before the scale (decided at run time here)
+    const float slope2 = (a.slopes != nullptr) ? a.slopes[(row / (uint32_t)a.sq) % a.np] * a.scale : 0.f;
+    const int ipos = alibi_row_position<MASK>(i, a);
     // bias tensor given -> added to the scores before the scale (decided at run time here)
     const char* brow = nullptr;
     if (a.bias != nullptr) brow = static_cast<const char*>(a.bias) + (size_t)bias_row(row, a) * sk * 2;
     auto score = [&](int j) {
         float xj = Elem<T>::load1(x + (size_t)j * 2);
         if (brow != nullptr) xj += Elem<T>::load1(brow + (size_t)j * 2);
-        return fmaf(xj, a.scale, slope2 * (float)(j - (int)i));
+        return fmaf(xj, a.scale, slope2 * alibi_distance<MASK>(j, ipos));
     };
 
     float mx = ninf;

@@ -7,14 +7,19 @@ kernels behind ``neox_masked_softmax_fwd/_bwd``.
 Differences: no ``key_seq_len <= 2048`` / ``query_seq_len > 1`` limits; masked
 scores are excluded (probability exactly 0) instead of being set to -10000; any
 non-zero mask byte masks; ``scale`` stays fp32.
+Additions: ``forward_alibi``, ``forward_bias``, ``forward_dropout`` / ``backward_dropout`` and
+``classify_mask``.
 """
 import torch
 
 from .. import _lib
 
 from .attention_dropout import state_pointer as _state_ptr
+from .scaled_upper_triang_masked_softmax_cuda import _grads, check_bias, check_slopes
 
 _HALF = (torch.float16, torch.bfloat16)
+_MASK_TYPES = (torch.bool, torch.uint8)
+_check, _code, _guard, _stream, _lib_handle = _lib.check, _lib.dtype_code, _lib.device_guard, _lib.current_stream, _lib.lib
 
 
 def _check_forward(input, mask):
@@ -25,88 +30,91 @@ def _check_forward(input, mask):
     if mask.dim() != 4:
         raise RuntimeError("expected 4D tensor")
     b, np_, sq, sk = input.shape
-    pad_batches = mask.size(0)
-    if not (pad_batches == 1 or pad_batches == b):
+    mb, m1, msq, msk = mask.shape
+    if not (mb == 1 or mb == b):
         raise RuntimeError("mask.size(0) must be 1 or the batch size")
-    if mask.size(1) != 1 or mask.size(2) != sq or mask.size(3) != sk:
+    if m1 != 1 or msq != sq or msk != sk:
         raise RuntimeError("mask must have shape [1 or b, 1, sq, sk]")
-    if mask.dtype not in (torch.bool, torch.uint8):
+    if mask.dtype not in _MASK_TYPES:
         raise RuntimeError("mask must be a bool or uint8 tensor")
-    _lib.require_gpu(input, mask)
-    return input.contiguous(), mask.contiguous()
+    if not (input.is_cuda and mask.is_cuda):
+        _lib.require_gpu(input, mask)
+    return (input if input.is_contiguous() else input.contiguous(),
+            mask if mask.is_contiguous() else mask.contiguous())
 
 
 def forward(input, mask, scale_factor):
     input, mask = _check_forward(input, mask)
     b, np_, sq, sk = input.shape
-    pad_batches = mask.size(0)
-    softmax_results = torch.empty_like(input, requires_grad=False)
+    softmax_results = torch.empty_like(input)
     if input.numel() == 0:
         return softmax_results
-    with _lib.device_guard(input):
-        _lib.check(
-            _lib.lib().neox_masked_softmax_fwd(
-                softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), float(scale_factor),
-                b, np_, sq, sk, pad_batches, _lib.dtype_code(input.dtype),
-                _lib.current_stream(input),
-            )
-        )
+    with _guard(input):
+        status = _lib_handle().neox_masked_softmax_fwd(
+            softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), float(scale_factor),
+            b, np_, sq, sk, mask.size(0), _code(input.dtype), _stream(input))
+    if status:
+        _check(status)
     return softmax_results
 
 
-def forward_bias(input, mask, bias, scale_factor):
-    """Mask-tensor softmax of ``scale * (input + bias)`` with the bias read inside the kernel;
-    ``bias``: ``[1 or b, np, sq, sk]`` (megatron/model/transformer.py:526-528).  No counterpart
-    in the reference's extension: it adds the bias in a separate pass."""
-    from .scaled_upper_triang_masked_softmax_cuda import check_bias
-
+def forward_alibi(input, mask, slopes, scale_factor):
+    """Mask-tensor softmax of ``scale * (input + alibi_bias)`` without materialising the bias:
+    head h adds ``slopes[h] * min(j - i', 0)`` with ``i' = i + sk - sq``, the matrix the
+    reference's ``AliBi`` module adds -- ``-slope * tril(i - j)``, and for a one-query decode step
+    its last row (megatron/model/positional_embeddings.py:210-257).  No counterpart in the
+    reference's extension: it adds the bias in a separate pass."""
     input, mask = _check_forward(input, mask)
-    _lib.require_gpu(bias)
+    b, np_, sq, sk = input.shape
+    slopes = check_slopes(slopes, np_)
+    softmax_results = torch.empty_like(input)
+    if input.numel() == 0:
+        return softmax_results
+    with _guard(input):
+        _check(_lib_handle().neox_masked_softmax_alibi_fwd(
+            softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), slopes.data_ptr(),
+            float(scale_factor), b, np_, sq, sk, mask.size(0), _code(input.dtype), _stream(input)))
+    return softmax_results
+
+
+def forward_bias(input, mask, bias, scale_factor, slopes=None):
+    """Mask-tensor softmax of ``scale * (input + bias)`` with the bias read inside the kernel;
+    ``bias``: ``[1 or b, np, sq, sk]`` (megatron/model/transformer.py:526-528); ``slopes``
+    (optional) adds the ALiBi bias of :func:`forward_alibi` as well.  No counterpart
+    in the reference's extension: it adds the bias in a separate pass."""
+    input, mask = _check_forward(input, mask)
     bias = check_bias(input, bias)
     b, np_, sq, sk = input.shape
-    softmax_results = torch.empty_like(input, requires_grad=False)
+    if slopes is not None:
+        slopes = check_slopes(slopes, np_)
+    softmax_results = torch.empty_like(input)
     if input.numel() == 0:
         return softmax_results
-    with _lib.device_guard(input):
-        _lib.check(
-            _lib.lib().neox_masked_softmax_bias_fwd(
-                softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), bias.data_ptr(),
-                float(scale_factor), b, np_, sq, sk, mask.size(0), bias.size(0),
-                _lib.dtype_code(input.dtype), _lib.current_stream(input),
-            )
-        )
+    with _guard(input):
+        _check(_lib_handle().neox_masked_softmax_bias_fwd(
+            softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(), bias.data_ptr(),
+            slopes.data_ptr() if slopes is not None else None, float(scale_factor),
+            b, np_, sq, sk, mask.size(0), bias.size(0), _code(input.dtype), _stream(input)))
     return softmax_results
-
-
-def _check_backward(output_grads, softmax_results):
-    if output_grads.dim() != 4 or softmax_results.dim() != 4:
-        raise RuntimeError("expected 4D tensor")
-    if output_grads.dtype not in _HALF or softmax_results.dtype not in _HALF:
-        raise RuntimeError("Only fp16 and bf16 are supported")
-    if output_grads.dtype != softmax_results.dtype or output_grads.shape != softmax_results.shape:
-        raise RuntimeError("output_grads and softmax_results must have the same dtype and shape")
-    _lib.require_gpu(output_grads, softmax_results)
-    return output_grads.contiguous(), softmax_results.contiguous()
 
 
 def backward(output_grads, softmax_results, scale_factor):
     """Returns d(input), written into ``output_grads`` itself when it is contiguous."""
-    output_grads, softmax_results = _check_backward(output_grads, softmax_results)
+    output_grads, softmax_results = _grads(output_grads, softmax_results, (4,))
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
-    with _lib.device_guard(output_grads):
-        _lib.check(
-            _lib.lib().neox_masked_softmax_bwd(
-                output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
-                float(scale_factor), b * np_ * sq, sk, _lib.dtype_code(output_grads.dtype),
-                _lib.current_stream(output_grads),
-            )
-        )
+    grads = output_grads.data_ptr()
+    with _guard(output_grads):
+        status = _lib_handle().neox_masked_softmax_bwd(
+            grads, grads, softmax_results.data_ptr(), float(scale_factor), b * np_ * sq, sk,
+            _code(output_grads.dtype), _stream(output_grads))
+    if status:
+        _check(status)
     return output_grads
 
 
-def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias=None):
+def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias=None, slopes=None):
     """Mask-tensor softmax and the attention dropout that follows it, in one kernel.
 
     Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
@@ -114,55 +122,81 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias
     the keep pattern drawn from Philox state ``(seed, offset)``
     (megatron/model/transformer.py:533-539).  ``state``, if given, is an int64 device tensor
     ``[seed, offset]`` read by the kernel when it runs (for launches recorded into a HIP graph)
-    and replaces the two numbers.  ``bias`` (optional) is added to the scores as in
-    :func:`forward_bias`.  No counterpart in the reference's extension.
+    and replaces the two numbers.  ``bias`` and ``slopes`` (optional) add to the scores as in
+    :func:`forward_bias` and :func:`forward_alibi`.  No counterpart in the reference's extension.
     """
     input, mask = _check_forward(input, mask)
     if bias is not None:
-        from .scaled_upper_triang_masked_softmax_cuda import check_bias
-
-        _lib.require_gpu(bias)
         bias = check_bias(input, bias)
     b, np_, sq, sk = input.shape
-    softmax_results = torch.empty_like(input, requires_grad=False)
-    dropped = torch.empty_like(input, requires_grad=False)
+    if slopes is not None:
+        slopes = check_slopes(slopes, np_)
+    softmax_results = torch.empty_like(input)
+    dropped = torch.empty_like(input)
     if input.numel() == 0:
         return softmax_results, dropped
-    with _lib.device_guard(input):
-        _lib.check(
-            _lib.lib().neox_masked_softmax_dropout_fwd(
-                dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
-                bias.data_ptr() if bias is not None else None, bias.size(0) if bias is not None else 0,
-                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
-                mask.size(0),
-                _lib.dtype_code(input.dtype), _lib.current_stream(input),
-            )
-        )
+    with _guard(input):
+        _check(_lib_handle().neox_masked_softmax_dropout_fwd(
+            dropped.data_ptr(), softmax_results.data_ptr(), input.data_ptr(), mask.data_ptr(),
+            slopes.data_ptr() if slopes is not None else None,
+            bias.data_ptr() if bias is not None else None, bias.size(0) if bias is not None else 0,
+            float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
+            mask.size(0), _code(input.dtype), _stream(input)))
     return softmax_results, dropped
 
 
 def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset, state=None):
     """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
     that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
-    output_grads, softmax_results = _check_backward(output_grads, softmax_results)
+    output_grads, softmax_results = _grads(output_grads, softmax_results, (4,))
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
-    with _lib.device_guard(output_grads):
-        _lib.check(
-            _lib.lib().neox_masked_softmax_dropout_bwd(
-                output_grads.data_ptr(), output_grads.data_ptr(), softmax_results.data_ptr(),
-                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b * np_ * sq, sk,
-                _lib.dtype_code(output_grads.dtype), _lib.current_stream(output_grads),
-            )
-        )
+    grads = output_grads.data_ptr()
+    with _guard(output_grads):
+        _check(_lib_handle().neox_masked_softmax_dropout_bwd(
+            grads, grads, softmax_results.data_ptr(), float(scale_factor), float(p), int(seed), int(offset),
+            _state_ptr(state), b * np_ * sq, sk, _code(output_grads.dtype), _stream(output_grads)))
     return output_grads
+
+
+def classify_mask(mask):
+    """Folds a mask ``[mask_b, 1, s, s]`` (bool/uint8 on the GPU) into four int32 on its device, from
+    which :func:`decode_mask_record` tells a causal mask -- plain or with a sliding window
+    (megatron/utils.py:67-80) -- from any other.  Asynchronous: the record is valid once the
+    current stream has got there.  No counterpart in the reference, whose causal branch never
+    looks at the mask (megatron/model/fused_softmax.py:173-179)."""
+    if mask.dim() != 4 or mask.size(1) != 1 or mask.size(2) != mask.size(3):
+        raise RuntimeError("mask must have shape [mask_b, 1, s, s]")
+    if mask.dtype not in _MASK_TYPES:
+        raise RuntimeError("mask must be a bool or uint8 tensor")
+    _lib.require_gpu(mask)
+    if not mask.is_contiguous():
+        mask = mask.contiguous()
+    record = torch.empty(4, dtype=torch.int32, device=mask.device)
+    with _guard(mask):
+        _check(_lib_handle().neox_mask_classify(record.data_ptr(), mask.data_ptr(), mask.size(0), mask.size(2),
+                                                mask.size(3), _stream(mask)))
+    return record
+
+
+def decode_mask_record(record):
+    """What four numbers of :func:`classify_mask` say: ``"causal"``, a sliding-window width (int),
+    or False for any other mask."""
+    bad, wmin, wmax, top = (int(v) for v in record)
+    if bad:
+        return False
+    if wmax < 0:
+        return "causal"
+    if wmin == wmax and top <= wmin:
+        return wmin
+    return False
 
 
 def get_batch_per_block(query_seq_len, key_seq_len, batches, attn_heads):
     """Rows per block of the reference's launch shape on a 64-wide wavefront
     (megatron/fused_kernels/scaled_masked_softmax.h:338-352); host arithmetic only."""
-    r = _lib.lib().neox_get_batch_per_block(query_seq_len, key_seq_len, batches, attn_heads)
+    r = _lib_handle().neox_get_batch_per_block(query_seq_len, key_seq_len, batches, attn_heads)
     if r < 0:
-        _lib.check(r)
+        _check(r)
     return r

@@ -19,18 +19,18 @@ Deliberate differences from the reference:
   runs the torch path beyond it) and need none of the ``sq % 4``,
   ``attn_batches % 4`` or ``% batch_per_block`` divisibility rules, which were
   artefacts of the CUDA launch shape -- see :meth:`is_kernel_available`;
-* by default the causal branch checks once per mask (per storage region, so ``detach()``ed
-  aliases share the verdict) that the mask really is the plain upper-triangular one and
-  otherwise (sliding-window masks, packed-sequence masks) runs the mask-tensor kernel with
-  the mask it was given -- the reference's causal kernel ignores the mask's contents, so
-  above its 2048 limit (torch path) and below it (fused kernel) the reference computes two
-  different things for such masks; here both agree with the torch path.  The constructor's
-  ``causal_mask_check`` selects how: ``"verify"`` (default) waits for the device-side
-  comparison the first time a mask is seen (one host synchronisation per new mask),
-  ``"lazy"`` never synchronises -- calls made while the comparison is in flight run the
-  mask-tensor kernel, which is right for any mask -- and ``"trust"`` restores the
-  reference's behaviour of never reading the mask
-  (megatron/model/fused_softmax.py:173-179).  A causal-fusion call with ``sq != sk`` (a step
+* by default the causal branch finds out once per mask (per storage region, so ``detach()``ed
+  aliases share the verdict) whether the mask really is the plain upper-triangular one, the
+  causal mask with a sliding window (served by a kernel that skips everything outside the
+  band) or something else (packed-sequence masks, ...: the mask-tensor kernel with the mask it
+  was given) -- the reference's causal kernel ignores the mask's contents, so above its 2048
+  limit (torch path) and below it (fused kernel) the reference computes two different things
+  for such masks; here both agree with the torch path.  The constructor's
+  ``causal_mask_check`` selects how: ``"lazy"`` (default) never synchronises -- one small
+  kernel reads the mask the first time it is seen, and calls made while its answer is in flight
+  run the mask-tensor kernel, which is right for any mask --, ``"verify"`` waits for that answer
+  (one host synchronisation per new mask), and ``"trust"`` restores the reference's behaviour of
+  never reading the mask (megatron/model/fused_softmax.py:173-179).  A causal-fusion call with ``sq != sk`` (a step
   against a key/value cache, where the reference asserts) also runs the mask-tensor kernel;
 * masked scores are excluded, so their probability is exactly 0 as in the torch
   path (the reference's padded kernel fills -10000), and a fully masked row is
@@ -92,8 +92,9 @@ def _recall(ctx):
 
 class _MaskVerdict:
     """One remembered mask region: the storage it lives in (weakly), the version counter it had,
-    and the verdict -- True / False, or None while the device-side comparison is still running
-    (then ``pending`` holds the pinned result slot and the event that follows the copy)."""
+    and the verdict -- ``"causal"``, a sliding-window width (int) or False for any other mask; None
+    while the device-side classification is still running (then ``pending`` holds the pinned
+    result slot and the event that follows the copy)."""
 
     __slots__ = ("storage", "version", "verdict", "pending")
 
@@ -104,18 +105,22 @@ class _MaskVerdict:
         self.pending = pending
 
     def poll(self, wait):
-        if self.verdict is None and self.pending is not None:
+        """The verdict if it is known by now.  ``wait``: True blocks until it is, False asks the
+        event, None does not touch the event at all (for use while a HIP graph is captured)."""
+        if self.verdict is None and self.pending is not None and wait is not None:
             slot, event = self.pending
             if wait:
                 event.synchronize()
             if wait or event.query():
-                self.verdict = bool(slot.item())  # host memory, the copy has finished: no sync
+                # host memory, the copy has finished: no synchronisation
+                self.verdict = _masked_ext.decode_mask_record(slot.tolist())
                 self.pending = None
         return self.verdict
 
 
 class _CausalMaskMemo:
-    """Remembers, per mask region, whether it equals ``triu(ones, 1)``.
+    """Remembers, per mask region, whether it is the causal mask ``triu(ones, 1)``, the causal mask
+    with a sliding window, or something else.
 
     A region is (storage address, offset, shape, strides); an entry is valid while the storage
     object it was decided for is alive (weak reference -- a recycled allocation is another
@@ -125,9 +130,11 @@ class _CausalMaskMemo:
     share the storage, the region and the version counter, hence the verdict.  (A write through
     ``.data`` or from outside torch bumps no counter and is not seen.)
 
-    The comparison runs on the device.  ``is_plain_causal(mask, wait=True)`` waits for it (one
-    host synchronisation per new mask); with ``wait=False`` it returns None while the result is
-    on its way and the caller uses a kernel that is right for any mask in the meantime."""
+    The classification is one kernel on the mask's device and stream that reads the mask once
+    (``neox_mask_classify``), followed by a 16-byte copy into pinned memory and an event.
+    ``classify(mask, wait=True)`` waits for it (one host synchronisation per new mask); with
+    ``wait=False`` it returns None while the result is on its way and the caller uses a kernel
+    that is right for any mask in the meantime."""
 
     def __init__(self, limit=64):
         self._entries = {}
@@ -149,49 +156,69 @@ class _CausalMaskMemo:
         return None
 
     def lookup(self, mask, wait=False):
-        """The verdict for this region in its current version: True, False, or None if it is
-        unknown (never asked, or still being computed and ``wait`` is False)."""
+        """The verdict for this region in its current version, or None if it is unknown (never
+        asked, or still being computed and ``wait`` is not True; see ``_MaskVerdict.poll``)."""
         hit = self._entry(mask)
         return None if hit is None else hit.poll(wait)
 
     def _result_slot(self, entry):
-        """A pinned host byte for the verdict of ``entry``.  The slots are handed out in turn; an
+        """Four pinned host words for the record of ``entry``.  The slots are handed out in turn; an
         entry that still waits for the slot's previous content reads it first (its copy finished
         long ago), so a slot is never overwritten under an entry that has not looked yet."""
         if self._slots is None:
-            self._slots = torch.zeros(256, dtype=torch.bool, pin_memory=True)
-            self._slot_owner = [None] * self._slots.numel()
-        self._next_slot = (self._next_slot + 1) % self._slots.numel()
+            self._slots = torch.zeros(256, 4, dtype=torch.int32, pin_memory=True)
+            self._slot_owner = [None] * self._slots.shape[0]
+        self._next_slot = (self._next_slot + 1) % self._slots.shape[0]
         owner = self._slot_owner[self._next_slot]
         if owner is not None:
             owner.poll(wait=True)
         self._slot_owner[self._next_slot] = entry
-        return self._slots[self._next_slot : self._next_slot + 1]
+        return self._slots[self._next_slot]
 
-    def is_plain_causal(self, mask, wait=True):
+    @staticmethod
+    def _classify_on_host(mask):
+        """The same verdict for a mask in host memory (plain torch)."""
+        s = mask.shape[-1]
+        hidden = mask.reshape(-1, s, s) != 0
+        rows = torch.arange(s).view(s, 1)
+        cols = torch.arange(s).view(1, s)
+        if bool((hidden == (cols > rows)).all()):
+            return "causal"
+        first = (~hidden[0]).float().argmax(-1)  # first visible key of every row of the first sample
+        widths = (torch.arange(s) - first)[first > 0]
+        if widths.numel() and bool((widths == widths[0]).all()):
+            w = int(widths[0])
+            if bool((hidden == ((cols > rows) | (cols < rows - w))).all()):
+                return w
+        return False
+
+    def classify(self, mask, wait=True):
+        """``"causal"``, a window width, False, or None (still running and ``wait`` is False)."""
         hit = self._entry(mask)
         if hit is not None:
             return hit.poll(wait)
-        sq, sk = mask.shape[-2], mask.shape[-1]
-        expected = torch.ones(sq, sk, dtype=torch.bool, device=mask.device).triu_(1)
-        same = (mask.bool() == expected).all()  # a 0-dim tensor on the mask's device
         key, storage = self._key(mask)
         if mask.is_cuda:
+            record = _masked_ext.classify_mask(mask)
             entry = _MaskVerdict(storage, mask._version)
             slot = self._result_slot(entry)
             with torch.cuda.device(mask.device):  # copy and event on the mask's device and stream
-                slot.copy_(same.view(1), non_blocking=True)
+                slot.copy_(record, non_blocking=True)
                 event = torch.cuda.Event()
                 event.record()
             entry.pending = (slot, event)
         else:
-            entry = _MaskVerdict(storage, mask._version, verdict=bool(same))
+            entry = _MaskVerdict(storage, mask._version, verdict=self._classify_on_host(mask))
         if len(self._entries) >= self._limit:
             self._entries = {k: v for k, v in self._entries.items() if v.storage() is not None}
             if len(self._entries) >= self._limit:
                 self._entries.clear()
         self._entries[key] = entry
         return entry.poll(wait)
+
+    def is_plain_causal(self, mask, wait=True):
+        verdict = self.classify(mask, wait)
+        return None if verdict is None else verdict == "causal"
 
 
 _causal_memo = _CausalMaskMemo()
@@ -217,6 +244,26 @@ class ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
         return _causal_ext.backward(output_grads, probs, scale), None
 
 
+class _CausalSoftmax4D(torch.autograd.Function):
+    """``ScaledUpperTriangMaskedSoftmax`` on ``[b, np, sq, sk]`` as the module holds it.  The
+    reference views the scores to three dims and the probabilities back
+    (megatron/model/fused_softmax.py:173-179); here the leading dims simply count as batches, which
+    spares the autograd graph two view nodes -- about 15 us of host time per forward + backward."""
+
+    @staticmethod
+    def forward(ctx, inputs, scale):
+        if not inputs.is_contiguous():
+            inputs = inputs.contiguous()
+        return _remember(ctx, _causal_ext.forward_nd(inputs, scale), scale)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        if not output_grads.is_contiguous():
+            output_grads = output_grads.contiguous()
+        return _causal_ext.backward_nd(output_grads, probs, scale), None
+
+
 class ScaledUpperTriangMaskedSoftmaxAlibi(torch.autograd.Function):
     """Causal softmax of ``scale * (inputs + alibi_bias(slopes))`` in one kernel; the bias is
     computed from the per-head slopes inside the kernel instead of being added to the scores
@@ -233,9 +280,9 @@ class ScaledUpperTriangMaskedSoftmaxAlibi(torch.autograd.Function):
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        b, np, sq, sk = probs.shape
-        grads = _causal_ext.backward(output_grads.reshape(-1, sq, sk), probs.view(-1, sq, sk), scale)
-        return grads.view(b, np, sq, sk), None, None
+        if not output_grads.is_contiguous():
+            output_grads = output_grads.contiguous()
+        return _causal_ext.backward_nd(output_grads, probs, scale), None, None
 
 
 def _bias_gradient(grads, bias_shape):
@@ -250,21 +297,21 @@ class ScaledUpperTriangMaskedSoftmaxBias(torch.autograd.Function):
     """Causal softmax of ``scale * (inputs + bias)`` in one kernel, the bias being a tensor
     ``[1 or b, np, sq, sk]`` such as the relative-position bias that the reference adds to the
     scores in a pass of its own (megatron/model/transformer.py:526-534).  Differentiable with
-    respect to ``inputs`` and ``bias``."""
+    respect to ``inputs`` and ``bias``.  ``slopes`` (optional, ``[np]``) adds the ALiBi bias as well."""
 
     @staticmethod
-    def forward(ctx, inputs, bias, scale):
+    def forward(ctx, inputs, bias, scale, slopes=None):
         scale = _fp32(scale)
         ctx.bias_shape = bias.shape
-        return _remember(ctx, _causal_ext.forward_bias(inputs, bias, scale), scale)
+        return _remember(ctx, _causal_ext.forward_bias(inputs, bias, scale, slopes), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        b, np, sq, sk = probs.shape
-        grads = _causal_ext.backward(output_grads.reshape(-1, sq, sk), probs.view(-1, sq, sk), scale)
-        grads = grads.view(b, np, sq, sk)
-        return grads, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[1] else None), None
+        if not output_grads.is_contiguous():
+            output_grads = output_grads.contiguous()
+        grads = _causal_ext.backward_nd(output_grads, probs, scale)
+        return grads, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[1] else None), None, None
 
 
 class ScaledMaskedSoftmaxBias(torch.autograd.Function):
@@ -272,16 +319,53 @@ class ScaledMaskedSoftmaxBias(torch.autograd.Function):
     ``ScaledUpperTriangMaskedSoftmaxBias``."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, bias, scale):
+    def forward(ctx, inputs, mask, bias, scale, slopes=None):
         scale = _fp32(scale)
         ctx.bias_shape = bias.shape
-        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale), scale)
+        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale, slopes), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
         grads = _masked_ext.backward(output_grads, probs, scale)
-        return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None
+        return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None, None
+
+
+class ScaledMaskedSoftmaxAlibi(torch.autograd.Function):
+    """Mask-tensor softmax of ``scale * (inputs + alibi_bias(slopes))`` in one kernel: what the
+    reference computes with ``AliBi.forward`` followed by the softmax when the fused causal kernel
+    does not serve the call -- general fusion, a sliding-window or other mask, or a one-query
+    step against a key/value cache (megatron/model/positional_embeddings.py:210-257,
+    megatron/model/transformer.py:529-534).  Gradient with respect to ``inputs`` only."""
+
+    @staticmethod
+    def forward(ctx, inputs, mask, slopes, scale):
+        scale = _fp32(scale)
+        return _remember(ctx, _masked_ext.forward_alibi(inputs, mask, slopes, scale), scale)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        return _masked_ext.backward(output_grads, probs, scale), None, None, None
+
+
+class ScaledSlidingWindowSoftmax(torch.autograd.Function):
+    """scale -> causal mask with a sliding window -> softmax, in one kernel that reads no mask
+    and no score outside the band: row i sees the keys ``max(0, i - window) .. i``, as under
+    ``get_attn_mask(seq_length, device, sliding_window_width=window)`` (megatron/utils.py:67-80).
+    ``inputs``: ``[attn_batches, sq, sk]`` or ``[b, np, sq, sk]`` as ``_causal_ext.window_kernel_takes``
+    describes."""
+
+    @staticmethod
+    def forward(ctx, inputs, scale, window):
+        scale = _fp32(scale)
+        ctx.window = window
+        return _remember(ctx, _causal_ext.forward_window(inputs, scale, window), scale)
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        probs, scale = _recall(ctx)
+        return _causal_ext.backward_window(output_grads, probs, scale, ctx.window), None, None
 
 
 class ScaledMaskedSoftmax(torch.autograd.Function):
@@ -314,8 +398,8 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
     there from the saved generator state instead of being stored.
 
     ``inputs``: ``[attn_batches, sq, sk]``, or ``[b, np, sq, sk]`` -- required with ``slopes``
-    (ALiBi slopes ``[np]``) or ``bias`` (``[1 or b, np, sq, sk]``, differentiable), which add to
-    the scores as in ``ScaledUpperTriangMaskedSoftmaxAlibi`` / ``...Bias``; at most one of them."""
+    (ALiBi slopes ``[np]``) and ``bias`` (``[1 or b, np, sq, sk]``, differentiable), which add to
+    the scores as in ``ScaledUpperTriangMaskedSoftmaxAlibi`` / ``...Bias``."""
 
     @staticmethod
     def forward(ctx, inputs, scale, p, slopes=None, bias=None):
@@ -339,14 +423,14 @@ class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
 class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     """Mask-tensor softmax followed by dropout with probability ``p``, in one kernel per
     pass; see ``ScaledUpperTriangMaskedSoftmaxDropout``.  ``bias`` (optional,
-    ``[1 or b, np, sq, sk]``, differentiable) adds to the scores."""
+    ``[1 or b, np, sq, sk]``, differentiable) and ``slopes`` (optional, ALiBi) add to the scores."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, p, bias=None):
+    def forward(ctx, inputs, mask, scale, p, bias=None, slopes=None):
         scale = _fp32(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
         probs, dropped = _masked_ext.forward_dropout(
-            inputs, mask, scale, p, seed, offset, state, bias=bias)
+            inputs, mask, scale, p, seed, offset, state, bias=bias, slopes=slopes)
         _remember(ctx, probs, scale)
         ctx.dropout = (p, seed, offset, state)
         ctx.bias_shape = None if bias is None else bias.shape
@@ -357,7 +441,7 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         probs, scale = _recall(ctx)
         grads = _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout)
         wants_bias = ctx.bias_shape is not None and ctx.needs_input_grad[4]
-        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None)
+        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None), None
 
 
 class SoftmaxFusionTypes(enum.Enum):
@@ -374,14 +458,14 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     mask_func: ``mask_func(scores, mask) -> scores`` used by the torch branch.
     softmax_in_fp32: torch branch computes in fp32 (the kernels always do).
     scale: multiplier applied before the softmax, or None.
-    causal_mask_check (not in the reference): ``"verify"`` | ``"lazy"`` | ``"trust"`` -- how the
-        upper_triang fusion treats the mask it is given; see the module text.
+    causal_mask_check (not in the reference): ``"lazy"`` (default) | ``"verify"`` | ``"trust"`` -- how
+        the upper_triang fusion treats the mask it is given; see the module text.
 
     Reference: megatron/model/fused_softmax.py:92-205.
     """
 
     def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
-                 causal_mask_check="verify"):
+                 causal_mask_check="lazy"):
         super().__init__()
         assert fusion_type in list(SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
         assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
@@ -398,6 +482,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         self.mask_func = mask_func
         self.softmax_in_fp32 = softmax_in_fp32
         self.scale = scale
+        self._last_mask = None  # (weak reference to the mask of the previous call, its version, its verdict)
         if self.fusion:
             load_fused_kernels()  # ImportError here, not at the first forward
 
@@ -405,7 +490,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         """``alibi_slopes`` (optional, ``[np]``) is an addition to the reference signature:
         ``forward(scores, mask, alibi_slopes=alibi.slopes)`` equals
         ``forward(alibi(scores), mask)`` (megatron/model/transformer.py:529-534) with the bias
-        evaluated in fp32 inside the causal kernel instead of a separate pass in half precision.
+        evaluated in fp32 inside the softmax kernel instead of a separate pass in half precision.
 
         ``dropout_p`` (optional, training only) is the second addition:
         ``forward(scores, mask, dropout_p=p)`` equals ``dropout(forward(scores, mask), p)``
@@ -415,40 +500,42 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         ``bias`` (optional, ``[1 or b, np, sq, sk]``) is the third:
         ``forward(scores, mask, bias=rpe)`` equals ``forward(scores + rpe, mask)``
         (megatron/model/transformer.py:526-534) with the bias read inside the softmax kernel and
-        the sum taken in fp32."""
+        the sum taken in fp32.
+
+        Every combination of the three runs in one kernel per pass whenever the fused softmax
+        serves the call."""
         assert input.dim() == 4  # [b, np, sq, sk]
-        if dropout_p:
-            return self.forward_with_dropout(input, mask, alibi_slopes, dropout_p, bias)
-        fused = self.is_kernel_available(mask, *input.size())
+        b, np, sq, sk = input.size()
+        if self.is_kernel_available(mask, b, np, sq, sk):
+            if alibi_slopes is None and bias is None and not dropout_p:
+                return self.forward_fused_softmax(input, mask)
+            return self.forward_fused_features(input, mask, alibi_slopes, dropout_p, bias)
+        # the unfused sequence of the reference: bias, ALiBi, softmax, dropout
         if bias is not None:
-            if fused and alibi_slopes is None:
-                return self.forward_fused_softmax(input, mask, bias)
             input = input + bias
         if alibi_slopes is not None:
-            b, np, sq, sk = input.size()
-            if fused and self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask):
-                scale = 1.0 if self.scale is None else self.scale
-                return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
             input = input + alibi_bias(alibi_slopes, sq, sk, input.device, input.dtype)
-        return self.forward_fused_softmax(input, mask) if fused else self.forward_torch_softmax(input, mask)
+        probs = self.forward_torch_softmax(input, mask)
+        return torch.nn.functional.dropout(probs, dropout_p, True) if dropout_p else probs
 
-    def forward_with_dropout(self, input, mask, alibi_slopes, dropout_p, bias=None):
-        """Softmax and dropout in one kernel per pass when the fused softmax serves the call --
-        with the ALiBi slopes (plain causal mask only) or a bias tensor folded in as well, though
-        not both at once; otherwise the softmax above followed by torch's dropout.  Under HIP
-        graph capture the fused kernels follow ``attention_dropout.graph_state(device)``, which
-        has to exist before the capture starts."""
+    def forward_fused_features(self, input, mask, alibi_slopes, dropout_p, bias):
+        """The fused branch with ALiBi slopes, a bias tensor and/or dropout folded in."""
         b, np, sq, sk = input.size()
-        fusable = self.is_kernel_available(mask, b, np, sq, sk) and (alibi_slopes is None or bias is None)
-        causal = fusable and self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask)
-        if fusable and alibi_slopes is not None and not causal:
-            fusable = False  # the mask-tensor kernels have no ALiBi variant
-        if not fusable:
-            return torch.nn.functional.dropout(self.forward(input, mask, alibi_slopes, 0.0, bias), dropout_p, True)
         scale = 1.0 if self.scale is None else self.scale
+        if alibi_slopes is not None:
+            assert sq == sk or sq == 1, "assumption sq == sk unless at inference time with cache in layer_past with sq == 1"
+        causal = self.mask_kind(mask, sq, sk) == "causal"
+        if dropout_p:
+            if causal:
+                return ScaledUpperTriangMaskedSoftmaxDropout.apply(input, scale, dropout_p, alibi_slopes, bias)
+            return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p, bias, alibi_slopes)
+        if bias is not None:
+            if causal:
+                return ScaledUpperTriangMaskedSoftmaxBias.apply(input, bias, scale, alibi_slopes)
+            return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale, alibi_slopes)
         if causal:
-            return ScaledUpperTriangMaskedSoftmaxDropout.apply(input, scale, dropout_p, alibi_slopes, bias)
-        return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p, bias)
+            return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
+        return ScaledMaskedSoftmaxAlibi.apply(input, mask, alibi_slopes, scale)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """Whether the fused branch serves this call.
@@ -488,42 +575,73 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         per_block = FusedScaleMaskSoftmax.get_batch_per_block(sq, sk, b, np)
         return ((b * np) if upper_triang else sq) % per_block == 0
 
-    def forward_fused_softmax(self, input, mask, bias=None):
+    def forward_fused_softmax(self, input, mask):
         b, np, sq, sk = input.size()
         scale = 1.0 if self.scale is None else self.scale
-        if not (self.upper_triang_mask_fusion and sq == sk and self.mask_is_plain_causal(mask)):
-            # general fusion, or a causal-fusion call whose mask is not the plain square triangle (a
-            # sliding-window mask, a step against a key/value cache): what the torch path computes,
-            # from the mask itself
-            if bias is not None:
-                return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale)
-            if not (torch.is_grad_enabled() and input.requires_grad):
-                return _masked_ext.forward(input, mask, _fp32(scale))
-            return ScaledMaskedSoftmax.apply(input, mask, scale)
-        if bias is not None:
-            return ScaledUpperTriangMaskedSoftmaxBias.apply(input, bias, scale)
-        # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
-        if not (torch.is_grad_enabled() and input.requires_grad):
-            # nothing to record: straight to the extension (the autograd Function costs the host
-            # several microseconds per call)
-            return _causal_ext.forward(input.view(-1, sq, sk), _fp32(scale)).view(b, np, sq, sk)
-        probs = ScaledUpperTriangMaskedSoftmax.apply(input.view(-1, sq, sk), scale)
-        return probs.view(b, np, sq, sk)
+        kind = self.mask_kind(mask, sq, sk)
+        records = torch.is_grad_enabled() and input.requires_grad
+        if kind == "causal":
+            # the causal kernel works on [attn_batches, sq, sk] and never reads `mask`
+            if not input.is_contiguous():
+                input = input.contiguous()
+            if not records:
+                # nothing to record: straight to the extension (the autograd Function costs the host
+                # several microseconds per call)
+                return _causal_ext.forward_nd(input, _fp32(scale))
+            return _CausalSoftmax4D.apply(input, _fp32(scale))
+        if kind is not None and _causal_ext.window_kernel_takes(input, kind):
+            # the causal mask with a sliding window: the band kernel reads neither the mask nor
+            # the scores outside the band
+            if not records:
+                return _causal_ext.forward_window(input, _fp32(scale), kind)
+            return ScaledSlidingWindowSoftmax.apply(input, scale, kind)
+        # general fusion, or a causal-fusion call whose mask is not (known to be) a causal one -- some
+        # other pattern, a step against a key/value cache, a verdict still on its way: what the torch
+        # path computes, from the mask itself
+        if not records:
+            return _masked_ext.forward(input, mask, _fp32(scale))
+        return ScaledMaskedSoftmax.apply(input, mask, scale)
 
-    def mask_is_plain_causal(self, mask):
-        """True if the causal kernel may serve ``mask``: it hides exactly the keys ``j > i``
-        (``"verify"``, ``"lazy"``; decided once per mask region, see ``_CausalMaskMemo``), or
-        without looking (``"trust"``).  ``"lazy"`` answers False while the comparison is still
-        running.  While a HIP graph is being captured nothing can be compared: a mask decided
-        before the capture keeps its verdict, for any other the answer is False and the
-        mask-tensor kernel is used."""
+    def mask_kind(self, mask, sq, sk):
+        """What the upper_triang fusion knows about ``mask``: ``"causal"``, a sliding-window width, or
+        None -- use the mask tensor (general fusion, ``sq != sk``, any other pattern, or a
+        classification that has not arrived yet).  See ``classify_mask``."""
+        if not self.upper_triang_mask_fusion or sq != sk:
+            return None
+        return self.classify_mask(mask)
+
+    def classify_mask(self, mask):
+        """``"causal"`` -- the mask hides exactly the keys ``j > i``, or ``causal_mask_check`` is
+        ``"trust"`` --, an int ``w`` -- the causal mask with a sliding window of that width --, or
+        None: not (known to be) either.
+
+        ``"verify"`` and ``"lazy"`` decide once per mask region (see ``_CausalMaskMemo``);
+        ``"lazy"`` never waits and answers None until the verdict has arrived.  While a HIP graph
+        is being captured nothing can be classified and no event may be asked: a mask decided
+        before the capture keeps its verdict, any other is None."""
         if self.causal_mask_check == "trust":
-            return True
-        if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
+            return "causal"
+        last = self._last_mask
+        if last is not None and last[0]() is mask and last[1] == mask._version:
+            verdict = last[2]  # the tensor object of the previous call, unchanged: no lookup
+        else:
+            verdict = self._classify_mask(mask)
+            if verdict is not None:
+                self._last_mask = (weakref.ref(mask), mask._version, verdict)
+        return None if verdict is False else verdict  # (a window of width 0 is a verdict too)
+
+    def _classify_mask(self, mask):
+        """The memo's answer: a verdict, False for any other mask, None while it is on its way."""
+        if (mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != mask.shape[3]
+                or mask.dtype not in (torch.bool, torch.uint8)):
             return False
         if mask.is_cuda and torch.cuda.is_current_stream_capturing():
-            return bool(_causal_memo.lookup(mask))
-        return bool(_causal_memo.is_plain_causal(mask, wait=self.causal_mask_check == "verify"))
+            return _causal_memo.lookup(mask, wait=None)
+        return _causal_memo.classify(mask, wait=self.causal_mask_check == "verify")
+
+    def mask_is_plain_causal(self, mask):
+        """True if the causal kernel may serve ``mask``; see ``classify_mask``."""
+        return self.classify_mask(mask) == "causal"
 
     def forward_torch_softmax(self, input, mask):
         """The unfused path: optional upcast, scale, ``mask_func``, softmax, cast back."""

@@ -232,6 +232,23 @@ def apply_rotary_pos_emb_torch(q, k, cos, sin, offset: int = 0):
     return apply_rotary_pos_emb(q, k, cos, sin, offset)
 
 
+# Writes made through raw pointers are invisible to autograd: the tensors' version counters have to be
+# bumped by hand, or a tensor that another op saved for its backward pass could be rotated in place
+# without the error autograd raises for such a change.
+_increment_version = getattr(torch.autograd.graph, "increment_version", None)
+
+
+def _may_bypass_autograd(*tensors):
+    """The in-place rotation may skip the autograd Function: nothing needs a gradient and the
+    version counters can still be bumped (or no graph is being recorded at all)."""
+    return not _needs_grad(*tensors) and (_increment_version is not None or not torch.is_grad_enabled())
+
+
+def _written_in_place(*tensors):
+    if _increment_version is not None:
+        _increment_version(tensors)
+
+
 def _rotary_in_place(q, k, cos, sin, offset, d_rot):
     cos2 = _as_table(cos, d_rot, offset + q.shape[0])
     sin2 = _as_table(sin, d_rot, offset + q.shape[0])
@@ -274,8 +291,9 @@ def apply_rotary_pos_emb_(q, k, cos, sin, offset: int = 0, rotary_ndims=None):
         )
     if d_rot > q.shape[-1] or d_rot % 2:
         raise RuntimeError(f"rotary_ndims={d_rot} must be even and <= head size {q.shape[-1]}")
-    if not _needs_grad(q, k):
+    if _may_bypass_autograd(q, k):
         _rotary_in_place(q, k, _on(cos, q.device), _on(sin, q.device), offset, d_rot)
+        _written_in_place(q, k)
         return q, k
     return _FusedRotaryInplace.apply(q, k, _on(cos, q.device), _on(sin, q.device), offset, d_rot)
 
@@ -332,10 +350,11 @@ def apply_rotary_pos_emb_qkv_(mixed_x_layer, cos, sin, offset: int = 0, rotary_n
             "cos/sin in fp32 or its dtype"
         )
     dev = mixed_x_layer.device
-    if not _needs_grad(mixed_x_layer):
+    if _may_bypass_autograd(mixed_x_layer):
         mixed = mixed_x_layer
         if mixed.numel():
             _rotary_in_place(mixed[..., :hn], mixed[..., hn : 2 * hn], _on(cos, dev), _on(sin, dev), offset, d_rot)
+            _written_in_place(mixed)
         return mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]
     mixed = _FusedQKVRotary.apply(mixed_x_layer, _on(cos, dev), _on(sin, dev), offset, d_rot)
     return mixed[..., :hn], mixed[..., hn : 2 * hn], mixed[..., 2 * hn :]

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NEOX_FUSED_ABI_VERSION 2
+#define NEOX_FUSED_ABI_VERSION 3
 
 typedef enum neox_dtype {
     NEOX_F16 = 0,  /* IEEE binary16 */
@@ -77,6 +77,21 @@ int neox_causal_softmax_alibi_fwd(void* y, const void* x, const float* slopes, f
                                   int32_t np, int32_t sq, int32_t sk, int32_t dtype, void* stream);
 
 /*
+ * Mask-tensor softmax with the ALiBi bias folded in:
+ *   y[n,h,i,j] = softmax_j(scale * (x[n,h,i,j] + slopes[h] * min(j - i', 0))),  i' = i + sk - sq,
+ * masked keys excluded as in neox_masked_softmax_fwd.  The bias is the reference's matrix
+ * -slope * tril(i - j) (zero above the diagonal); with sq == 1 the one query row stands at the
+ * last key position, the reference's rule for a decode step against a key/value cache.
+ * The gradient with respect to x is neox_masked_softmax_bwd.
+ * Replaces AliBi.forward followed by scaled_masked_softmax_cuda.forward or the torch branch
+ *   megatron/model/positional_embeddings.py:210-257 (the sq == 1 case: 236-250)
+ *   megatron/model/transformer.py:529-534
+ */
+int neox_masked_softmax_alibi_fwd(void* y, const void* x, const uint8_t* mask, const float* slopes, float scale,
+                                  int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b, int32_t dtype,
+                                  void* stream);
+
+/*
  * Causal softmax backward:  dx = scale * y * (dy - sum_j(dy*y)) over j <= i,
  * dx = 0 for j > i.  dx may alias dy (the reference overwrites dy in place).
  * Replaces scaled_upper_triang_masked_softmax_cuda.backward
@@ -116,16 +131,17 @@ int neox_masked_softmax_bwd(void* dx, const void* dy, const void* y, float scale
  * dtype of x, bias_b in {1, b} (1 = shared by all samples).  Causal / mask-tensor variants as
  * neox_causal_softmax_fwd / neox_masked_softmax_fwd.  The gradient with respect to x is
  * neox_*_softmax_bwd; the gradient with respect to the bias is that same tensor (summed over
- * the samples that share it).
- * Replaces "attention_scores += rpe" followed by the softmax extension call
+ * the samples that share it).  alibi_slopes (fp32 [np], NULL when absent) adds the ALiBi bias of
+ * neox_*_softmax_alibi_fwd on top, as a model with both a relative-position bias and ALiBi has it.
+ * Replaces "attention_scores += rpe" (and AliBi.forward) followed by the softmax extension call
  *   megatron/model/transformer.py:526-534, megatron/mpu/layers.py:353-380 (the bias)
  */
-int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, float scale, int32_t b,
-                                 int32_t np, int32_t sq, int32_t sk, int32_t bias_b, int32_t dtype,
-                                 void* stream);
+int neox_causal_softmax_bias_fwd(void* y, const void* x, const void* bias, const float* alibi_slopes,
+                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t bias_b,
+                                 int32_t dtype, void* stream);
 int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, const void* bias,
-                                 float scale, int32_t b, int32_t np, int32_t sq, int32_t sk,
-                                 int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream);
+                                 const float* alibi_slopes, float scale, int32_t b, int32_t np, int32_t sq,
+                                 int32_t sk, int32_t mask_b, int32_t bias_b, int32_t dtype, void* stream);
 
 /*
  * Softmax with the attention dropout that follows it folded in (training only).
@@ -142,8 +158,8 @@ int neox_masked_softmax_bias_fwd(void* y, const void* x, const uint8_t* mask, co
  * from the one counter value offset / 4, so the caller advances the generator's offset by 4
  * per call and no other consumer of the generator draws the same blocks.  0 <= p <= 1.
  * The forward entry points take x as [b, np, sq, sk] and two optional additions to the scores,
- * NULL when absent: alibi_slopes (causal only, as neox_causal_softmax_alibi_fwd) or a bias tensor
- * [bias_b, np, sq, sk] (as neox_*_softmax_bias_fwd), not both.
+ * NULL when absent: alibi_slopes (as neox_*_softmax_alibi_fwd) and a bias tensor
+ * [bias_b, np, sq, sk] (as neox_*_softmax_bias_fwd).
  * device_state, if not NULL, points to {seed, offset} (two uint64) in device memory that the
  * kernel reads when it runs, instead of the seed and offset arguments: a launch recorded into
  * a HIP graph then follows a state that the graph itself advances between replays.
@@ -161,7 +177,7 @@ int neox_causal_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
                                     int64_t batches, int32_t sq,
                                     int32_t sk, int32_t dtype, void* stream);
 int neox_masked_softmax_dropout_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask,
-                                    const void* bias, int32_t bias_b, float scale, float p,
+                                    const float* alibi_slopes, const void* bias, int32_t bias_b, float scale, float p,
                                     uint64_t seed, uint64_t offset, const uint64_t* device_state,
                                     int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                     int32_t dtype, void* stream);
@@ -171,6 +187,39 @@ int neox_masked_softmax_dropout_bwd(void* dx, const void* dy, const void* y, flo
                                     int32_t dtype, void* stream);
 int neox_dropout_keep_mask(uint8_t* keep, float p, uint64_t seed, uint64_t offset,
                            const uint64_t* device_state, int64_t n, void* stream);
+
+/*
+ * Causal softmax under a sliding window, forward and backward: row i sees the keys
+ * max(0, i - window) .. i, every other position is exactly 0 -- the mask that
+ * get_attn_mask(seq_length, device, sliding_window_width) builds, without reading a mask tensor
+ * and without reading the scores outside the band.  x, y (dy, dx): [batches, sq, sk] contiguous,
+ * 16-byte aligned, sq == sk, sk a multiple of 8 in (512, 32768]; other shapes are served by
+ * neox_masked_softmax_fwd with the mask tensor (NEOX_ERR_BAD_SHAPE / NEOX_ERR_MISALIGNED here).
+ * window >= sk - 1 is the plain causal softmax.  dx may alias dy.
+ * Replaces the torch branch with the sliding-window mask (the reference's fused causal kernel
+ * ignores the mask's contents and has no such variant)
+ *   megatron/utils.py:67-80, megatron/model/fused_softmax.py:173-199
+ */
+int neox_sliding_window_softmax_fwd(void* y, const void* x, float scale, int64_t batches, int32_t sq, int32_t sk,
+                                    int32_t window, int32_t dtype, void* stream);
+int neox_sliding_window_softmax_bwd(void* dx, const void* dy, const void* y, float scale, int64_t batches,
+                                    int32_t sq, int32_t sk, int32_t window, int32_t dtype, void* stream);
+
+/*
+ * Tells whether a mask tensor [mask_b, 1, sq, sk] (bytes, non-zero = masked, sq == sk) is the causal
+ * mask, plain or with a sliding window, so that a caller that is handed only the tensor can use the
+ * kernels that never read it.  Asynchronous like every entry point: it writes four int32 to
+ * `record` (device memory), which the caller reads once the stream has got there:
+ *   record[0]  != 0: some row's visible keys are not a contiguous run that ends on the diagonal
+ *   record[1], record[2]  smallest and largest i - lo over the rows whose first visible key lo is > 0
+ *                         (INT32_MAX and -1 if there is no such row)
+ *   record[3]  largest i over the rows with lo == 0 (-1 if none)
+ * Plain causal: record[0] == 0 and record[2] == -1.  Sliding window w: record[0] == 0,
+ * record[1] == record[2] == w and record[3] <= w.
+ * No counterpart in the reference, whose causal branch trusts the caller
+ *   megatron/model/fused_softmax.py:173-179, megatron/utils.py:67-80 (the masks it recognises)
+ */
+int neox_mask_classify(int32_t* record, const uint8_t* mask, int32_t mask_b, int32_t sq, int32_t sk, void* stream);
 
 /*
  * Rows-per-block figure the reference's dispatcher predicate consumes; kept for

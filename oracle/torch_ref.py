@@ -145,12 +145,16 @@ def alibi_slopes(n):
 
 
 def alibi_bias_fp32(slopes, sq, sk, device="cpu"):
-    """fp32 ALiBi bias [np, sq, sk]: -slope_h * (i - j) on j <= i, 0 above the diagonal.
-    Follows AliBi.forward, megatron/model/positional_embeddings.py:210-257 (sq == sk)."""
-    assert sq == sk
-    i = torch.arange(sq, device=device, dtype=torch.int32).view(sq, 1)
+    """fp32 ALiBi bias [np, sq, sk]: -slope_h * (i - j) on j <= i, 0 above the diagonal; with
+    sq == 1 (a decode step against a key/value cache) the last row of the [sk, sk] matrix.
+    Follows AliBi.forward, megatron/model/positional_embeddings.py:210-257 (sq != sk: 236-250)."""
     j = torch.arange(sk, device=device, dtype=torch.int32).view(1, sk)
-    dist = -torch.tril(i - j).float()
+    if sq != sk:
+        assert sq == 1, "assumption sq == sk unless at inference time with cache in layer_past with sq == 1"
+        dist = -((sk - 1) - j).float()  # row sk - 1 of the [sk, sk] matrix, without building it
+    else:
+        i = torch.arange(sk, device=device, dtype=torch.int32).view(sk, 1)
+        dist = -torch.tril(i - j).float()
     return dist * torch.as_tensor(slopes, dtype=torch.float32, device=device).view(-1, 1, 1)
 
 

@@ -99,6 +99,15 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 6, st, None, st, None, 8, 0, F16, F32, 0, None) == -3
     assert b"smaller than d_rot" in lib.neox_fused_last_error()
     assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, 9, 0, None) == -2
+    # the d dims a call delivers per head must fit the head stride of every tensor with several heads:
+    # a full 16-dim head given with a narrower output view would run into the next head
+    wide = (ctypes.c_int64 * 3)(64, 32, 16)
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 16, wide, None, st, None, 8, 0, F16, F32, 0, None) == -4
+    assert b"out_q head stride 8 is smaller than d=16" in lib.neox_fused_last_error()
+    assert rope(p, None, p, None, p, p, 4, 1, 2, 0, 8, 16, st, None, wide, None, 8, 0, F16, F32, 0, None) == -4
+    assert b"q head stride 8 is smaller than d=16" in lib.neox_fused_last_error()
+    assert rope(p, p, p, p, p, p, 4, 1, 1, 2, 8, 16, st, st, wide, wide, 8, 0, F16, F32, 0, None) == -4
+    assert b"k head stride" in lib.neox_fused_last_error()
     freqs = lib.neox_rope_apply_freqs
     assert freqs(p, None, p, None, None, 4, 1, 2, 0, 8, 8, st, None, st, None, 8, 0, F16, 0, None) == -1
     assert freqs(p, None, p, None, p, 4, 1, 2, 0, 8, 8, st, None, st, None, 4, 0, F16, 0, None) == -4
@@ -248,6 +257,12 @@ def test_plain_causal_mask_detection_and_memo():
     assert f(plain) and f(plain)
     assert f(plain.expand(3, 1, 9, 9).contiguous()) and f(plain.to(torch.uint8))
     assert not f(R.get_attn_mask(9, sliding_window_width=2))
+    assert mod.classify_mask(R.get_attn_mask(9, sliding_window_width=2)) == 2
+    assert mod.classify_mask(R.get_attn_mask(9, sliding_window_width=0)) == 0
+    assert mod.classify_mask(R.get_attn_mask(9, sliding_window_width=8)) == "causal"  # the window hides nothing
+    ragged = R.get_attn_mask(9, sliding_window_width=2).clone()
+    ragged[0, 0, 7, 5] = True  # one row with a narrower window: no single width
+    assert mod.classify_mask(ragged) is None
     assert not f(torch.zeros(1, 1, 9, 9, dtype=torch.bool))
     assert not f(plain[0])  # not 4-D
     per_sample = plain.expand(2, 1, 9, 9).clone()
@@ -270,11 +285,11 @@ def test_aliases_of_a_mask_share_its_verdict():
     assert memo.lookup(plain) is None  # never asked
     assert mod.mask_is_plain_causal(plain)
     for alias in (plain.detach(), plain.view(1, 1, 12, 12), plain[:], plain.detach().detach()):
-        assert alias is not plain and memo.lookup(alias) is True
+        assert alias is not plain and memo.lookup(alias) == "causal"
     assert memo.lookup(plain[..., :11, :11]) is None  # another region of the same storage
     assert memo.lookup(plain.clone()) is None          # another storage
     window = R.get_attn_mask(12, sliding_window_width=3)
-    assert not mod.mask_is_plain_causal(window) and memo.lookup(window.detach()) is False
+    assert not mod.mask_is_plain_causal(window) and memo.lookup(window.detach()) == 3
     alias = plain.detach()
     alias[0, 0, 11, 0] = True  # a write through an alias bumps the shared version counter
     assert memo.lookup(plain) is None and not mod.mask_is_plain_causal(plain)
@@ -299,7 +314,9 @@ def test_causal_mask_check_modes():
     assert not module("lazy").mask_is_plain_causal(window)  # CPU masks are decided at once
     assert module("lazy").mask_is_plain_causal(R.get_attn_mask(7))
     assert module("trust").mask_is_plain_causal(window)  # the reference never reads the mask
-    assert FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None).causal_mask_check == "verify"
+    # the default never synchronises the host: the reference's causal branch does not either
+    # (megatron/model/fused_softmax.py:173-179), and GPT-NeoX builds a fresh mask per micro-batch
+    assert FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.none, None, True, None).causal_mask_check == "lazy"
     with pytest.raises(AssertionError):
         module("sometimes")
 
@@ -336,11 +353,11 @@ def test_public_names_and_signatures_match_the_reference_modules():
     def params(fn):
         return list(inspect.signature(fn).parameters)
 
-    # the reference's positional parameters, plus one optional keyword that defaults to checking
+    # the reference's positional parameters, plus one optional keyword that defaults to checking without waiting
     assert params(FusedScaleMaskSoftmax.__init__) == [
         "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale",
         "causal_mask_check"]
-    assert inspect.signature(FusedScaleMaskSoftmax.__init__).parameters["causal_mask_check"].default == "verify"
+    assert inspect.signature(FusedScaleMaskSoftmax.__init__).parameters["causal_mask_check"].default == "lazy"
     # the reference's positional parameters, plus three optional additions that default to "off"
     assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask", "alibi_slopes", "dropout_p", "bias"]
     assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["bias"].default is None

@@ -424,7 +424,8 @@ def test_fused_dropout_in_a_hip_graph_draws_a_fresh_pattern_per_replay(device):
     g = normal(shape, torch.float16, device, 33)
     pad = R.padding_mask(torch.tensor([256, 100]), 256, 256, device)
     causal = R.get_attn_mask(256, device)
-    mc = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func, True, 0.5)
+    mc = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.upper_triang, R.gpt2_attention_mask_func, True, 0.5,
+                               causal_mask_check="verify")
     mg = FusedScaleMaskSoftmax(True, False, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.5)
     assert mc.mask_is_plain_causal(causal)  # decided (with a host sync) before the capture
     torch.manual_seed(99)
@@ -510,8 +511,10 @@ def test_causal_dropout_with_alibi_or_bias(device, shape, dtype):
         dx = causal_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
         ref = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
         assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
-    with pytest.raises(RuntimeError, match="not both"):
-        causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
+    # both at once: the probabilities of the bias kernel with the slopes on top, dropped alike
+    y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
+    assert torch.equal(y, causal_ext.forward_bias(x, bias, scale, slopes))
+    assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
     with pytest.raises(RuntimeError, match="4D"):
         causal_ext.forward_dropout(x.view(-1, s, s), scale, p, seed, offset, slopes=slopes)
 

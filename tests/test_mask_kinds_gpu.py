@@ -1,0 +1,309 @@
+"""Causal masks recognised on the device, the sliding-window kernels, and the module's default of
+never synchronising the host (through the C-ABI; the oracle is the reference's torch path with the
+mask that megatron/utils.py:67-80 builds).
+
+Bars: forward within 2e-3 (bf16) / 1e-3 (fp16) of the fp32 probabilities, backward within the same
+bars of fp32 autograd from x, hidden positions exactly 0 in both.
+"""
+import pytest
+import torch
+
+from gpt_neox_amd import fused_softmax as fs
+from gpt_neox_amd.fused_kernels import scaled_masked_softmax_cuda as masked_ext
+from gpt_neox_amd.fused_kernels import scaled_upper_triang_masked_softmax_cuda as causal_ext
+from gpt_neox_amd.fused_softmax import FusedScaleMaskSoftmax, ScaledSlidingWindowSoftmax, SoftmaxFusionTypes
+from bars import assert_grad
+from oracle import torch_ref as R
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-3, torch.float16: 1e-3}
+DTYPES = [torch.float16, torch.bfloat16]
+
+
+def gen(device, seed):
+    return torch.Generator(device=device).manual_seed(seed)
+
+
+def scores(shape, dtype, device, seed):
+    return (torch.randn(shape, device=device, generator=gen(device, seed)) * 8).to(dtype)
+
+
+def normal(shape, dtype, device, seed):
+    return torch.randn(shape, device=device, generator=gen(device, seed)).to(dtype)
+
+
+def max_err(a, b):
+    return (a.float() - b.float()).abs().max().item()
+
+
+def verdict(mask):
+    return masked_ext.decode_mask_record(masked_ext.classify_mask(mask).tolist())
+
+
+# ---------------------------------------------------------------------------------
+# neox_mask_classify
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("s", [1, 2, 7, 8, 37, 64, 200, 512, 513, 1000, 1024, 2048, 4100])
+def test_classify_recognises_the_masks_get_attn_mask_builds(device, s):
+    plain = R.get_attn_mask(s, device)
+    assert verdict(plain) == "causal"
+    assert verdict(plain.to(torch.uint8) * 255) == "causal"  # any non-zero byte hides
+    assert verdict(plain.expand(3, 1, s, s).contiguous()) == "causal"
+    for w in sorted({0, 1, 3, 7, 8, s // 3, s // 2, s - 2}):
+        if 0 <= w < s - 1:
+            assert verdict(R.get_attn_mask(s, device, sliding_window_width=w)) == w, (s, w)
+    # a window that hides nothing is the plain mask
+    assert verdict(R.get_attn_mask(s, device, sliding_window_width=s - 1)) == "causal"
+    assert verdict(R.get_attn_mask(s, device, sliding_window_width=s + 5)) == "causal"
+
+
+@pytest.mark.parametrize("s", [8, 37, 520, 2048])
+def test_classify_rejects_everything_else(device, s):
+    plain = R.get_attn_mask(s, device)
+    for i, j in ((s - 1, 1), (s // 2, s // 2), (0, s - 1), (s - 1, s - 2), (s // 2, s // 2 + 1)):
+        other = plain.clone()
+        other[0, 0, i, j] = not bool(other[0, 0, i, j])  # one key flipped anywhere
+        assert verdict(other) is False, (s, i, j)
+    assert verdict(torch.zeros(1, 1, s, s, dtype=torch.bool, device=device)) is False
+    assert verdict(torch.ones(1, 1, s, s, dtype=torch.bool, device=device)) is False
+    # samples that disagree: the second one has a window
+    two = torch.cat((plain, R.get_attn_mask(s, device, sliding_window_width=2)))
+    assert verdict(two) is False
+    # rows with different window widths
+    w3 = R.get_attn_mask(s, device, sliding_window_width=3).clone()
+    w3[0, 0, s - 1, s - 4] = True
+    assert verdict(w3) is False
+    # a window mask whose first rows are cut shorter than the window allows
+    if s > 6:
+        cut = R.get_attn_mask(s, device, sliding_window_width=4).clone()
+        cut[0, 0, 3, 0] = True  # row 3 would see key 0
+        assert verdict(cut) is False
+    # padding masks
+    assert verdict(R.padding_mask(torch.tensor([max(1, s // 2)]), s, s, device)) is False
+
+
+def test_classify_checks_its_arguments(device):
+    with pytest.raises(RuntimeError, match="shape"):
+        masked_ext.classify_mask(torch.zeros(1, 1, 4, 5, dtype=torch.bool, device=device))
+    with pytest.raises(RuntimeError, match="bool or uint8"):
+        masked_ext.classify_mask(torch.zeros(1, 1, 4, 4, dtype=torch.int32, device=device))
+    with pytest.raises(RuntimeError, match="GPU"):
+        masked_ext.classify_mask(torch.zeros(1, 1, 4, 4, dtype=torch.bool))
+    # a view that is not contiguous is classified by its contents
+    wide = torch.ones(1, 1, 16, 32, dtype=torch.bool, device=device)
+    wide[..., :16] = R.get_attn_mask(16, device)
+    assert verdict(wide[..., :16]) == "causal"
+
+
+# ---------------------------------------------------------------------------------
+# sliding-window kernels
+# ---------------------------------------------------------------------------------
+def check_window(device, batches, s, w, dtype, scale, seed):
+    x = scores((batches, s, s), dtype, device, seed)
+    g = normal((batches, s, s), dtype, device, seed + 1)
+    keep_x = x.clone()
+    y = causal_ext.forward_window(x, scale, w)
+    assert torch.equal(x, keep_x) and y.dtype == dtype and y.shape == x.shape
+    mask = R.get_attn_mask(s, device, sliding_window_width=w)
+    hidden = mask[0].expand_as(y)
+    ref, auto = R.softmax_autograd_fp32(x.unsqueeze(0), mask, scale, g.unsqueeze(0))
+    assert max_err(y, ref[0]) <= TOL[dtype], (s, w, dtype)
+    assert (y[hidden] == 0).all()
+    dx = causal_ext.backward_window(g.clone(), y, scale, w)
+    assert_grad(dx, auto[0], dtype, (s, w), y=y, g=g, scale=scale)
+    assert max_err(dx, R.softmax_backward_fp32(g, y, scale)) <= TOL[dtype]
+    assert (dx[hidden] == 0).all()
+    # the mask-tensor kernel on the same mask: the same function (not necessarily the same bits:
+    # the row's sums are taken over other chunks)
+    assert max_err(y, masked_ext.forward(x.unsqueeze(0), mask, scale)[0]) <= 2 * 2.0 ** -8
+    return x, y, g, dx
+
+
+WINDOW_CASES = [(520, 0), (520, 1), (520, 7), (520, 8), (520, 100), (520, 511), (520, 518),
+                (1024, 5), (1024, 512), (1024, 513), (1536, 600), (2048, 1), (2048, 511), (2048, 1024), (2048, 2040),
+                (2056, 1000), (2560, 3), (3072, 2049), (4096, 1024), (4104, 4000), (6144, 100), (8192, 4096), (8200, 4096)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("s,w", WINDOW_CASES)
+def test_sliding_window_sizes(device, s, w, dtype):
+    check_window(device, 3 if s <= 2056 else 1, s, w, dtype, 0.125, seed=s + w)
+
+
+@pytest.mark.parametrize("s,w", [(10240, 4096), (12288, 511), (16384, 8192), (20000, 4096), (28672, 1000), (32768, 4096)])
+def test_sliding_window_very_long_rows(device, s, w):
+    x = scores((1, s, s), torch.bfloat16, device, s)
+    y = causal_ext.forward_window(x, 0.05, w)
+    rows = torch.tensor([0, 1, w - 1, w, w + 1, w + 2, 511, 512, 513, s // 2, s - 2, s - 1], device=device).clamp_(0, s - 1)
+    mask = R.get_attn_mask(s, device, sliding_window_width=w)[0, 0][rows]
+    assert max_err(y[0][rows], R.softmax_fp32(x[0][rows], mask, 0.05)) <= TOL[torch.bfloat16]
+    assert (y[0][rows][mask] == 0).all()
+    # every row sums to one, and nothing lies outside the band anywhere
+    assert torch.allclose(y.float().sum(-1), torch.ones(1, s, device=device), atol=3e-2)
+    i = torch.arange(s, device=device).view(s, 1)
+    j = torch.arange(s, device=device).view(1, s)
+    assert (y[0][(j > i) | (j < i - w)] == 0).all()
+    g = normal((1, s, s), torch.bfloat16, device, 5)
+    dx = causal_ext.backward_window(g.clone(), y, 0.05, w)
+    assert max_err(dx[0][rows], R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)) <= TOL[torch.bfloat16]
+    assert (dx[0][rows][mask] == 0).all()
+
+
+def test_window_that_hides_nothing_is_the_causal_kernel(device):
+    # window >= s - 1: the same rows, the same order of summation, the same bits
+    for s in (1024, 2560, 8192):
+        x = scores((2, s, s), torch.float16, device, s)
+        g = normal((2, s, s), torch.float16, device, s + 1)
+        y = causal_ext.forward(x, 0.25)
+        for w in (s - 1, s, 10 * s):
+            assert torch.equal(causal_ext.forward_window(x, 0.25, w), y)
+            assert torch.equal(causal_ext.backward_window(g.clone(), y, 0.25, w), causal_ext.backward(g.clone(), y, 0.25))
+
+
+def test_sliding_window_kernels_ignore_what_lies_outside_the_band(device):
+    # NaN and Inf outside the band -- also in the columns that share a 128-bit access with its
+    # two ends -- change nothing, in the scores, the gradient and the probabilities
+    s, w, dtype = 2048, 700, torch.bfloat16
+    x = scores((2, s, s), dtype, device, 1)
+    g = normal((2, s, s), dtype, device, 2)
+    hidden = R.get_attn_mask(s, device, sliding_window_width=w)[0].expand_as(x)
+    y = causal_ext.forward_window(x, 0.125, w)
+    dx = causal_ext.backward_window(g.clone(), y, 0.125, w)
+    for poison in (float("nan"), float("inf"), float("-inf")):
+        xp, gp, yp = x.clone(), g.clone(), y.clone()
+        xp[hidden] = poison
+        gp[hidden] = poison
+        yp[hidden] = poison
+        assert torch.equal(causal_ext.forward_window(xp, 0.125, w), y)
+        assert torch.equal(causal_ext.backward_window(gp, yp, 0.125, w), dx)
+
+
+def test_sliding_window_entry_points_refuse_what_the_kernels_do_not_take(device):
+    x = scores((1, 512, 512), torch.float16, device, 1)
+    assert not causal_ext.window_kernel_takes(x, 4)
+    with pytest.raises(RuntimeError, match="sk=512"):
+        causal_ext.forward_window(x, 1.0, 4)
+    x = scores((1, 1001, 1001), torch.float16, device, 1)
+    assert not causal_ext.window_kernel_takes(x, 4)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        causal_ext.forward_window(x, 1.0, 4)
+    x = scores((1, 1024, 1024), torch.float16, device, 1)
+    assert causal_ext.window_kernel_takes(x, 4) and not causal_ext.window_kernel_takes(x, -1)
+    with pytest.raises(RuntimeError, match="negative"):
+        causal_ext.forward_window(x, 1.0, -1)
+    odd = scores((1024 * 1024 + 8,), torch.float16, device, 1)[1:1 + 1024 * 1024].view(1, 1024, 1024)  # 2-byte aligned
+    assert not causal_ext.window_kernel_takes(odd, 4)
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        causal_ext.forward_window(odd, 1.0, 4)
+
+
+# ---------------------------------------------------------------------------------
+# the module: which kernel serves which mask, without a host synchronisation by default
+# ---------------------------------------------------------------------------------
+def module(dtype, scale=0.25, **kw):
+    return FusedScaleMaskSoftmax(dtype == torch.float16, dtype == torch.bfloat16, SoftmaxFusionTypes.upper_triang,
+                                 R.gpt2_attention_mask_func, True, scale, **kw)
+
+
+def test_module_serves_sliding_window_masks_with_the_window_kernel(device):
+    s, w, dtype = 2048, 512, torch.bfloat16
+    mod = module(dtype, causal_mask_check="verify")
+    x = scores((2, 3, s, s), dtype, device, 3)
+    g = normal((2, 3, s, s), dtype, device, 4)
+    window = R.get_attn_mask(s, device, sliding_window_width=w)
+    assert mod.mask_kind(window, s, s) == w
+    xin = x.clone().requires_grad_(True)
+    y = mod(xin, window)
+    assert torch.equal(y.detach(), causal_ext.forward_window(x.view(-1, s, s), 0.25, w).view_as(x))
+    ref, auto = R.softmax_autograd_fp32(x, window, 0.25, g)
+    assert max_err(y, ref) <= TOL[dtype] and (y[window.expand_as(y)] == 0).all()
+    y.backward(g.clone())
+    assert_grad(xin.grad, auto, dtype, y=y.detach(), g=g, scale=0.25)
+    assert (xin.grad[window.expand_as(y)] == 0).all()
+    with torch.no_grad():
+        assert torch.equal(mod(x, window), y.detach())
+    assert torch.equal(ScaledSlidingWindowSoftmax.apply(x.view(-1, s, s), 0.25, w).view_as(x), y.detach())
+    # shapes the window kernels do not take go to the mask-tensor kernel with the same mask
+    small = R.get_attn_mask(200, device, sliding_window_width=17)
+    xs = scores((1, 2, 200, 200), dtype, device, 5)
+    assert mod.mask_kind(small, 200, 200) == 17
+    assert torch.equal(mod(xs, small), masked_ext.forward(xs, small, 0.25))
+    # general fusion never classifies: the mask tensor is used as it is
+    gen_mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.25)
+    assert gen_mod.mask_kind(window, s, s) is None
+    assert torch.equal(gen_mod(x, window), masked_ext.forward(x, window, 0.25))
+
+
+def test_default_module_never_synchronises_the_host(device, monkeypatch):
+    # GPT-NeoX builds a fresh mask for every micro-batch (megatron/utils.py:82-109, called from
+    # megatron/training.py:377,525) and the reference's causal branch never looks at it
+    # (megatron/model/fused_softmax.py:173-179): the default module must not wait for the device
+    # either.  Fifty calls, each with a mask never seen before, with every way of waiting closed.
+    s, dtype = 1024, torch.float16
+    mod = module(dtype)
+    assert mod.causal_mask_check == "lazy"
+    x = scores((1, 2, s, s), dtype, device, 7).requires_grad_(True)
+    g = normal((1, 2, s, s), dtype, device, 8)
+    want = causal_ext.forward(x.detach().view(-1, s, s), 0.25).view_as(x)
+    want_w = masked_ext.forward(x.detach(), R.get_attn_mask(s, device, sliding_window_width=100), 0.25)
+    torch.cuda.synchronize()
+
+    def refuse(*args, **kwargs):
+        raise AssertionError("the default module waited for the device")
+
+    monkeypatch.setattr(torch.cuda.Event, "synchronize", refuse)
+    monkeypatch.setattr(torch.Tensor, "item", refuse)
+    monkeypatch.setattr(torch.cuda, "synchronize", refuse)
+    monkeypatch.setattr(torch.cuda.Stream, "synchronize", refuse)
+    outs, grads, outs_w = [], [], []
+    for call in range(50):
+        fresh = R.get_attn_mask(s, device)  # a new tensor every time
+        y = mod(x, fresh)
+        (dx,) = torch.autograd.grad(y, x, g.clone())
+        outs.append(y.detach())
+        grads.append(dx)
+        if call % 10 == 0:
+            # the same tensor again, later: its verdict has usually arrived and is read without waiting
+            outs.append(mod(x, fresh).detach())
+            outs_w.append(mod(x, R.get_attn_mask(s, device, sliding_window_width=100)).detach())
+    monkeypatch.undo()
+    torch.cuda.synchronize()
+    for y in outs:
+        assert torch.equal(y, want)  # whichever kernel served the call: the same bits
+    for y in outs_w:
+        assert max_err(y, want_w) <= 2 * 2.0 ** -11
+    ref = R.softmax_backward_fp32(g, want, 0.25)
+    for dx in grads:
+        assert max_err(dx, ref) <= TOL[dtype]
+    # afterwards every verdict is there, and none was waited for
+    assert fs._causal_memo.lookup(fresh) == "causal"
+
+
+def test_pending_verdicts_are_not_polled_during_graph_capture(device):
+    s, dtype = 1024, torch.float16
+    mod = module(dtype)
+    x = scores((1, 2, s, s), dtype, device, 9)
+    known = R.get_attn_mask(s, device)
+    mod(x, known)
+    torch.cuda.synchronize()
+    assert mod.mask_kind(known, s, s) == "causal"
+    pending = R.get_attn_mask(s, device)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mod(x, pending)  # classification launched on the capture stream, eagerly
+        with torch.cuda.graph(graph, stream=side):
+            kinds = (mod.mask_kind(known, s, s), mod.mask_kind(pending, s, s),
+                     mod.mask_kind(R.get_attn_mask(s, device), s, s))
+            out = mod(x, known)
+    torch.cuda.synchronize()
+    # decided before the capture: kept; in flight or never seen: the mask-tensor kernel, no event asked
+    assert kinds[0] == "causal" and kinds[2] is None and kinds[1] in (None, "causal")
+    for _ in range(3):
+        out.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, causal_ext.forward(x.view(-1, s, s), 0.25).view_as(x))

@@ -134,28 +134,52 @@ def test_dropout_and_bias_entry_points_validate_before_touching_the_gpu():
     assert status == -1
     status, msg = _call("neox_causal_softmax_dropout_bwd", a, b, c, 1.0, -0.1, 0, 0, None, 1, 8, 8, 0, None)
     assert status == -3
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, None, None, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
     assert status == -1
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, None, 0, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 3, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, None, None, 0, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "mask batch" in msg
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 0, 8, 0, None)
     assert status == -3
     status, msg = _call("neox_masked_softmax_dropout_bwd", a, b, c, 1.0, 0.1, 0, 0, None, 4, 8, 2, None)
     assert status == -2
-    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, a, b, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 0, None)
-    assert status == -3 and "not both" in msg
+    # ALiBi slopes that are not aligned to their element size, with and without a bias tensor
+    status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, a + 2, b, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 0, None)
+    assert status == -5
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, a + 2, None, 0, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
+    assert status == -5
     status, msg = _call("neox_causal_softmax_dropout_fwd", a, b, c, None, a, 3, 1.0, 0.1, 0, 0, None, 2, 1, 8, 8, 0, None)
     assert status == -3 and "bias batch" in msg
-    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, a + 1, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
+    status, msg = _call("neox_masked_softmax_dropout_fwd", a, b, c, a, None, a + 1, 1, 1.0, 0.1, 0, 0, None, 1, 1, 8, 8, 1, 0, None)
     assert status == -5
-    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, c, 1.0, 2, 1, 8, 8, 3, 0, None)
+    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, c, None, 1.0, 2, 1, 8, 8, 3, 0, None)
     assert status == -3 and "bias batch" in msg
-    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, None, 1.0, 2, 1, 8, 8, 1, 0, None)
+    status, msg = _call("neox_causal_softmax_bias_fwd", a, b, None, None, 1.0, 2, 1, 8, 8, 1, 0, None)
     assert status == -1
-    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 1, 4, 0, None)
+    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, None, 1.0, 2, 1, 8, 8, 1, 4, 0, None)
     assert status == -3 and "bias batch" in msg
-    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 1, 1, 7, None)
+    status, msg = _call("neox_masked_softmax_bias_fwd", a, b, c, a, None, 1.0, 2, 1, 8, 8, 1, 1, 7, None)
     assert status == -2
+    status, msg = _call("neox_masked_softmax_alibi_fwd", a, b, c, None, 1.0, 2, 1, 8, 8, 1, 0, None)
+    assert status == -1
+    status, msg = _call("neox_masked_softmax_alibi_fwd", a, b, c, a, 1.0, 2, 1, 8, 8, 3, 0, None)
+    assert status == -3 and "mask batch" in msg
+    # the sliding-window entry points take aligned square rows of 513 to 32768 columns only
+    status, msg = _call("neox_sliding_window_softmax_fwd", a, b, 1.0, 1, 512, 512, 4, 0, None)
+    assert status == -3 and "sk=512" in msg
+    status, msg = _call("neox_sliding_window_softmax_fwd", a, b, 1.0, 1, 1024, 2048, 4, 0, None)
+    assert status == -3 and "equal" in msg
+    status, msg = _call("neox_sliding_window_softmax_fwd", a, b, 1.0, 1, 1024, 1024, -1, 0, None)
+    assert status == -3 and "window" in msg
+    status, msg = _call("neox_sliding_window_softmax_bwd", a, b, c + 2, 1.0, 1, 1024, 1024, 4, 1, None)
+    assert status == -5
+    status, msg = _call("neox_sliding_window_softmax_bwd", a, None, c, 1.0, 1, 1024, 1024, 4, 1, None)
+    assert status == -1
+    status, msg = _call("neox_mask_classify", None, a, 1, 8, 8, None)
+    assert status == -1
+    status, msg = _call("neox_mask_classify", a, b, 1, 8, 9, None)
+    assert status == -3 and "equal" in msg
+    status, msg = _call("neox_mask_classify", a, b, 0, 8, 8, None)
+    assert status == -3
     status, msg = _call("neox_dropout_keep_mask", None, 0.1, 0, 0, None, 8, None)
     assert status == -1
     status, msg = _call("neox_dropout_keep_mask", a, float("nan"), 0, 0, None, 8, None)

@@ -196,6 +196,12 @@ def test_alibi_slopes_and_bias_closed_forms():
         for i in range(4):
             for j in range(4):
                 assert bias[h, i, j].item() == (-m * (i - j) if j <= i else 0.0)
+    # one query against a key/value cache: the query stands at the last key position
+    last = R.alibi_bias_fp32([0.5, 0.25], 1, 5)
+    assert last.shape == (2, 1, 5)
+    assert last[0, 0].tolist() == [-2.0, -1.5, -1.0, -0.5, 0.0] and last[1, 0].tolist() == [-1.0, -0.75, -0.5, -0.25, 0.0]
+    with pytest.raises(AssertionError):
+        R.alibi_bias_fp32([0.5], 2, 5)
 
 
 def test_alibi_softmax_row_closed_form():
