@@ -125,7 +125,7 @@ def test_alibi_and_a_bias_tensor_together(device, shape, shared, dtype):
     assert torch.equal(masked_ext.forward_bias(x, mask, bias, 0.125, torch.zeros_like(slopes)), masked_ext.forward_bias(x, mask, bias, 0.125))
 
 
-DROP_SHAPES = [(2, 3, 8, 8), (2, 2, 136, 136), (1, 4, 512, 512), (1, 2, 640, 640), (2, 2, 1024, 1024), (1, 2, 2048, 2048),
+DROP_SHAPES = [(2, 3, 8, 8), (2, 2, 5, 5), (2, 2, 136, 136), (1, 4, 512, 512), (1, 2, 640, 640), (2, 2, 1024, 1024), (1, 2, 2048, 2048),
                (1, 2, 4096, 4096), (2, 2, 37, 37), (1, 2, 1001, 1001), (2, 3, 1, 520)]
 
 
@@ -149,10 +149,16 @@ def test_dropout_with_alibi_on_every_kernel_family(device, shape, dtype):
         dx = masked_ext.backward_dropout(g.clone(), y, scale, p, seed, offset)
         ref = R.softmax_dropout_backward_fp32(g, y, keep, p, scale)
         assert max_err(dx, ref) <= TOL[dtype] * max(1.0, ref.abs().max().item())
+    y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
+    assert torch.equal(y, masked_ext.forward_bias(x, mask, bias, scale))
+    assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
     if sq == sk:
-        y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
-        assert torch.equal(y, causal_ext.forward_bias(x, bias, scale, slopes))
-        assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
+        for kwargs, plain in ((dict(slopes=slopes, bias=bias), causal_ext.forward_bias(x, bias, scale, slopes)),
+                              (dict(slopes=slopes), causal_ext.forward_alibi(x, slopes, scale)),
+                              (dict(bias=bias), causal_ext.forward_bias(x, bias, scale))):
+            y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, **kwargs)
+            assert torch.equal(y, plain)
+            assert torch.equal(dropped, R.dropout_with_mask(y, keep, p))
 
 
 def test_autograd_functions_with_slopes(device):

@@ -560,11 +560,27 @@ def test_dropout_function_gradient_reaches_the_bias(device, shared):
         assert max_err(bias.grad, br.grad) <= tol * max(1.0, br.grad.abs().max().item()) * (b if shared else 1)
 
 
+def alibi_bias_any_shape(slopes, sq, sk, device):
+    """The ALiBi bias as the C-ABI defines it for any sq: slope * min(j - i', 0) with i' = i + sk - sq,
+    fp32 [np, sq, sk].  For sq == sk and sq == 1 -- all the reference's module produces -- it is the
+    oracle's matrix (asserted in test_alibi_definition_for_any_query_count)."""
+    i = torch.arange(sq, device=device).view(sq, 1) + (sk - sq)
+    j = torch.arange(sk, device=device).view(1, sk)
+    return (j - i).clamp(max=0).float() * slopes.float().view(-1, 1, 1)
+
+
+def test_alibi_definition_for_any_query_count(device):
+    slopes = torch.tensor(R.alibi_slopes(6), device=device)
+    for sq, sk in ((9, 9), (1, 9), (1, 1), (520, 520), (1, 777)):
+        assert torch.equal(alibi_bias_any_shape(slopes, sq, sk, device), R.alibi_bias_fp32(slopes, sq, sk, device))
+
+
 def check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, shift, case):
     """One call of the kernels with the given mask kind (causal / random mask bytes), optional bias
-    tensor ("bias", "shared bias") or ALiBi slopes ("alibi"), dropout probability p and every tensor
-    (those of the backward pass too) starting `shift` elements into its allocation: forward and
-    backward against the oracle's fp32 expressions, with the kernels' own keep pattern."""
+    tensor ("bias", "shared bias") and / or ALiBi slopes ("alibi", "alibi+bias", "alibi+shared bias"),
+    dropout probability p and every tensor (those of the backward pass too) starting `shift` elements
+    into its allocation: forward and backward against the oracle's fp32 expressions, with the
+    kernels' own keep pattern."""
 
     def shifted(t, by):
         flat = torch.empty(t.numel() + by, dtype=t.dtype, device=device)
@@ -577,11 +593,11 @@ def check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, 
     bias = slopes = None
     logits = x.float()
     if "bias" in extra:
-        bias = shifted(normal((1 if extra == "shared bias" else b, heads, sq, sk), dtype, device, 2000 + case), shift)
+        bias = shifted(normal((1 if "shared bias" in extra else b, heads, sq, sk), dtype, device, 2000 + case), shift)
         logits = logits + bias.float()
-    if extra == "alibi":
+    if "alibi" in extra:
         slopes = torch.rand(heads, device=device, generator=gen(device, case)) * 0.5
-        logits = logits + R.alibi_bias_fp32(slopes, sq, sk, device)
+        logits = logits + alibi_bias_any_shape(slopes, sq, sk, device)
     if causal:
         mask = R.get_attn_mask(sk, device)
     else:
@@ -592,15 +608,20 @@ def check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, 
     seed, offset = 77 + case, 4 * case
     if p == 0.0:
         if causal:
-            if slopes is not None:
+            if bias is not None:
+                y = causal_ext.forward_bias(x, bias, scale, slopes)
+            elif slopes is not None:
                 y = causal_ext.forward_alibi(x, slopes, scale)
-            elif bias is not None:
-                y = causal_ext.forward_bias(x, bias, scale)
             else:
                 y = causal_ext.forward(x.view(-1, sq, sk), scale).view(x.shape)
             dx = causal_ext.backward(shifted(g, shift).view(-1, sq, sk), shifted(y, shift).view(-1, sq, sk), scale).view(x.shape)
         else:
-            y = masked_ext.forward_bias(x, mask, bias, scale) if bias is not None else masked_ext.forward(x, mask, scale)
+            if bias is not None:
+                y = masked_ext.forward_bias(x, mask, bias, scale, slopes)
+            elif slopes is not None:
+                y = masked_ext.forward_alibi(x, mask, slopes, scale)
+            else:
+                y = masked_ext.forward(x, mask, scale)
             dx = masked_ext.backward(shifted(g, shift), shifted(y, shift), scale)
         want_dx = R.softmax_backward_fp32(g, y, scale)
     else:
@@ -608,7 +629,7 @@ def check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, 
             y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, slopes=slopes, bias=bias)
             dx = causal_ext.backward_dropout(shifted(g, shift), shifted(y, shift), scale, p, seed, offset)
         else:
-            y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
+            y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias, slopes=slopes)
             dx = masked_ext.backward_dropout(shifted(g, shift), shifted(y, shift), scale, p, seed, offset)
         keep = rng.keep_mask(y.numel(), p, seed, offset, device).view(y.shape)
         if y.numel() <= 1 << 20:
@@ -632,7 +653,7 @@ def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
     import random
 
     rnd = random.Random(20250101)
-    for case in range(60):
+    for case in range(90):
         dtype = rnd.choice(DTYPES)
         sk = rnd.choice([rnd.randint(8, 70), rnd.randint(71, 520), rnd.randint(521, 2100), rnd.randint(2101, 9000)])
         causal = rnd.random() < 0.5
@@ -642,9 +663,7 @@ def test_seeded_random_row_lengths_alignments_and_feature_combinations(device):
             b, heads = 1, 1
         scale = rnd.choice([0.125, 0.5, 1.0])
         p = rnd.choice([0.0, 0.0, 0.1, 0.5])
-        extra = rnd.choice(["none", "none", "bias", "shared bias", "alibi"])
-        if extra == "alibi" and not causal:
-            extra = "none"
+        extra = rnd.choice(["none", "none", "bias", "shared bias", "alibi", "alibi+bias", "alibi+shared bias"])
         check_combination(device, dtype, causal, b, heads, sq, sk, scale, p, extra, rnd.randint(0, 9), case)
 
 
@@ -656,7 +675,7 @@ SHAPE_LENGTHS = [8, 16, 32, 64, 128, 160, 256, 320, 512, 640, 1024, 1280, 1536, 
                  20480, 28672]
 
 
-@pytest.mark.parametrize("extra", ["none", "bias", "shared bias", "alibi"])
+@pytest.mark.parametrize("extra", ["none", "bias", "shared bias", "alibi", "alibi+bias", "alibi+shared bias"])
 @pytest.mark.parametrize("p", [0.0, 0.25])
 def test_every_kernel_shape_with_every_feature_combination(device, extra, p):
     # each length as it is (aligned rows) and one column shorter (ragged rows of odd length), in
@@ -668,8 +687,7 @@ def test_every_kernel_shape_with_every_feature_combination(device, extra, p):
         for sk, shift in ((n, 0), (n - 1, 0) if n > 8 else (9, 0)) + (((8, 3),) if n == 8 else ()):
             for dtype in DTYPES:
                 case += 1
-                if extra != "alibi":
-                    check_combination(device, dtype, False, 2, 2, 3, sk, 0.25, p, extra, shift, case)
+                check_combination(device, dtype, False, 2, 2, 3, sk, 0.25, p, extra, shift, case)
                 check_combination(device, dtype, True, 1, 2 if sk <= 4096 else 1, sk, sk, 0.25, p, extra, shift, 500 + case)
         if n > 4096:
             torch.cuda.empty_cache()

@@ -69,7 +69,11 @@ def test_rows_with_a_mask_tensor_beyond_4_gib(device, sk, dtype):
     bias = big_normal((1, 1, sq, sk), dtype, device, 3)
     rows = sample_rows(sq, device, 4)
     xs, ms, bs = x[0, 0][rows].float(), mask[0, 0][rows], bias[0, 0][rows].float()
-    want = {False: R.softmax_fp32(xs, ms, scale), True: R.softmax_fp32(xs + bs, ms, scale)}
+    # ALiBi for sq != sk as the C-ABI defines it: slope * min(j - i', 0), i' = i + sk - sq (only the last sk rows get any)
+    slopes = torch.tensor([0.37], device=device)
+    ab = (torch.arange(sk, device=device).view(1, sk) - (rows.view(-1, 1) + sk - sq)).clamp(max=0).float() * slopes[0]
+    want = {False: R.softmax_fp32(xs, ms, scale), True: R.softmax_fp32(xs + bs, ms, scale),
+            "alibi": R.softmax_fp32(xs + ab, ms, scale), "alibi+bias": R.softmax_fp32(xs + ab + bs, ms, scale)}
     keep = rng.keep_mask(x.numel(), p, seed, offset, device).view(x.shape)[0, 0][rows]
 
     def check(y, with_bias, dropped=None):
@@ -83,6 +87,12 @@ def test_rows_with_a_mask_tensor_beyond_4_gib(device, sk, dtype):
     check(masked_ext.forward_bias(x, mask, bias, scale), True)
     y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset)
     check(y, False, dropped)
+    check(masked_ext.forward_alibi(x, mask, slopes, scale), "alibi")
+    check(masked_ext.forward_bias(x, mask, bias, scale, slopes), "alibi+bias")
+    y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, slopes=slopes)
+    check(y, "alibi", dropped)
+    y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias, slopes=slopes)
+    check(y, "alibi+bias", dropped)
     y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, bias=bias)
     check(y, True, dropped)
     # the backward pass reads neither mask nor bias: packed kernels on tensors beyond 4 GiB
@@ -118,6 +128,12 @@ def test_short_causal_rows_with_a_bias_tensor_beyond_4_gib(device, s, dtype):
 
     check(causal_ext.forward(x.view(-1, s, s), scale), want_plain)  # packed kernel beyond 4 GiB
     check(causal_ext.forward_bias(x, bias, scale), want_bias)
+    slopes = torch.rand(heads, device=device, generator=gen(device, 14)) * 0.5
+    ab = R.alibi_bias_fp32(slopes[pick], s, s, device)
+    want_both = R.softmax_fp32(x[0, pick].float() + bias[0, pick].float() + ab, mask, scale)
+    check(causal_ext.forward_bias(x, bias, scale, slopes), want_both)
+    y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, bias=bias, slopes=slopes)
+    check(y, want_both, dropped)
     y, dropped = causal_ext.forward_dropout(x, scale, p, seed, offset, bias=bias)
     check(y, want_bias, dropped)
     g = bias

@@ -131,22 +131,28 @@ def test_sliding_window_sizes(device, s, w, dtype):
     check_window(device, 3 if s <= 2056 else 1, s, w, dtype, 0.125, seed=s + w)
 
 
-@pytest.mark.parametrize("s,w", [(10240, 4096), (12288, 511), (16384, 8192), (20000, 4096), (28672, 1000), (32768, 4096)])
+@pytest.mark.parametrize("s,w", [(10240, 4096), (12288, 511), (13312, 4096), (16384, 8192), (20000, 4096), (28672, 1000), (32768, 4096)])
 def test_sliding_window_very_long_rows(device, s, w):
-    x = scores((1, s, s), torch.bfloat16, device, s)
+    for dtype in DTYPES:
+        check_very_long_window(device, s, w, dtype)
+        torch.cuda.empty_cache()
+
+
+def check_very_long_window(device, s, w, dtype):
+    x = scores((1, s, s), dtype, device, s)
     y = causal_ext.forward_window(x, 0.05, w)
     rows = torch.tensor([0, 1, w - 1, w, w + 1, w + 2, 511, 512, 513, s // 2, s - 2, s - 1], device=device).clamp_(0, s - 1)
     mask = R.get_attn_mask(s, device, sliding_window_width=w)[0, 0][rows]
-    assert max_err(y[0][rows], R.softmax_fp32(x[0][rows], mask, 0.05)) <= TOL[torch.bfloat16]
+    assert max_err(y[0][rows], R.softmax_fp32(x[0][rows], mask, 0.05)) <= TOL[dtype]
     assert (y[0][rows][mask] == 0).all()
     # every row sums to one, and nothing lies outside the band anywhere
     assert torch.allclose(y.float().sum(-1), torch.ones(1, s, device=device), atol=3e-2)
     i = torch.arange(s, device=device).view(s, 1)
     j = torch.arange(s, device=device).view(1, s)
     assert (y[0][(j > i) | (j < i - w)] == 0).all()
-    g = normal((1, s, s), torch.bfloat16, device, 5)
+    g = normal((1, s, s), dtype, device, 5)
     dx = causal_ext.backward_window(g.clone(), y, 0.05, w)
-    assert max_err(dx[0][rows], R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)) <= TOL[torch.bfloat16]
+    assert max_err(dx[0][rows], R.softmax_backward_fp32(g[0][rows], y[0][rows], 0.05)) <= TOL[dtype]
     assert (dx[0][rows][mask] == 0).all()
 
 
