@@ -199,8 +199,12 @@ template <typename T, Mask M, bool BWD, int EXTRA>
 static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t st) {
     int chunks = (a.sk + kChunk - 1) / kChunk;
     if constexpr ((EXTRA & kBand) != 0) {
-        // sliding-window rows: the row kernels below only (aligned rows of two chunks or more)
+        // sliding-window rows: the row kernels below only (aligned rows of two chunks or more), and the
+        // kernel shape goes by the chunks a band can touch -- w + 1 keys lie in at most w / 512 + 2
+        // chunks -- not by the row length: the waves hold the band, the rest of the row is zeros
         if (!vec_ok || chunks < 2 || a.sk > kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+        const int band_chunks = a.window / kChunk + 2;
+        if (band_chunks < chunks) chunks = band_chunks;
     } else if constexpr ((EXTRA & kRagged) != 0) {
         // rows at any alignment: the packed kernels up to 512 columns, the row kernels below beyond
         if (a.sk < kVec || a.sk >= kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
@@ -224,7 +228,7 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
             return launch_shape<T, M, BWD, EXTRA, 2, 2, 4>(a, st);
         }
     }
-    if constexpr (!BWD) {
+    if constexpr (!BWD && (EXTRA & kBand) == 0) {
         // Forward, rows that would leave a quarter or more of the 2-chunk shape's slots empty:
         // half as many waves with 3 or 4 chunks each.  Measured in an interleaved comparison:
         // +20-50 % just above a power of two (2056, 4104, 8200 columns), +4-15 % up to 3/4 (7/8 with

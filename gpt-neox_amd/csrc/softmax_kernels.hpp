@@ -268,6 +268,17 @@ __device__ __forceinline__ float row_combine(float v, float* red, int wib, int r
     }
 }
 
+// kBand: the waves of a row hold the NCH * WPR chunks from the band's first chunk on; the chunks of
+// the row in front of those and behind them hold nothing but zeros, which the waves store here,
+// dealt round-robin.  `first` = the band's first chunk (wave-uniform).
+template <bool NT, int NCH, int WPR>
+__device__ __forceinline__ void band_zero_fill(rsrc_t out, int first, int sk, int wir, int lane) {
+    const int all = (sk + kChunk - 1) / kChunk;
+    for (int g = wir; g < all; g += WPR) {
+        if (g < first || g >= first + NCH * WPR) buf_st128<NT>(out, u32x4{0, 0, 0, 0}, g * kChunk * 2 + lane * 16, 0);
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // forward
 //
@@ -300,7 +311,14 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     // kRagged: the row lies one position later on the lanes when it starts on an odd element
     int sh = 0;
     if constexpr (kRag) sh = ragged_shift(a.in0, pos.row, sk);
-    const int voff = lane * 16 + wir * kChunk * 2 - 2 * sh;
+    // kBand: first visible key of the row, and the start of the 128-bit access that holds it.  The
+    // waves' chunks are counted from the chunk that holds that key (wch instead of wir), so that a
+    // row needs only as many chunk slots as its band is long; see band_zero_fill for the rest.
+    int lo = 0;
+    if constexpr (kBnd) lo = max((int)pos.i - a.window, 0);
+    const int lo8 = lo & ~(kVec - 1);
+    const int wch = wir + lo / kChunk;  // the wave's first chunk of the row (wir without a window)
+    const int voff = lane * 16 + wch * kChunk * 2 - 2 * sh;
     const bool head = kRag && sh != 0 && wir == 0;  // wave-uniform: this wave holds the row start
     const bool first_lane = head && lane == 0;      // its first access would begin in front of the row
     DropoutArgs drop = a.drop;
@@ -309,10 +327,6 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
     float slope2 = 0.f;
     if constexpr ((FLAGS & kAlibi) != 0) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
     const int ipos = alibi_row_position<MASK>(pos.i, a);
-    // kBand: first visible key of the row, and the start of the 128-bit access that holds it
-    int lo = 0;
-    if constexpr (kBnd) lo = max((int)pos.i - a.window, 0);
-    const int lo8 = lo & ~(kVec - 1);
     u32x4 raw[NCH];
     u32x4 rawb[NCH];  // kBias
     u32x2 mk[NCH];
@@ -361,6 +375,11 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
             }
         }
     }
+    if constexpr (kBnd) {
+        // while the loads are in flight: the zeros of the chunks that no wave holds
+        const rsrc_t rz = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, pos.store ? (uint32_t)sk * 2u : 0u);
+        band_zero_fill<kStNt, NCH, WPR>(rz, lo / kChunk, sk, wir, lane);
+    }
     {
         const int len = pos.len;
         const int plen = len + sh;  // the row's columns lie at the positions [sh, plen)
@@ -370,7 +389,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         float mx = ninf;
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;  // first position of the chunk (wave-uniform)
+            const int c0 = (wch + WPR * c) * kChunk;  // first position of the chunk (wave-uniform)
             if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 const int col = c0 + lane * kVec - sh;  // first column of the lane, -1 in front of the row
                 if constexpr (kRag) {
@@ -428,7 +447,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         float sum = 0.f;
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;
+            const int c0 = (wch + WPR * c) * kChunk;
             if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
@@ -444,7 +463,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
                 sum = 0.f;
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
-                    const int col = (wir + WPR * c) * kChunk + lane * kVec - sh;
+                    const int col = (wch + WPR * c) * kChunk + lane * kVec - sh;
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         v[c][k] = ((col + k) < len && (col + k) >= 0) ? 1.f : 0.f;
@@ -467,7 +486,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         u32x4 o[NCH];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;
+            const int c0 = (wch + WPR * c) * kChunk;
             o[c] = u32x4{0, 0, 0, 0};
             if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
 #pragma unroll
@@ -485,7 +504,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
             // second output after the first: each stream is written in runs of whole rows
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
-                const int c0 = (wir + WPR * c) * kChunk;
+                const int c0 = (wch + WPR * c) * kChunk;
                 u32x4 o2 = u32x4{0, 0, 0, 0};
                 if (c0 < plen) {
                     const uint32_t bits = keep_bits_row8<kRag>(drop, pos.row, sk, c0 + lane * kVec - sh);
@@ -520,15 +539,17 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
     const int wir = wib % WPR;
     const int sk = a.sk;
     const RowPos pos = locate<MASK>(xcd_slot(blockIdx.x, rib, RPB, a), a);
-    // kBand: first visible key of the row, and the start of the 128-bit access that holds it
+    // kBand: first visible key of the row, the start of the 128-bit access that holds it, and the
+    // wave's first chunk of the row counted from the chunk that holds that key (see the forward kernel)
     int lo = 0;
     if constexpr (kBnd) lo = max((int)pos.i - a.window, 0);
     const int lo8 = lo & ~(kVec - 1);
+    const int wch = wir + lo / kChunk;
     // kRagged: the row lies one position later on the lanes when it starts on an odd element; the
     // position in front of it stays zero in both tensors and is never stored
     int sh = 0;
     if constexpr (kRag) sh = ragged_shift(a.in0, pos.row, sk);
-    const int voff = lane * 16 + wir * kChunk * 2 - 2 * sh;  // the range check ignores a scalar offset
+    const int voff = lane * 16 + wch * kChunk * 2 - 2 * sh;  // the range check ignores a scalar offset
     const bool head = kRag && sh != 0 && wir == 0;  // wave-uniform: this wave holds the row start
     const bool first_lane = head && lane == 0;      // its first access would begin in front of the row
     DropoutArgs drop = a.drop;
@@ -563,6 +584,12 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
             }
         }
     }
+    if constexpr (kBnd) {
+        // the zeros of the chunks that no wave holds.  dx may alias dy: those chunks lie outside the
+        // band, where nothing is read
+        const rsrc_t rz = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, pos.store ? (uint32_t)sk * 2u : 0u);
+        band_zero_fill<kStNt, NCH, WPR>(rz, lo / kChunk, sk, wir, lane);
+    }
     {
         // dx may alias dy: a row is read and written by the same waves only, reads first
         const int len = pos.len;
@@ -573,7 +600,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         uint32_t kb[NCH];  // keep bits of the lane's 8 columns per chunk (kDropout)
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;
+            const int c0 = (wch + WPR * c) * kChunk;
             kb[c] = 0xffu;
             if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 const int col = c0 + lane * kVec - sh;  // first column of the lane
@@ -615,7 +642,7 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_bwd_kernel(SoftmaxArg
         const rsrc_t rdx = make_rsrc(dx, pos.store ? (uint32_t)sk * 2u : 0u);
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-            const int c0 = (wir + WPR * c) * kChunk;
+            const int c0 = (wch + WPR * c) * kChunk;
             u32x4 o = u32x4{0, 0, 0, 0};
             if (c0 < plen && (!kBnd || c0 + kChunk > lo)) {
                 float gv[8], pv[8];
