@@ -131,7 +131,10 @@ def test_sliding_window_sizes(device, s, w, dtype):
     check_window(device, 3 if s <= 2056 else 1, s, w, dtype, 0.125, seed=s + w)
 
 
-@pytest.mark.parametrize("s,w", [(10240, 4096), (12288, 511), (13312, 4096), (16384, 8192), (20000, 4096), (28672, 1000), (32768, 4096)])
+# (the kernel shape goes by the chunks a band can touch, w / 512 + 2, capped by the row's: narrow windows on long
+# rows take few waves per row, the last three cases the 16-wave shapes with 2, 3 and 4 chunks per wave)
+@pytest.mark.parametrize("s,w", [(10240, 4096), (12288, 511), (13312, 4096), (16384, 8192), (20000, 4096), (28672, 1000), (32768, 4096),
+                                 (16384, 12288), (20000, 16384), (28672, 26000)])
 def test_sliding_window_very_long_rows(device, s, w):
     for dtype in DTYPES:
         check_very_long_window(device, s, w, dtype)
