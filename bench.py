@@ -28,8 +28,8 @@ The LAST line of stdout is one compact ASCII JSON object (under 6 KB):
 
 --studies adds the measurements around the table (fused dropout, bias and ALiBi variants, sliding-window
 masks, other head sizes, ragged lengths, a scan over the row lengths, the unfused torch branches on this GPU,
-the Python modules against the C-ABI, a plain copy) and writes them to
-gpurun_out/bench_studies.json; none of them runs by default and none enters the line.
+the Python modules against the C-ABI, a plain copy) and writes them to the
+JSON file STUDIES_PATH names; none of them runs by default and none enters the line.
 
 The oracle is imported by the CPU-baseline leg only (--no-cpu runs never load it); the inputs
 of the measured launches are built without it.
@@ -67,7 +67,7 @@ def parse():
                     help="run only the table rows / study sections whose name contains this text, or one of "
                          "several texts separated by commas (profiling aid)")
     ap.add_argument("--studies", action="store_true",
-                    help="also run the study sections and write them to gpurun_out/bench_studies.json")
+                    help="also run the study sections and write them to " + os.path.relpath(STUDIES_PATH, ROOT))
     return ap.parse_args()
 
 
@@ -562,7 +562,7 @@ def main():
 
 def run_studies(c):
     """The measurements around the BASELINE table; returns a dict that main() writes to
-    gpurun_out/bench_studies.json.  `c` holds main()'s helpers and the table's rows."""
+    STUDIES_PATH.  `c` holds main()'s helpers and the table's rows."""
     import torch
 
     from gpt_neox_amd import _lib
