@@ -179,7 +179,7 @@ struct SoftmaxCall {
     int launch(bool backward, Mask m, void* stream) const {
         const bool vec = vec_ok && a.sk % kVec == 0;
         int flags = backward ? (features & kDropout) : features;
-        if (!vec && a.sk >= kVec && a.sk < kMaxRegisterRow) flags |= kRagged;
+        if (!vec && a.sk >= kVec && a.sk < kMaxStagedRow) flags |= kRagged;
         const hipError_t e = backward ? launch_softmax_bwd(flags, a, m, dtype, vec, (hipStream_t)stream)
                                       : launch_softmax_fwd(flags, a, m, dtype, vec, (hipStream_t)stream);
         return check_launch(e, what);

@@ -16,7 +16,7 @@ int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)))
 // Launchers: pick the kernel shape for the row length and launch on `stream`.
 // `vec_ok` says that every row starts on a 16-byte boundary (sk % 8 == 0, pointers 16-byte
 // aligned); without it the launchers of a feature set without kRagged use their element-wise
-// kernels, and those with kRagged (8 <= sk <= kMaxRegisterRow) ignore it.
+// kernels, and those with kRagged (8 <= sk < kMaxStagedRow) ignore it.
 // One specialisation per feature set, each in a translation unit of its own: FLAGS combines
 // kAlibi (a.slopes, a.np), kBias (a.bias, a.bias_rows, a.bias_bytes), kDropout (a.drop, and a.out2
 // in the forward pass) and kRagged for the forward pass, kDropout and kRagged for the backward pass.
@@ -52,5 +52,7 @@ hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, 
 
 // Longest row the register-resident kernels take (16 waves x 4 chunks x 512 columns).
 constexpr int kMaxRegisterRow = 16 * 4 * kChunk;
+// Longest row the LDS-staged kernels take (159 KiB of 16-bit values); a ragged row must be shorter.
+constexpr int kMaxStagedRow = 159 * 1024 / 2;
 
 }  // namespace neox

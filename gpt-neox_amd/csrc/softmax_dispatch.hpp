@@ -20,11 +20,10 @@
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
-//   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk <= 32768)
-//                  the same packed and one- to sixteen-wave row kernels with the kRagged flag
+//   ragged rows    (sk % 8 != 0 or pointers not 16-byte aligned; 8 <= sk < 81408)
+//                  the same packed, one- to sixteen-wave row and LDS-staged kernels with the kRagged flag
 //   sliding window (kBand) the one- to sixteen-wave row kernels, aligned rows of 513-32768 columns
-//   anything else  element-wise kernels (ragged rows outside that range, rows beyond 81408
-//                  columns, and rows beyond 32768 columns with ALiBi, bias or dropout)
+//   anything else  element-wise kernels (rows shorter than 8 columns or beyond 81408)
 #pragma once
 
 #include <optional>
@@ -141,28 +140,41 @@ static hipError_t dispatch_short_rows(const SoftmaxArgs& a, hipStream_t st) {
     return dispatch_packed<T, M, BWD, EXTRA>(a, st);
 }
 
+// Rows beyond the register budget, staged in LDS: in half of a CU's LDS when the row fits there,
+// two blocks per CU, else in all of it.  Ragged rows need room for one position more.
+static_assert(kMaxStagedRow == kMaxLdsRow, "the range the callers check is the range of the kernels");
+template <typename T, Mask M, bool BWD, int EXTRA>
+static hipError_t launch_lds(const SoftmaxArgs& a, hipStream_t st) {
+    const int positions = a.sk + ((EXTRA & kRagged) != 0 ? 1 : 0);
+    if (positions > kMaxLdsRow) return hipErrorInvalidValue;  // the caller checks
+    const bool half = positions <= kMaxLdsHalfRow;
+    const dim3 grid(a.rows), block(kLdsThreads);
+    if constexpr (BWD) {
+        // ragged rows with dropout need more than the 64 registers per lane that two blocks on a CU
+        // leave each: all of the LDS, one block per CU, at any length
+        constexpr bool half_fits = EXTRA != (kRagged | kDropout);
+        if constexpr (half_fits) {
+            if (half) {
+                hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 5, kLdsHalf, EXTRA>), grid, block, 0, st, a);
+                return hipGetLastError();
+            }
+        }
+        hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 10, kLdsBytes, EXTRA>), grid, block, 0, st, a);
+    } else {
+        if (half) hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsHalf, EXTRA>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsBytes, EXTRA>), grid, block, 0, st, a);
+    }
+    return hipGetLastError();
+}
+
 // The shapes that need 16-byte aligned rows: element-wise kernels when they are not, LDS-staged
 // and packed kernels.  No value: none of them applies, the row kernels take the call.
 template <typename T, Mask M, bool BWD, int EXTRA>
 static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec_ok, int chunks, hipStream_t st) {
     if (!vec_ok) return launch_generic<T, M, BWD, EXTRA>(a, st);
     if (a.sk > kMaxRegisterRow) {
-        // beyond the register budget: the row is staged in LDS (plain kernels only), in half
-        // of a CU's LDS when it fits there
-        if constexpr (EXTRA == 0) {
-            if (a.sk <= kMaxLdsRow) {
-                const bool half = a.sk <= kMaxLdsHalfRow;
-                const dim3 grid(a.rows), block(kLdsThreads);
-                if constexpr (BWD) {
-                    if (half) hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 5, kLdsHalf>), grid, block, 0, st, a);
-                    else hipLaunchKernelGGL((softmax_bwd_lds_kernel<T, M, 10, kLdsBytes>), grid, block, 0, st, a);
-                } else {
-                    if (half) hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsHalf>), grid, block, 0, st, a);
-                    else hipLaunchKernelGGL((softmax_fwd_lds_kernel<T, M, kLdsBytes>), grid, block, 0, st, a);
-                }
-                return hipGetLastError();
-            }
-        }
+        // beyond the register budget: the row is staged in LDS while it fits there
+        if (a.sk <= kMaxLdsRow) return launch_lds<T, M, BWD, EXTRA>(a, st);
         return launch_generic<T, M, BWD, EXTRA>(a, st);
     }
     if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
@@ -207,7 +219,8 @@ static hipError_t dispatch_rows(const SoftmaxArgs& a, bool vec_ok, hipStream_t s
         if (band_chunks < chunks) chunks = band_chunks;
     } else if constexpr ((EXTRA & kRagged) != 0) {
         // rows at any alignment: the packed kernels up to 512 columns, the row kernels below beyond
-        if (a.sk < kVec || a.sk >= kMaxRegisterRow) return hipErrorInvalidValue;  // the caller checks
+        if (a.sk < kVec || a.sk >= kMaxLdsRow) return hipErrorInvalidValue;  // the caller checks
+        if (a.sk >= kMaxRegisterRow) return launch_lds<T, M, BWD, EXTRA>(a, st);
         if (chunks > 1) {
             // rows of odd length: the row kernels lay those that start on an odd element one
             // position later on their lanes

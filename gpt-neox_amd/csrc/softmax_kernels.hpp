@@ -983,6 +983,13 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
 // backward pass stages the probabilities and keeps the gradient packed in registers.  Each
 // wave stages and re-reads its own chunks only, so the only barriers are those of the
 // reductions.
+//
+// Features (FLAGS): the ALiBi term is a function of the column and is formed again in every
+// pass; a bias tensor is not staged -- the staging area holds one 16-bit value per column --
+// but read again by the second pass, from the caches when the row is still there;
+// dropout regenerates its keep bits where they are used.  Ragged rows (kRagged) are staged by
+// position, columns + sh, like the row kernels lay them over their lanes, with the same
+// fix-ups at the two ends of the row; the staging area then needs room for sk + 1 values.
 // ---------------------------------------------------------------------------------
 constexpr int kLdsWaves = 16;
 constexpr int kLdsThreads = kLdsWaves * kWave;
@@ -1018,178 +1025,333 @@ __device__ __forceinline__ u32x4 stage_masked(const u32x4& raw, uint32_t keep) {
     return u32x4{o[0], o[1], o[2], o[3]};
 }
 
-// BYTES: size of the staging area, at least 2 * sk.
-template <typename T, Mask MASK, int BYTES>
+// What the LDS-staged kernels share: where the block's row lies and how its two ends are handled.
+// Chunk c of the row holds the positions c * 512 .. c * 512 + 511, position = column + sh.
+struct LdsRow {
+    int lane, wib;     // lane of the wave, wave of the block
+    int sh;            // kRagged: 1 if the row lies one position later (it starts on an odd element)
+    int plen;          // the row's columns that take part lie at the positions [sh, plen)
+    bool head;         // wave-uniform: sh != 0 and this wave holds chunk 0
+    bool first_lane;   // the lane whose access to chunk 0 would begin in front of the row
+
+    // byte offset of the lane's 128-bit access to chunk c of a 16-bit row, of its 64-bit access to the mask bytes
+    __device__ __forceinline__ uint32_t off16(int c) const {
+        return (c == 0 && first_lane) ? kOutOfRange : (uint32_t)(c * kChunk * 2 + lane * 16 - 2 * sh);
+    }
+    __device__ __forceinline__ uint32_t off8(int c) const {
+        return (c == 0 && first_lane) ? kOutOfRange : (uint32_t)(c * kChunk + lane * kVec - sh);
+    }
+    __device__ __forceinline__ int pos0(int c) const { return c * kChunk + lane * kVec; }  // the lane's first position
+    // kRagged: what a 128-bit load of chunk c could not fetch -- the columns 0 .. 6 of a row that
+    // lies one position later, and the last element when its dword crosses the row end
+    __device__ __forceinline__ void fix16(u32x4& raw, int c, rsrc_t r, uint32_t tail) const {
+        if (head && c == 0) raw |= ragged_head_load(r, first_lane);
+        if ((c + 1) * kChunk >= plen) ragged_patch16(raw, pos0(c), plen, tail);
+    }
+    // 128-bit store of chunk c of an output row of sk columns, with the same two fix-ups
+    template <bool RAG>
+    __device__ __forceinline__ void store(rsrc_t r, const u32x4& o, int c, int sk) const {
+        buf_st128<true>(r, o, off16(c), 0);
+        if constexpr (RAG) {
+            if (c == 0 && head) ragged_head_store(r, o, first_lane);
+            if (c * kChunk < sk + sh && (c + 1) * kChunk >= sk + sh)
+                ragged_store16(r, o, pos0(c), sk + sh, (uint32_t)(sk - 1) * 2u);
+        }
+    }
+};
+
+template <bool RAG>
+__device__ __forceinline__ LdsRow lds_row(const void* base, const RowPos& pos, int sk) {
+    LdsRow r;
+    r.lane = threadIdx.x & (kWave - 1);
+    r.wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    r.sh = 0;
+    if constexpr (RAG) r.sh = ragged_shift(base, pos.row, sk);
+    r.plen = pos.len + r.sh;
+    r.head = RAG && r.sh != 0 && r.wib == 0;
+    r.first_lane = r.head && r.lane == 0;
+    return r;
+}
+
+// BYTES: size of the staging area, at least 2 * sk (2 * (sk + 1) with kRagged).
+template <typename T, Mask MASK, int BYTES, int FLAGS = 0>
 __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softmax_fwd_lds_kernel(SoftmaxArgs a) {
+    constexpr bool kRag = (FLAGS & kRagged) != 0, kAli = (FLAGS & kAlibi) != 0;
+    constexpr bool kBia = (FLAGS & kBias) != 0, kDrp = (FLAGS & kDropout) != 0;
+    static_assert((FLAGS & ~(kRagged | kAlibi | kBias | kDropout)) == 0, "features only: the memory hints are fixed here");
+    // chunks of a wave whose loads are in flight together, by the registers they take: a block that
+    // has a CU to itself has 128 per lane, two that share one have 64 each -- enough for the 5 chunks
+    // a wave holds of the rows staged in half of the LDS, unless the fix-ups of ragged rows need some
+    // too --, and a bias tensor doubles the registers per chunk
+    constexpr int UN = kBia ? (BYTES <= kLdsHalf ? 2 : 4) : (BYTES <= kLdsHalf ? (kRag ? (kAli ? 3 : 4) : 5) : 8);
+    constexpr int UB = kBia ? UN : 1;  // the same for the pass that fetches nothing but the bias
     __shared__ __align__(16) char staged[BYTES];
     __shared__ float red_max[kLdsWaves];
     __shared__ float red_sum[kLdsWaves];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int sk = a.sk;
     const float ninf = -__builtin_inff();
     const RowPos pos = locate<MASK>(blockIdx.x, a);
-    const int len = pos.len;
-    const int data_chunks = (len + kChunk - 1) / kChunk;  // chunks that hold columns of the row
-    const int all_chunks = (sk + kChunk - 1) / kChunk;
+    const LdsRow lr = lds_row<kRag>(a.in0, pos, sk);
+    const int lane = lr.lane, wib = lr.wib, sh = lr.sh;
+    const int len = pos.len, plen = lr.plen;
+    const int data_chunks = (plen + kChunk - 1) / kChunk;  // chunks that hold columns of the row
+    const int all_chunks = (sk + sh + kChunk - 1) / kChunk;
 
-    const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2,
-                                (uint32_t)((len + kVec - 1) & ~(kVec - 1)) * 2u);
-    rsrc_t rm = rx;
+    // whole 128-bit accesses up to the valid length; a ragged row ends where the next one begins
+    const uint32_t row_bytes = (uint32_t)(kRag ? len : (len + kVec - 1) & ~(kVec - 1)) * 2u;
+    const rsrc_t rx = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2, row_bytes);
+    rsrc_t rm = rx, rb = rx;
     if constexpr (MASK == Mask::Bytes) {
         const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
         rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)len);
     }
-
-    // ---- pass 1: HBM -> LDS, running maximum of the scaled scores
-    float mx = ninf;
-    bool hidden = false;  // wave-uniform: this wave staged a -inf in place of a masked or out-of-row element
-    for (int c0 = wib; c0 < data_chunks; c0 += kLdsWaves * kLdsUnroll) {
-        u32x4 raw[kLdsUnroll];
-        u32x2 mk[kLdsUnroll];
+    if constexpr (kBia) rb = make_rsrc(static_cast<const char*>(a.bias) + (size_t)bias_row(pos.row, a) * sk * 2, row_bytes);
+    uint32_t tail_x = 0, tail_b = 0, tail_m = 0;  // kRagged: what the range check drops at the row end
+    if constexpr (kRag) {
+        tail_x = ragged_tail16(rx, len, sh);
+        if constexpr (kBia) tail_b = ragged_tail16(rb, len, sh);
+        if constexpr (MASK == Mask::Bytes) tail_m = ragged_tail_mask(rm, len, sh);
+    }
+    DropoutArgs drop = a.drop;
+    if constexpr (kDrp) drop = resolve(drop);
+    // ALiBi: scale*(x + slope*(j - i')) = x*scale + slope2*(j - i'), slope2 row-uniform
+    float slope2 = 0.f;
+    if constexpr (kAli) slope2 = a.slopes[(pos.row / (uint32_t)a.sq) % a.np] * a.scale;
+    const int ipos = alibi_row_position<MASK>(pos.i, a);
+    // the scaled scores of a lane's 8 columns from `col` on, from the raw scores and the raw bias
+    auto scores = [&](const float (&xv)[8], const u32x4& braw, int col, float (&t)[8]) {
+        float bv[8];
+        if constexpr (kBia) unpack8<T>(braw, bv);
 #pragma unroll
-        for (int u = 0; u < kLdsUnroll; ++u) {
+        for (int k = 0; k < 8; ++k) {
+            float x = xv[k];
+            if constexpr (kBia) x += bv[k];
+            if constexpr (kAli) t[k] = fmaf(x, a.scale, slope2 * alibi_distance<MASK>(col + k, ipos));
+            else t[k] = x * a.scale;
+        }
+    };
+
+    // ---- pass 1: HBM -> LDS; every lane keeps the running maximum mx of its scaled scores and the
+    // sum of exp2(score - mx), rescaled whenever a chunk raises the maximum, so that the exponentials
+    // are taken while the next loads are under way and no second pass over the row is needed
+    float mx = ninf, sum = 0.f;
+    // the reference point of the exponentials for a maximum m: m, or 0 while nothing is visible yet
+    auto ref_of = [&](float m) { return m == ninf ? 0.f : m; };
+    bool hidden = false;  // wave-uniform: this wave staged a -inf in place of a masked or out-of-row element
+    for (int c0 = wib; c0 < data_chunks; c0 += kLdsWaves * UN) {
+        u32x4 raw[UN], rawb[UN];
+        u32x2 mk[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
             const int c = c0 + u * kLdsWaves;  // wave-uniform; chunks past the data load nothing
-            raw[u] = buf_ld128<true>(rx, c * kChunk * 2 + lane * 16, 0);
-            if constexpr (MASK == Mask::Bytes) mk[u] = buf_ld64(rm, c * kChunk + lane * 8, 0);
+            raw[u] = buf_ld128<true>(rx, lr.off16(c), 0);
+            if constexpr (kBia) rawb[u] = buf_ld128<false>(rb, lr.off16(c), 0);
+            else rawb[u] = u32x4{0, 0, 0, 0};
+            if constexpr (MASK == Mask::Bytes) mk[u] = buf_ld64(rm, lr.off8(c), 0);
+        }
+        if constexpr (kRag && MASK == Mask::Bytes) {
+            if (lr.head && c0 == 0) {
+                const u32x2 hm = ragged_head_mask(rm, lr.first_lane);
+                mk[0].x |= hm.x;
+                mk[0].y |= hm.y;
+            }
         }
 #pragma unroll
-        for (int u = 0; u < kLdsUnroll; ++u) {
+        for (int u = 0; u < UN; ++u) {
             const int c = c0 + u * kLdsWaves;
             if (c < data_chunks) {
-                const int col = c * kChunk + lane * kVec;
-                float v[8];
-                unpack8<T>(raw[u], v);
-                bool plain = (c + 1) * kChunk <= len;  // no lane of the wave crosses the row end
+                const int col = lr.pos0(c) - sh;  // first column of the lane, -1 in front of the row
+                if constexpr (kRag) {
+                    lr.fix16(raw[u], c, rx, tail_x);
+                    if constexpr (kBia) lr.fix16(rawb[u], c, rb, tail_b);
+                    if constexpr (MASK == Mask::Bytes) {
+                        if ((c + 1) * kChunk >= plen) ragged_patch_mask(mk[u], lr.pos0(c), plen, tail_m);
+                    }
+                }
+                float xv[8], t[8];
+                unpack8<T>(raw[u], xv);
+                scores(xv, rawb[u], col, t);
+                // no lane of the wave crosses the row end (or holds the position in front of the row)
+                bool plain = (c + 1) * kChunk <= plen && !(lr.head && c == 0);
                 if constexpr (MASK == Mask::Bytes) plain = plain && (__ballot((mk[u].x | mk[u].y) != 0u) == 0ull);
                 u32x4 keep_raw = raw[u];
-                if (plain) {
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) mx = fmaxf(mx, v[k] * a.scale);
-                } else {
+                if (!plain) {
                     hidden = true;
                     uint32_t keep = 0;
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         bool kept = (col + k) < len;
+                        if constexpr (kRag) kept = kept && (col + k) >= 0;
                         if constexpr (MASK == Mask::Bytes) {
                             const uint32_t w = (k < 4) ? mk[u].x : mk[u].y;
                             kept = kept && (((w >> (8 * (k & 3))) & 0xffu) == 0);
                         }
                         keep |= (kept ? 1u : 0u) << k;
-                        mx = fmaxf(mx, kept ? v[k] * a.scale : ninf);
+                        t[k] = kept ? t[k] : ninf;
                     }
                     keep_raw = stage_masked<T>(raw[u], keep);
                 }
                 *reinterpret_cast<u32x4*>(staged + c * kChunk * 2 + lane * 16) = keep_raw;
+                float top = mx;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) top = fmaxf(top, t[k]);
+                const float ref = ref_of(top);
+                float part = 0.f;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) part += fast_exp2(t[k] - ref);
+                sum = fmaf(sum, fast_exp2(mx - ref), part);
+                mx = top;
             }
         }
     }
-    mx = wave_reduce<OpMax>(mx);
-    if (lane == 0) red_max[wib] = mx;
-    __syncthreads();
-    mx = red_max[0];
+    {
+        // the lanes' sums to the maximum of the wave, the waves' sums to the maximum of the row
+        const float lane_mx = mx;
+        mx = wave_reduce<OpMax>(mx);
+        sum = wave_reduce<OpSum>(sum * fast_exp2(lane_mx - ref_of(mx)));
+        if (lane == 0) {
+            red_max[wib] = mx;
+            red_sum[wib] = sum;
+        }
+        __syncthreads();
+        mx = red_max[0];
 #pragma unroll
-    for (int w = 1; w < kLdsWaves; ++w) mx = fmaxf(mx, red_max[w]);
+        for (int w = 1; w < kLdsWaves; ++w) mx = fmaxf(mx, red_max[w]);
+        sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < kLdsWaves; ++w) sum = fmaf(red_sum[w], fast_exp2(red_max[w] - ref_of(mx)), sum);
+    }
     // a row whose every key is masked: uniform over the sk columns, as the unfused path gives
     const bool all_masked = (MASK == Mask::Bytes) && (mx == ninf);
-
-    // ---- pass 2: sum of the exponentials, from LDS.  Only a wave that staged a -inf looks for them.
-    float sum = 0.f;
-    auto add_chunks = [&](auto with_hidden) {
-        for (int c = wib; c < data_chunks; c += kLdsWaves) {
-            float v[8];
-            unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), v);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const float e = fast_exp2(v[k] * a.scale - mx);
-                sum += (decltype(with_hidden)::value && v[k] == ninf) ? 0.f : e;
-            }
-        }
-    };
-    if (hidden) add_chunks(std::true_type{});
-    else add_chunks(std::false_type{});
-    sum = wave_reduce<OpSum>(sum);
-    if (lane == 0) red_sum[wib] = sum;
-    __syncthreads();
-    sum = red_sum[0];
-#pragma unroll
-    for (int w = 1; w < kLdsWaves; ++w) sum += red_sum[w];
     const float inv = all_masked ? 1.0f / (float)len : 1.0f / sum;
 
-    // ---- pass 3: normalise and store; chunks above the diagonal store zeros
-    const rsrc_t ry = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, (uint32_t)sk * 2u);
-    auto store_chunks = [&](auto with_hidden) {
-        for (int c = wib; c < all_chunks; c += kLdsWaves) {
-            u32x4 o = u32x4{0, 0, 0, 0};
-            if (c < data_chunks) {
-                float v[8];
-                unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), v);
-                const int col = c * kChunk + lane * kVec;
+    // the bias of the chunks c0, c0 + 16, ... for the second pass (kBias)
+    auto load_bias = [&](int c0, u32x4 (&rawb)[UB]) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const float e = fast_exp2(v[k] * a.scale - mx) * inv;
-                    if constexpr (decltype(with_hidden)::value) {
-                        v[k] = (v[k] == ninf) ? 0.f : e;
-                        if (all_masked) v[k] = ((col + k) < len) ? inv : 0.f;
-                    } else {
-                        v[k] = e;
+        for (int u = 0; u < UB; ++u) {
+            if constexpr (kBia) rawb[u] = buf_ld128<false>(rb, lr.off16(c0 + u * kLdsWaves), 0);
+            else rawb[u] = u32x4{0, 0, 0, 0};
+        }
+        if constexpr (kBia && kRag) {
+#pragma unroll
+            for (int u = 0; u < UB; ++u) lr.fix16(rawb[u], c0 + u * kLdsWaves, rb, tail_b);
+        }
+    };
+
+    // ---- pass 2: normalise and store, from LDS; chunks above the diagonal store zeros.  Only a wave
+    // that staged a -inf looks for them.
+    const rsrc_t ry = make_rsrc(static_cast<char*>(a.out) + (size_t)pos.row * sk * 2, (uint32_t)sk * 2u);
+    rsrc_t ry2 = ry;
+    if constexpr (kDrp) ry2 = make_rsrc(static_cast<char*>(a.out2) + (size_t)pos.row * sk * 2, (uint32_t)sk * 2u);
+    auto store_chunks = [&](auto with_hidden) {
+        for (int c0 = wib; c0 < all_chunks; c0 += kLdsWaves * UB) {
+            u32x4 rawb[UB];
+            load_bias(c0, rawb);
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const int c = c0 + u * kLdsWaves;
+                if (c >= all_chunks) continue;
+                u32x4 o = u32x4{0, 0, 0, 0}, o2 = u32x4{0, 0, 0, 0};
+                if (c < data_chunks) {
+                    float xv[8], t[8];
+                    unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), xv);
+                    const int col = lr.pos0(c) - sh;
+                    scores(xv, rawb[u], col, t);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const float e = fast_exp2(t[k] - mx) * inv;
+                        if constexpr (decltype(with_hidden)::value) {
+                            t[k] = (xv[k] == ninf) ? 0.f : e;
+                            if (all_masked) t[k] = ((col + k) < len && (col + k) >= 0) ? inv : 0.f;
+                        } else {
+                            t[k] = e;
+                        }
                     }
+                    o = pack8<T>(t);
+                    if constexpr (kDrp) o2 = dropout8<T>(o, keep_bits_row8<kRag>(drop, pos.row, sk, col), drop.scale);
                 }
-                o = pack8<T>(v);
+                lr.template store<kRag>(ry, o, c, sk);
+                if constexpr (kDrp) lr.template store<kRag>(ry2, o2, c, sk);
             }
-            buf_st128<true>(ry, o, c * kChunk * 2 + lane * 16, 0);
         }
     };
     if (hidden) store_chunks(std::true_type{});
     else store_chunks(std::false_type{});
 }
 
-// NCH: chunks per wave, kLdsWaves * NCH * 512 >= sk; BYTES: size of the staging area, >= 2 * sk.
-template <typename T, Mask MASK, int NCH, int BYTES>
+// NCH: chunks per wave, kLdsWaves * NCH * 512 >= sk (sk + 1 with kRagged); BYTES: size of the
+// staging area, at least twice that many bytes.
+template <typename T, Mask MASK, int NCH, int BYTES, int FLAGS = 0>
 __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softmax_bwd_lds_kernel(SoftmaxArgs a) {
     static_assert(NCH * kLdsWaves * kChunk * 2 >= BYTES, "the waves' chunks must cover the staging area");
+    static_assert((FLAGS & ~(kRagged | kDropout)) == 0, "features only: the memory hints are fixed here");
+    static_assert(FLAGS != (kRagged | kDropout) || BYTES > kLdsHalf, "both features together do not fit 64 registers per lane");
+    constexpr bool kRag = (FLAGS & kRagged) != 0, kDrp = (FLAGS & kDropout) != 0;
+    // chunks of a wave whose probabilities are in flight together: the keep bits need registers too,
+    // of which the kernels that share a CU have 64 per lane
+    constexpr int UN = (kDrp && BYTES <= kLdsHalf) ? 2 : kLdsUnroll;
     __shared__ __align__(16) char staged[BYTES];  // the probabilities of the row
     __shared__ float red_sum[kLdsWaves];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int sk = a.sk;
     const RowPos pos = locate<MASK>(blockIdx.x, a);
-    const int len = pos.len;
-    const int data_chunks = (len + kChunk - 1) / kChunk;
-    const uint32_t bytes = (uint32_t)((len + kVec - 1) & ~(kVec - 1)) * 2u;
+    const LdsRow lr = lds_row<kRag>(a.in0, pos, sk);
+    const int lane = lr.lane, wib = lr.wib, sh = lr.sh;
+    const int len = pos.len, plen = lr.plen;
+    const int data_chunks = (plen + kChunk - 1) / kChunk;
+    const uint32_t bytes = (uint32_t)(kRag ? len : (len + kVec - 1) & ~(kVec - 1)) * 2u;
     const rsrc_t bg = make_rsrc(static_cast<const char*>(a.in0) + (size_t)pos.row * sk * 2, bytes);
     const rsrc_t by = make_rsrc(static_cast<const char*>(a.in1) + (size_t)pos.row * sk * 2, bytes);
+    uint32_t tail_g = 0, tail_p = 0;  // kRagged: what the range check drops at the row end
+    if constexpr (kRag) {
+        tail_g = ragged_tail16(bg, len, sh);
+        tail_p = ragged_tail16(by, len, sh);
+    }
+    DropoutArgs drop = a.drop;
+    if constexpr (kDrp) drop = resolve(drop);
 
     // ---- pass 1: the gradient into registers (chunk wib + 16 u; chunks past the data load
     // nothing), the probabilities into LDS, their dot product on the way
     u32x4 rg[NCH];
+    uint32_t kb[(NCH + 3) / 4];  // kDropout: keep bits of the lane's 8 columns, a byte per chunk
 #pragma unroll
-    for (int u = 0; u < NCH; ++u) rg[u] = buf_ld128<true>(bg, (wib + u * kLdsWaves) * kChunk * 2 + lane * 16, 0);
+    for (int u = 0; u < (NCH + 3) / 4; ++u) kb[u] = 0u;
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) rg[u] = buf_ld128<true>(bg, lr.off16(wib + u * kLdsWaves), 0);
     float dot = 0.f;
 #pragma unroll
-    for (int u0 = 0; u0 < NCH; u0 += kLdsUnroll) {
-        u32x4 rp[kLdsUnroll];
+    for (int u0 = 0; u0 < NCH; u0 += UN) {
+        u32x4 rp[UN];
 #pragma unroll
-        for (int u = 0; u < kLdsUnroll; ++u)
-            if (u0 + u < NCH) rp[u] = buf_ld128<true>(by, (wib + (u0 + u) * kLdsWaves) * kChunk * 2 + lane * 16, 0);
+        for (int u = 0; u < UN; ++u)
+            if (u0 + u < NCH) rp[u] = buf_ld128<true>(by, lr.off16(wib + (u0 + u) * kLdsWaves), 0);
 #pragma unroll
-        for (int u = 0; u < kLdsUnroll; ++u) {
+        for (int u = 0; u < UN; ++u) {
             if (u0 + u >= NCH) continue;
             const int c = wib + (u0 + u) * kLdsWaves;
             if (c < data_chunks) {
-                const int col = c * kChunk + lane * kVec;
+                const int col = lr.pos0(c) - sh;
+                if constexpr (kRag) {
+                    // (the position in front of a row that lies one later stays zero in both tensors)
+                    lr.fix16(rg[u0 + u], c, bg, tail_g);
+                    lr.fix16(rp[u], c, by, tail_p);
+                }
                 float gv[8], pv[8];
                 unpack8<T>(rg[u0 + u], gv);
                 unpack8<T>(rp[u], pv);
                 u32x4 keep = rp[u];
-                if ((c + 1) * kChunk > len) {
+                if ((c + 1) * kChunk > plen) {
                     // the lane at the diagonal may have loaded columns past it
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         if ((col + k) >= len) gv[k] = pv[k] = 0.f;
                     keep = pack8<T>(pv);
                     rg[u0 + u] = pack8<T>(gv);
+                }
+                if constexpr (kDrp) {
+                    const uint32_t bits = keep_bits_row8<kRag>(drop, pos.row, sk, col);
+                    kb[(u0 + u) / 4] |= bits << (8 * ((u0 + u) % 4));
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) gv[k] = ((bits >> k) & 1u) ? gv[k] * drop.scale : 0.f;
                 }
 #pragma unroll
                 for (int k = 0; k < 8; ++k) dot = fmaf(gv[k], pv[k], dot);
@@ -1219,10 +1381,13 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
             unpack8<T>(rg[u], gv);
             unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), pv);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) gv[k] = a.scale * (pv[k] * (gv[k] - dot));  // pv = 0 past the row
+            for (int k = 0; k < 8; ++k) {
+                if constexpr (kDrp) gv[k] = ((kb[u / 4] >> (8 * (u % 4) + k)) & 1u) ? gv[k] * drop.scale : 0.f;
+                gv[k] = a.scale * (pv[k] * (gv[k] - dot));  // pv = 0 past the row
+            }
             o = pack8<T>(gv);
         }
-        buf_st128<true>(rdx, o, c * kChunk * 2 + lane * 16, 0);  // chunks past the row end store nothing
+        lr.template store<kRag>(rdx, o, c, sk);  // chunks past the row end store nothing
     }
 }
 

@@ -60,7 +60,7 @@ def oracle(x, mask, slopes, scale, bias=None):
 
 
 # [b, np, sq, sk]: packed kernels (<= 512 columns; 513-768 and 1025-1536 with a mask tensor), one to
-# sixteen waves per row, ragged rows (sk % 8 != 0), the element-wise kernels (sk < 8, sk > 32768),
+# sixteen waves per row, ragged rows (sk % 8 != 0), the element-wise kernels (sk < 8), rows staged in LDS (sk > 32768),
 # and one-query decode steps
 MASKED_ALIBI_SHAPES = [(2, 3, 8, 8), (1, 4, 40, 40), (2, 2, 136, 136), (1, 6, 512, 512), (1, 2, 640, 640), (2, 2, 1000, 1000),
                        (1, 2, 1280, 1280), (1, 3, 2048, 2048), (1, 2, 2568, 2568), (1, 2, 4104, 4104), (1, 1, 9000, 9000),

@@ -152,7 +152,7 @@ def test_causal_forward(device, shape, dtype):
 
 MASKED_SHAPES = [(2, 3, 5, 8), (2, 2, 9, 40), (1, 3, 16, 136), (2, 2, 8, 512), (2, 2, 16, 1024),
                  (1, 2, 8, 1536), (1, 2, 8, 2048), (1, 1, 4, 4096), (1, 1, 2, 16384), (1, 1, 2, 32768),
-                 (2, 2, 5, 37), (1, 2, 3, 1001), (1, 1, 2, 40000),
+                 (2, 2, 5, 37), (1, 2, 3, 1001), (1, 1, 2, 40000), (1, 1, 2, 81416),  # ... staged in LDS, beyond it
                  (2, 2, 5, 9), (2, 3, 7, 129), (2, 2, 3, 515), (1, 2, 3, 2050), (1, 1, 3, 4099), (1, 1, 2, 9001)]
 
 

@@ -1440,8 +1440,8 @@ def test_lds_staged_causal_rows_in_both_storage_types(device, dtype, s):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("sk", [5, 33000])
-def test_bias_tensor_on_the_element_wise_kernels(device, sk, dtype):
-    # rows shorter than 8 columns, and rows beyond the register budget with a bias tensor
+def test_bias_tensor_on_very_short_and_very_long_rows(device, sk, dtype):
+    # rows shorter than 8 columns (element-wise kernels), and rows beyond the register budget (staged in LDS)
     b, heads, sq = 2, 2, (sk if sk < 8 else 3)
     x = scores((b, heads, sq, sk), dtype, device, sk)
     rpe = normal((1, heads, sq, sk), dtype, device, sk + 1)
