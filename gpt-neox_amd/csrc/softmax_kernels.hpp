@@ -998,6 +998,11 @@ constexpr int kLdsHalf = 79 * 1024;          // two blocks per CU
 constexpr int kMaxLdsRow = kLdsBytes / 2;    // 81408 columns (159 chunks)
 constexpr int kMaxLdsHalfRow = kLdsHalf / 2; // 40448 columns (79 chunks)
 constexpr int kLdsUnroll = 4;                // chunks of a wave whose loads are in flight together
+// Forward: a chunk whose keys are all hidden is staged and stored without per-element work.
+#ifndef NEOX_LDS_BLANK_CHUNKS
+#define NEOX_LDS_BLANK_CHUNKS 1
+#endif
+constexpr bool kLdsBlankChunks = NEOX_LDS_BLANK_CHUNKS != 0;
 
 // Waves per SIMD a kernel with a staging area of `bytes` is compiled for: the register budget
 // that lets as many blocks share a CU as its LDS allows.
@@ -1081,9 +1086,11 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
     static_assert((FLAGS & ~(kRagged | kAlibi | kBias | kDropout)) == 0, "features only: the memory hints are fixed here");
     // chunks of a wave whose loads are in flight together, by the registers they take: a block that
     // has a CU to itself has 128 per lane, two that share one have 64 each -- enough for the 5 chunks
-    // a wave holds of the rows staged in half of the LDS, unless the fix-ups of ragged rows need some
-    // too --, and a bias tensor doubles the registers per chunk
-    constexpr int UN = kBia ? (BYTES <= kLdsHalf ? 2 : 4) : (BYTES <= kLdsHalf ? (kRag ? (kAli ? 3 : 4) : 5) : 8);
+    // a wave holds of the rows staged in half of the LDS, unless mask bytes, the ALiBi term or the
+    // fix-ups of ragged rows need some too --, and a bias tensor doubles the registers per chunk
+    constexpr bool kMsk = MASK == Mask::Bytes;
+    constexpr int kHalfUn = kBia ? (kRag && kAli ? 1 : 2) : kRag ? (kMsk || kAli ? 3 : 4) : kMsk ? (kAli ? 3 : 4) : 5;
+    constexpr int UN = BYTES <= kLdsHalf ? kHalfUn : (kBia ? 4 : 8);
     constexpr int UB = kBia ? UN : 1;  // the same for the pass that fetches nothing but the bias
     __shared__ __align__(16) char staged[BYTES];
     __shared__ float red_max[kLdsWaves];
@@ -1138,6 +1145,7 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
     // the reference point of the exponentials for a maximum m: m, or 0 while nothing is visible yet
     auto ref_of = [&](float m) { return m == ninf ? 0.f : m; };
     bool hidden = false;  // wave-uniform: this wave staged a -inf in place of a masked or out-of-row element
+    uint32_t blank = 0;   // wave-uniform: bit j set = chunk wib + 16 j has no visible key at all
     for (int c0 = wib; c0 < data_chunks; c0 += kLdsWaves * UN) {
         u32x4 raw[UN], rawb[UN];
         u32x2 mk[UN];
@@ -1168,12 +1176,24 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
                         if ((c + 1) * kChunk >= plen) ragged_patch_mask(mk[u], lr.pos0(c), plen, tail_m);
                     }
                 }
+                // no lane of the wave crosses the row end (or holds the position in front of the row)
+                bool plain = (c + 1) * kChunk <= plen && !(lr.head && c == 0);
+                if constexpr (MASK == Mask::Bytes) {
+                    plain = plain && (__ballot((mk[u].x | mk[u].y) != 0u) == 0ull);
+                    if constexpr (kLdsBlankChunks) {
+                        // a chunk with no visible key (the hidden tail of a padded row): nothing but -inf to stage
+                        if (!plain && __ballot(!all_hidden(mk[u])) == 0ull) {
+                            hidden = true;
+                            blank |= 1u << (c / kLdsWaves);
+                            constexpr uint32_t pair = NegInf16<T>::bits * 0x10001u;
+                            *reinterpret_cast<u32x4*>(staged + c * kChunk * 2 + lane * 16) = u32x4{pair, pair, pair, pair};
+                            continue;
+                        }
+                    }
+                }
                 float xv[8], t[8];
                 unpack8<T>(raw[u], xv);
                 scores(xv, rawb[u], col, t);
-                // no lane of the wave crosses the row end (or holds the position in front of the row)
-                bool plain = (c + 1) * kChunk <= plen && !(lr.head && c == 0);
-                if constexpr (MASK == Mask::Bytes) plain = plain && (__ballot((mk[u].x | mk[u].y) != 0u) == 0ull);
                 u32x4 keep_raw = raw[u];
                 if (!plain) {
                     hidden = true;
@@ -1252,7 +1272,8 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
                 const int c = c0 + u * kLdsWaves;
                 if (c >= all_chunks) continue;
                 u32x4 o = u32x4{0, 0, 0, 0}, o2 = u32x4{0, 0, 0, 0};
-                if (c < data_chunks) {
+                // (a chunk with no visible key stores zeros, unless the whole row has none)
+                if (c < data_chunks && (all_masked || ((blank >> (c / kLdsWaves)) & 1u) == 0u)) {
                     float xv[8], t[8];
                     unpack8<T>(*reinterpret_cast<const u32x4*>(staged + c * kChunk * 2 + lane * 16), xv);
                     const int col = lr.pos0(c) - sh;
