@@ -848,10 +848,11 @@ def run_studies(c):
                 ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
                 del s_
             out["evaluation_lengths"] = ragged
-    # Rows beyond the register budget (staged in LDS) with every feature: [2, 4, sq, sk] bf16, 1 GiB of
-    # scores, a padding mask that hides the last tenth of every row; sk = 36864 (two blocks share a CU),
-    # 65536 (a block has a CU to itself) and their ragged neighbours.  Bytes: scores in, probabilities out
-    # (twice with dropout), the mask once per head, the bias where there is one; backward 3 tensors.
+    # Rows beyond the register budget (staged in LDS) with every feature: [2, 4, sq, sk] bf16, 1 GiB per
+    # tensor, three buffer sets taken in turn, a padding mask that hides the last tenth of every row;
+    # sk = 36864 (two blocks share a CU), 65536 (a block has a CU to itself) and their ragged neighbours.
+    # Bytes: scores in, probabilities out (twice with dropout), the mask once, the bias where there is
+    # one; backward 3 tensors.
     if want("staged") and not args.quick:
         with section("staged"):
             staged = []
@@ -862,49 +863,59 @@ def run_studies(c):
                 shape = (Bb, H, q_, n)
                 ne = Bb * H * q_ * n
                 g_ = gen(1300 + n % 7)
-                x = torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 4.0, generator=g_)
-                bias = torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 1.0, generator=g_)
-                g = torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 1.0, generator=g_)
-                y, y2 = torch.empty_like(x), torch.empty_like(x)
+                sets = []
+                for _ in range(3):
+                    t = {"x": torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 4.0, generator=g_),
+                         "bias": torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 1.0, generator=g_),
+                         "g": torch.empty(shape, dtype=dt, device=dev).normal_(0.0, 1.0, generator=g_),
+                         "y": torch.empty(shape, dtype=dt, device=dev), "y2": torch.empty(shape, dtype=dt, device=dev)}
+                    sets.append({k: v.data_ptr() for k, v in t.items()} | {"keep": t})
                 pad = torch.zeros(Bb, 1, q_, n, dtype=torch.bool, device=dev)
                 pad[..., int(0.9 * n):] = True
                 slopes = torch.tensor([2.0 ** (-2.0 * (h + 1)) for h in range(H)], device=dev)
-                mb = H * pad.numel()
-                P = lambda t: t.data_ptr()
+                mb, M_, S_ = pad.numel(), pad.data_ptr(), slopes.data_ptr()
 
-                def fwd(_):
-                    ok(lib.neox_masked_softmax_fwd(P(y), P(x), P(pad), sc, Bb, H, q_, n, Bb, code[dt], stream))
+                def fwd(t):
+                    ok(lib.neox_masked_softmax_fwd(t["y"], t["x"], M_, sc, Bb, H, q_, n, Bb, code[dt], stream))
 
-                def fwd_alibi(_):
-                    ok(lib.neox_masked_softmax_alibi_fwd(P(y), P(x), P(pad), P(slopes), sc, Bb, H, q_, n, Bb, code[dt], stream))
+                def fwd_alibi(t):
+                    ok(lib.neox_masked_softmax_alibi_fwd(t["y"], t["x"], M_, S_, sc, Bb, H, q_, n, Bb, code[dt], stream))
 
-                def fwd_bias(_):
-                    ok(lib.neox_masked_softmax_bias_fwd(P(y), P(x), P(pad), P(bias), None, sc, Bb, H, q_, n, Bb, Bb, code[dt], stream))
+                def fwd_bias(t):
+                    ok(lib.neox_masked_softmax_bias_fwd(t["y"], t["x"], M_, t["bias"], None, sc, Bb, H, q_, n, Bb, Bb, code[dt], stream))
 
-                def fwd_shared(_):
-                    ok(lib.neox_masked_softmax_bias_fwd(P(y), P(x), P(pad), P(bias), None, sc, Bb, H, q_, n, Bb, 1, code[dt], stream))
+                def fwd_shared(t):
+                    ok(lib.neox_masked_softmax_bias_fwd(t["y"], t["x"], M_, t["bias"], None, sc, Bb, H, q_, n, Bb, 1, code[dt], stream))
 
-                def fwd_drop(_):
-                    ok(lib.neox_masked_softmax_dropout_fwd(P(y2), P(y), P(x), P(pad), None, None, 0, sc, p_drop, 7, 0, None,
+                def fwd_drop(t):
+                    ok(lib.neox_masked_softmax_dropout_fwd(t["y2"], t["y"], t["x"], M_, None, None, 0, sc, p_drop, 7, 0, None,
                                                            Bb, H, q_, n, Bb, code[dt], stream))
 
-                def fwd_all(_):
-                    ok(lib.neox_masked_softmax_dropout_fwd(P(y2), P(y), P(x), P(pad), P(slopes), P(bias), Bb, sc, p_drop, 7, 0, None,
+                def fwd_all(t):
+                    ok(lib.neox_masked_softmax_dropout_fwd(t["y2"], t["y"], t["x"], M_, S_, t["bias"], Bb, sc, p_drop, 7, 0, None,
                                                            Bb, H, q_, n, Bb, code[dt], stream))
 
-                def bwd(_):
-                    ok(lib.neox_masked_softmax_bwd(P(y2), P(g), P(y), sc, Bb * H * q_, n, code[dt], stream))
+                def bwd(t):
+                    ok(lib.neox_masked_softmax_bwd(t["y2"], t["g"], t["y"], sc, Bb * H * q_, n, code[dt], stream))
 
-                def bwd_drop(_):
-                    ok(lib.neox_masked_softmax_dropout_bwd(P(y2), P(g), P(y), sc, p_drop, 7, 0, None, Bb * H * q_, n, code[dt], stream))
+                def bwd_drop(t):
+                    ok(lib.neox_masked_softmax_dropout_bwd(t["y2"], t["g"], t["y"], sc, p_drop, 7, 0, None, Bb * H * q_, n, code[dt], stream))
 
+                for t in sets:
+                    fwd(t)  # probabilities for the backward launches
                 tag = f"[{Bb},{H},{q_},{n}] bf16"
                 for name, fn, nbytes in (("fwd", fwd, 4 * ne + mb), ("fwd + ALiBi", fwd_alibi, 4 * ne + mb),
                                          ("fwd + bias", fwd_bias, 6 * ne + mb), ("fwd + bias shared by the samples", fwd_shared, 5 * ne + mb),
                                          ("fwd + dropout", fwd_drop, 6 * ne + mb), ("fwd + ALiBi + bias + dropout", fwd_all, 8 * ne + mb),
                                          ("bwd", bwd, 6 * ne), ("bwd + dropout", bwd_drop, 6 * ne)):
-                    staged.append(row(f"mask-tensor {name} {tag}", nbytes, *time_launches(fn, [None], 20)))
-                del x, bias, g, y, y2, pad
+                    staged.append(row(f"mask-tensor {name} {tag}", nbytes, *time_launches(fn, sets, 21)))
+                # hidden keys scattered over every chunk: no chunk takes a short cut
+                pad.copy_(torch.rand(pad.shape, device=dev, generator=g_) < 0.1)
+                staged.append(row(f"mask-tensor fwd {tag}, a tenth of the keys hidden at random", 4 * ne + mb,
+                                  *time_launches(fwd, sets, 21)))
+                staged.append(row(f"mask-tensor fwd + ALiBi + bias + dropout {tag}, a tenth of the keys hidden at random",
+                                  8 * ne + mb, *time_launches(fwd_all, sets, 21)))
+                del sets, pad
             out["rows_staged_in_lds"] = staged
     # Every kernel family over the row lengths, the shape boundaries of the dispatcher included (one
     # length at and one just above each power of two): % of the HBM peak by algorithmic bytes, fp16,
