@@ -14,7 +14,7 @@ import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(_CSRC, "libneox_fused.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 NEOX_F16, NEOX_BF16, NEOX_F32 = 0, 1, 2
 _DTYPE_CODE = {torch.float16: NEOX_F16, torch.bfloat16: NEOX_BF16, torch.float32: NEOX_F32}
@@ -63,6 +63,12 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
          _vp],
     ),
+    "neox_masked_softmax_ends_fwd": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
+         _vp],
+    ),
+    "neox_mask_scan": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "neox_masked_softmax_dropout_bwd": (
         ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _vp]
     ),

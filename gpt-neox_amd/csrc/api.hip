@@ -142,6 +142,15 @@ struct SoftmaxCall {
         a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
         features |= kBias;
     }
+    // where the visible keys of every mask row end, int32 [mask_b * sq]; null = no hint
+    void row_ends(const int32_t* ends) {
+        if (status || !ends) return;
+        if (!aligned(ends, 4)) {
+            status = fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+            return;
+        }
+        a.row_end = ends;
+    }
     // ALiBi slopes, fp32 [np]
     void alibi(const float* slopes, int np) {
         if (status) return;
@@ -281,6 +290,25 @@ int neox_causal_softmax_bwd(void* dx, const void* dy, const void* y, float scale
     if (c.status) return c.status;
     c.backward(dx, dy, y, scale);
     return c.launch(true, Mask::Causal, stream);
+}
+
+int neox_masked_softmax_ends_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask, const int32_t* row_end,
+                                 const float* alibi_slopes, const void* bias, int32_t bias_b, float scale, float p,
+                                 uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                 int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                 int32_t dtype, void* stream) {
+    // y_drop: null = no dropout, and p, seed, offset and device_state are not looked at
+    SoftmaxCall c("neox_masked_softmax_ends_fwd", dtype, {y, x, y_drop ? y_drop : y}, mask);
+    if (y_drop) c.second_output(y_drop, y);
+    c.head_rows(b, np, sq, sk);
+    c.mask(mask, b, np, mask_b);
+    c.row_ends(row_end);
+    if (alibi_slopes) c.alibi(alibi_slopes, np);
+    if (bias) c.bias(bias, b, np, bias_b);
+    if (y_drop) c.dropout(p, seed, offset, device_state);
+    if (c.status) return c.status;
+    c.forward(y, x, scale);
+    return c.launch(false, Mask::Bytes, stream);
 }
 
 int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,
@@ -452,7 +480,17 @@ int neox_mask_classify(int32_t* record, const uint8_t* mask, int32_t mask_b, int
     if (int e = check_rows((int64_t)mask_b * (sq < 1 ? 0 : sq), sq, sk, what)) return e;
     if (sq != sk) return fail(NEOX_ERR_BAD_SHAPE, "%s: sq=%d and sk=%d must be equal", what, sq, sk);
     if (!aligned(record, 4)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
-    return check_launch(launch_mask_classify(record, mask, (uint32_t)mask_b * (uint32_t)sq, sq, sk, (hipStream_t)stream), what);
+    return check_launch(launch_mask_classify(record, nullptr, mask, (uint32_t)mask_b * (uint32_t)sq, sq, sk, (hipStream_t)stream), what);
+}
+
+int neox_mask_scan(int32_t* record, int32_t* row_end, const uint8_t* mask, int32_t mask_b, int32_t sq, int32_t sk,
+                   void* stream) {
+    static const char* what = "neox_mask_scan";
+    if (!record || !row_end || !mask) return fail(NEOX_ERR_NULL_POINTER, "%s: null pointer", what);
+    if (mask_b < 1) return fail(NEOX_ERR_BAD_SHAPE, "%s: mask_b=%d must be >= 1", what, mask_b);
+    if (int e = check_rows((int64_t)mask_b * (sq < 1 ? 0 : sq), sq, sk, what)) return e;
+    if (!aligned(record, 8) || !aligned(row_end, 4)) return fail(NEOX_ERR_MISALIGNED, "%s: misaligned pointer", what);
+    return check_launch(launch_mask_classify(record, row_end, mask, (uint32_t)mask_b * (uint32_t)sq, sq, sk, (hipStream_t)stream), what);
 }
 
 int neox_get_batch_per_block(int32_t sq, int32_t sk, int32_t b, int32_t np) {

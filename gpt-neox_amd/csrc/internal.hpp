@@ -43,8 +43,10 @@ hipError_t launch_softmax_bwd(int flags, const SoftmaxArgs& a, Mask mask, int dt
 // Sliding-window causal rows (a.window): aligned rows of 513 .. kMaxRegisterRow columns only.
 hipError_t launch_softmax_band_fwd(const SoftmaxArgs& a, int dtype, bool vec_ok, hipStream_t stream);
 hipError_t launch_softmax_band_bwd(const SoftmaxArgs& a, int dtype, bool vec_ok, hipStream_t stream);
-// Folds a mask [rows / sq, 1, sq, sk] into the four-word record described in mask_classify.hip.
-hipError_t launch_mask_classify(int32_t* record, const uint8_t* mask, uint32_t rows, int sq, int sk, hipStream_t stream);
+// Folds a mask [rows / sq, 1, sq, sk] into the record described in mask_classify.hip: four words, or
+// eight together with the rows' visible ends (row_end, [rows]) when that pointer is given.
+hipError_t launch_mask_classify(int32_t* record, int32_t* row_end, const uint8_t* mask, uint32_t rows, int sq, int sk,
+                                hipStream_t stream);
 // cs_dtype: NEOX_F32 or the dtype of q for cos/sin tables, kRopeAngles for fp32 angles in a.cos
 constexpr int kRopeAngles = -1;
 hipError_t launch_rope(const RopeArgs& a, int s, int n_outer, int w, int dtype, int cs_dtype,

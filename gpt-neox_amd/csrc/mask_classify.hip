@@ -6,27 +6,37 @@
 // One wave per mask row finds the number of visible keys, the first and the last one.  The row fits
 // the pattern if the visible keys are the contiguous run [lo, i]; the rows then have to agree on one
 // w with lo = max(0, i - w): a row with lo > 0 fixes w = i - lo, a row with lo = 0 only says w >= i.
-// The wave's first lane folds its row into the four-word record the host reads afterwards.
+// The wave's first lane folds its row into the record the host reads afterwards.
+//
+// The same pass can note where every row's visible keys end (row_end[row] = last visible key + 1, 0
+// for a row without one): the mask-tensor forward kernels take that array as a hint and fetch neither
+// the scores nor the mask bytes of a row's hidden tail -- the padding of a batch of sequences of
+// different lengths, or the upper triangle of a causal mask that a caller combines with something
+// else.  The record then also holds the number of keys the hint saves, so that the caller can tell
+// whether it is worth passing on.
 #include <limits.h>
 
 #include "internal.hpp"
 
 namespace neox {
 
-// record[0]: 1 if some row does not fit the pattern; [1], [2]: smallest and largest i - lo over the rows
-// with lo > 0 (INT_MAX and -1 without such a row); [3]: largest i over the rows with lo = 0 (-1 if none).
-__global__ void mask_classify_init_kernel(int32_t* record) {
+// record[0]: 1 if some row does not fit the pattern (always, if the mask is not square); [1], [2]:
+// smallest and largest i - lo over the rows with lo > 0 (INT_MAX and -1 without such a row); [3]:
+// largest i over the rows with lo = 0 (-1 if none).  `words` = 8: [4], [5] the low and high half of the
+// 64-bit number of hidden keys behind the rows' last visible ones, [6], [7] zero.
+__global__ void mask_classify_init_kernel(int32_t* record, int words, int square) {
     if (threadIdx.x == 0) {
-        record[0] = 0;
+        record[0] = square ? 0 : 1;
         record[1] = INT_MAX;
         record[2] = -1;
         record[3] = -1;
+        for (int k = 4; k < words; ++k) record[k] = 0;
     }
 }
 
 template <bool WIDE>
-__global__ __launch_bounds__(256) void mask_classify_kernel(int32_t* record, const uint8_t* mask, uint32_t rows,
-                                                            int sq, int sk) {
+__global__ __launch_bounds__(256) void mask_classify_kernel(int32_t* record, int32_t* row_end, const uint8_t* mask,
+                                                            uint32_t rows, int sq, int sk) {
     const int lane = threadIdx.x & (kWave - 1);
     const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
     if (row >= rows) return;  // wave-uniform
@@ -67,6 +77,12 @@ __global__ __launch_bounds__(256) void mask_classify_kernel(int32_t* record, con
         last = max(last, __shfl_xor(last, step));
     }
     if (lane != 0) return;
+    if (row_end != nullptr) {
+        row_end[row] = last + 1;
+        if (count != 0 && last + 1 < sk)
+            atomicAdd(reinterpret_cast<unsigned long long*>(record + 4), (unsigned long long)(sk - (last + 1)));
+    }
+    if (sq != sk) return;  // record[0] says so already
     if (count == 0 || last != i || count != last - first + 1) {
         atomicOr(record, 1);
     } else if (first > 0) {
@@ -77,12 +93,13 @@ __global__ __launch_bounds__(256) void mask_classify_kernel(int32_t* record, con
     }
 }
 
-hipError_t launch_mask_classify(int32_t* record, const uint8_t* mask, uint32_t rows, int sq, int sk, hipStream_t st) {
-    hipLaunchKernelGGL(mask_classify_init_kernel, dim3(1), dim3(64), 0, st, record);
+hipError_t launch_mask_classify(int32_t* record, int32_t* row_end, const uint8_t* mask, uint32_t rows, int sq, int sk,
+                                hipStream_t st) {
+    hipLaunchKernelGGL(mask_classify_init_kernel, dim3(1), dim3(64), 0, st, record, row_end ? 8 : 4, sq == sk ? 1 : 0);
     const dim3 grid((rows + 3) / 4), block(256);
     const bool wide = sk % 8 == 0 && (reinterpret_cast<uintptr_t>(mask) & 7u) == 0;
-    if (wide) hipLaunchKernelGGL((mask_classify_kernel<true>), grid, block, 0, st, record, mask, rows, sq, sk);
-    else hipLaunchKernelGGL((mask_classify_kernel<false>), grid, block, 0, st, record, mask, rows, sq, sk);
+    if (wide) hipLaunchKernelGGL((mask_classify_kernel<true>), grid, block, 0, st, record, row_end, mask, rows, sq, sk);
+    else hipLaunchKernelGGL((mask_classify_kernel<false>), grid, block, 0, st, record, row_end, mask, rows, sq, sk);
     return hipGetLastError();
 }
 

@@ -48,6 +48,9 @@ struct SoftmaxArgs {
     uint32_t units_per_piece;
     uint32_t affine_blocks;        // leading blocks that take part: a multiple of 8
     int32_t window;                // kBand kernels: row i sees the keys max(0, i - window) .. i
+    // Mask-tensor forward, optional: per mask row [mask_b * sq], the number of leading keys that can be
+    // visible -- every key from there on is hidden whatever its mask byte says; 0 = the whole row
+    const int32_t* row_end;
 };
 
 enum class Mask { Causal, Bytes, None };
@@ -250,6 +253,15 @@ __device__ __forceinline__ RowPos locate(uint32_t row, const SoftmaxArgs& a) {
     p.row = p.store ? row : a.rows - 1;
     p.i = p.row % (uint32_t)a.sq;
     p.len = (MASK == Mask::Causal) ? min((int)p.i + 1, a.sk) : a.sk;
+    if constexpr (MASK == Mask::Bytes) {
+        // a row whose tail is known to be hidden ends there, like a causal row on its diagonal: the
+        // tail's scores and mask bytes are never fetched (one scalar load, the address is row-uniform)
+        if (a.row_end != nullptr) {
+            const uint32_t mb = a.mask_bcast ? 0u : p.row / a.rows_per_mask_batch;
+            const int end = a.row_end[(size_t)mb * a.sq + p.i];
+            if (end > 0 && end < a.sk) p.len = end;
+        }
+    }
     return p;
 }
 
@@ -339,7 +351,9 @@ __global__ __launch_bounds__(kWave* WPR* RPB) void softmax_fwd_kernel(SoftmaxArg
         const rsrc_t rx = make_rsrc(x, row_bytes);
         if constexpr (MASK == Mask::Bytes) {
             const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
-            const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)pos.len);
+            // (whole 64-bit accesses up to a row end that a hint has moved in front of sk, like the scores)
+            const rsrc_t rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk,
+                                        (uint32_t)(kRag ? pos.len : (pos.len + kVec - 1) & ~(kVec - 1)));
 #pragma unroll
             for (int c = 0; c < NCH; ++c)
                 mk[c] = buf_ld64(rm, (c == 0 && first_lane) ? kOutOfRange : lane * 8 + (wir + c * WPR) * kChunk - sh, 0);
@@ -1110,7 +1124,7 @@ __global__ __launch_bounds__(kLdsThreads, lds_waves_per_simd(BYTES)) void softma
     rsrc_t rm = rx, rb = rx;
     if constexpr (MASK == Mask::Bytes) {
         const uint32_t mb = a.mask_bcast ? 0u : pos.row / a.rows_per_mask_batch;
-        rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)len);
+        rm = make_rsrc(a.mask + ((size_t)mb * a.sq + pos.i) * sk, (uint32_t)(kRag ? len : (len + kVec - 1) & ~(kVec - 1)));
     }
     if constexpr (kBia) rb = make_rsrc(static_cast<const char*>(a.bias) + (size_t)bias_row(pos.row, a) * sk * 2, row_bytes);
     uint32_t tail_x = 0, tail_b = 0, tail_m = 0;  // kRagged: what the range check drops at the row end

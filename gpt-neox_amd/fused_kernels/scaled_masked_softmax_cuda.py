@@ -7,8 +7,9 @@ kernels behind ``neox_masked_softmax_fwd/_bwd``.
 Differences: no ``key_seq_len <= 2048`` / ``query_seq_len > 1`` limits; masked
 scores are excluded (probability exactly 0) instead of being set to -10000; any
 non-zero mask byte masks; ``scale`` stays fp32.
-Additions: ``forward_alibi``, ``forward_bias``, ``forward_dropout`` / ``backward_dropout`` and
-``classify_mask``.
+Additions: ``forward_alibi``, ``forward_bias``, ``forward_dropout`` / ``backward_dropout``,
+``classify_mask``, and ``scan_mask`` with the ``row_end=`` hint of the forward functions: rows whose
+visible keys end early (padding) are not fetched behind that point.
 """
 import torch
 
@@ -43,8 +44,38 @@ def _check_forward(input, mask):
             mask if mask.is_contiguous() else mask.contiguous())
 
 
-def forward(input, mask, scale_factor):
+def _check_row_end(row_end, mask):
+    """``row_end`` as :func:`scan_mask` returns it for ``mask``: int32 ``[mask_b * sq]`` on its device."""
+    if (row_end.dtype != torch.int32 or row_end.dim() != 1 or row_end.numel() != mask.size(0) * mask.size(2)
+            or row_end.device != mask.device):
+        raise RuntimeError("row_end must be an int32 tensor [mask_b * sq] on the mask's device")
+    return row_end if row_end.is_contiguous() else row_end.contiguous()
+
+
+def _forward_ends(input, mask, row_end, scale_factor, slopes=None, bias=None, dropout=None):
+    """The forward pass of any feature set with the hint ``row_end`` (see :func:`scan_mask`);
+    ``dropout``: ``(p, seed, offset, state)`` or None.  Arguments already checked."""
+    b, np_, sq, sk = input.shape
+    row_end = _check_row_end(row_end, mask)
+    softmax_results = torch.empty_like(input)
+    dropped = torch.empty_like(input) if dropout is not None else None
+    if input.numel() != 0:
+        p, seed, offset, state = dropout if dropout is not None else (0.0, 0, 0, None)
+        with _guard(input):
+            _check(_lib_handle().neox_masked_softmax_ends_fwd(
+                dropped.data_ptr() if dropped is not None else None, softmax_results.data_ptr(), input.data_ptr(),
+                mask.data_ptr(), row_end.data_ptr(), slopes.data_ptr() if slopes is not None else None,
+                bias.data_ptr() if bias is not None else None, bias.size(0) if bias is not None else 0,
+                float(scale_factor), float(p), int(seed), int(offset), _state_ptr(state), b, np_, sq, sk,
+                mask.size(0), _code(input.dtype), _stream(input)))
+    return softmax_results if dropout is None else (softmax_results, dropped)
+
+
+def forward(input, mask, scale_factor, row_end=None):
+    """``row_end`` (optional, an addition): the hint of :func:`scan_mask` for this mask."""
     input, mask = _check_forward(input, mask)
+    if row_end is not None:
+        return _forward_ends(input, mask, row_end, scale_factor)
     b, np_, sq, sk = input.shape
     softmax_results = torch.empty_like(input)
     if input.numel() == 0:
@@ -58,7 +89,7 @@ def forward(input, mask, scale_factor):
     return softmax_results
 
 
-def forward_alibi(input, mask, slopes, scale_factor):
+def forward_alibi(input, mask, slopes, scale_factor, row_end=None):
     """Mask-tensor softmax of ``scale * (input + alibi_bias)`` without materialising the bias:
     head h adds ``slopes[h] * min(j - i', 0)`` with ``i' = i + sk - sq``, the matrix the
     reference's ``AliBi`` module adds -- ``-slope * tril(i - j)``, and for a one-query decode step
@@ -67,6 +98,8 @@ def forward_alibi(input, mask, slopes, scale_factor):
     input, mask = _check_forward(input, mask)
     b, np_, sq, sk = input.shape
     slopes = check_slopes(slopes, np_)
+    if row_end is not None:
+        return _forward_ends(input, mask, row_end, scale_factor, slopes=slopes)
     softmax_results = torch.empty_like(input)
     if input.numel() == 0:
         return softmax_results
@@ -77,7 +110,7 @@ def forward_alibi(input, mask, slopes, scale_factor):
     return softmax_results
 
 
-def forward_bias(input, mask, bias, scale_factor, slopes=None):
+def forward_bias(input, mask, bias, scale_factor, slopes=None, row_end=None):
     """Mask-tensor softmax of ``scale * (input + bias)`` with the bias read inside the kernel;
     ``bias``: ``[1 or b, np, sq, sk]`` (megatron/model/transformer.py:526-528); ``slopes``
     (optional) adds the ALiBi bias of :func:`forward_alibi` as well.  No counterpart
@@ -87,6 +120,8 @@ def forward_bias(input, mask, bias, scale_factor, slopes=None):
     b, np_, sq, sk = input.shape
     if slopes is not None:
         slopes = check_slopes(slopes, np_)
+    if row_end is not None:
+        return _forward_ends(input, mask, row_end, scale_factor, slopes=slopes, bias=bias)
     softmax_results = torch.empty_like(input)
     if input.numel() == 0:
         return softmax_results
@@ -114,7 +149,7 @@ def backward(output_grads, softmax_results, scale_factor):
     return output_grads
 
 
-def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias=None, slopes=None):
+def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias=None, slopes=None, row_end=None):
     """Mask-tensor softmax and the attention dropout that follows it, in one kernel.
 
     Returns ``(softmax_results, dropped)``: the probabilities as :func:`forward` gives them
@@ -131,6 +166,9 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias
     b, np_, sq, sk = input.shape
     if slopes is not None:
         slopes = check_slopes(slopes, np_)
+    if row_end is not None:
+        return _forward_ends(input, mask, row_end, scale_factor, slopes=slopes, bias=bias,
+                             dropout=(p, seed, offset, state))
     softmax_results = torch.empty_like(input)
     dropped = torch.empty_like(input)
     if input.numel() == 0:
@@ -180,10 +218,42 @@ def classify_mask(mask):
     return record
 
 
+def scan_mask(mask):
+    """:func:`classify_mask` for a mask ``[mask_b, 1, sq, sk]`` of any shape, which also notes where
+    every row's visible keys end.  Returns ``(record, row_end)`` on the mask's device: eight int32 --
+    the first four as :func:`classify_mask` gives them, then the 64-bit number of hidden keys behind
+    the rows' last visible ones (see :func:`hidden_tail_keys`) -- and int32 ``[mask_b * sq]``, the
+    ``row_end=`` hint of the forward functions (last visible key + 1; 0 for a row with none).
+    Asynchronous like every call.  No counterpart in the reference."""
+    if mask.dim() != 4 or mask.size(1) != 1:
+        raise RuntimeError("mask must have shape [mask_b, 1, sq, sk]")
+    if mask.dtype not in _MASK_TYPES:
+        raise RuntimeError("mask must be a bool or uint8 tensor")
+    _lib.require_gpu(mask)
+    if not mask.is_contiguous():
+        mask = mask.contiguous()
+    record = torch.empty(8, dtype=torch.int32, device=mask.device)
+    row_end = torch.empty(mask.size(0) * mask.size(2), dtype=torch.int32, device=mask.device)
+    if row_end.numel() == 0 or mask.size(3) == 0:
+        record.copy_(torch.tensor([1, 2**31 - 1, -1, -1, 0, 0, 0, 0], dtype=torch.int32))
+        return record, row_end.zero_()
+    with _guard(mask):
+        _check(_lib_handle().neox_mask_scan(record.data_ptr(), row_end.data_ptr(), mask.data_ptr(), mask.size(0),
+                                            mask.size(2), mask.size(3), _stream(mask)))
+    return record, row_end
+
+
+def hidden_tail_keys(record):
+    """The number of keys that the ``row_end`` hint of :func:`scan_mask` saves: the sum over the
+    mask rows of ``sk - row_end`` (rows without a visible key not counted), from the eight numbers
+    of the record."""
+    return (int(record[4]) & 0xFFFFFFFF) | ((int(record[5]) & 0xFFFFFFFF) << 32)
+
+
 def decode_mask_record(record):
-    """What four numbers of :func:`classify_mask` say: ``"causal"``, a sliding-window width (int),
-    or False for any other mask."""
-    bad, wmin, wmax, top = (int(v) for v in record)
+    """What the (first) four numbers of :func:`classify_mask` / :func:`scan_mask` say: ``"causal"``, a
+    sliding-window width (int), or False for any other mask."""
+    bad, wmin, wmax, top = (int(v) for v in record[:4])
     if bad:
         return False
     if wmax < 0:

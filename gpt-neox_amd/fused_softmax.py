@@ -92,30 +92,42 @@ def _recall(ctx):
 
 class _MaskVerdict:
     """One remembered mask region: the storage it lives in (weakly), the version counter it had,
-    and the verdict -- ``"causal"``, a sliding-window width (int) or False for any other mask; None
-    while the device-side classification is still running (then ``pending`` holds the pinned
-    result slot and the event that follows the copy)."""
+    and what is known about it -- ``verdict``: ``"causal"``, a sliding-window width (int) or False for
+    any other mask; ``ends``: where every row's visible keys end (the ``row_end`` hint of the
+    mask-tensor kernels, a device tensor) if that saves a sixteenth of the keys or more, else None.
+    Both are None while the device-side scan is still running (then ``pending`` holds the pinned
+    result slot, the event that follows the copy, the hint and the number of keys of the mask)."""
 
-    __slots__ = ("storage", "version", "verdict", "pending")
+    __slots__ = ("storage", "version", "verdict", "ends", "pending")
 
     def __init__(self, storage, version, verdict=None, pending=None):
         self.storage = weakref.ref(storage)
         self.version = version
         self.verdict = verdict
+        self.ends = None
         self.pending = pending
 
     def poll(self, wait):
         """The verdict if it is known by now.  ``wait``: True blocks until it is, False asks the
         event, None does not touch the event at all (for use while a HIP graph is captured)."""
         if self.verdict is None and self.pending is not None and wait is not None:
-            slot, event = self.pending
+            slot, event, ends, keys = self.pending
             if wait:
                 event.synchronize()
             if wait or event.query():
                 # host memory, the copy has finished: no synchronisation
-                self.verdict = _masked_ext.decode_mask_record(slot.tolist())
+                record = slot.tolist()
+                self.verdict = _masked_ext.decode_mask_record(record)
+                # the kernels that read no mask serve the causal kinds; for the others the hint is
+                # kept when it spares the forward pass a sixteenth of its keys or more
+                if self.verdict is False and 16 * _masked_ext.hidden_tail_keys(record) >= keys:
+                    self.ends = ends
                 self.pending = None
         return self.verdict
+
+    def facts(self, wait):
+        """``(verdict, ends)``, or None while they are on their way."""
+        return None if self.poll(wait) is None else (self.verdict, self.ends)
 
 
 class _CausalMaskMemo:
@@ -131,7 +143,9 @@ class _CausalMaskMemo:
     ``.data`` or from outside torch bumps no counter and is not seen.)
 
     The classification is one kernel on the mask's device and stream that reads the mask once
-    (``neox_mask_classify``), followed by a 16-byte copy into pinned memory and an event.
+    (``neox_mask_scan``; it also notes where every row's visible keys end, the hint that spares the
+    mask-tensor kernels the hidden tail of a padded row), followed by a 32-byte copy into pinned
+    memory and an event.
     ``classify(mask, wait=True)`` waits for it (one host synchronisation per new mask); with
     ``wait=False`` it returns None while the result is on its way and the caller uses a kernel
     that is right for any mask in the meantime."""
@@ -161,12 +175,17 @@ class _CausalMaskMemo:
         hit = self._entry(mask)
         return None if hit is None else hit.poll(wait)
 
+    def lookup_facts(self, mask, wait=False):
+        """``(verdict, ends)`` likewise."""
+        hit = self._entry(mask)
+        return None if hit is None else hit.facts(wait)
+
     def _result_slot(self, entry):
-        """Four pinned host words for the record of ``entry``.  The slots are handed out in turn; an
+        """Eight pinned host words for the record of ``entry``.  The slots are handed out in turn; an
         entry that still waits for the slot's previous content reads it first (its copy finished
         long ago), so a slot is never overwritten under an entry that has not looked yet."""
         if self._slots is None:
-            self._slots = torch.zeros(256, 4, dtype=torch.int32, pin_memory=True)
+            self._slots = torch.zeros(256, 8, dtype=torch.int32, pin_memory=True)
             self._slot_owner = [None] * self._slots.shape[0]
         self._next_slot = (self._next_slot + 1) % self._slots.shape[0]
         owner = self._slot_owner[self._next_slot]
@@ -194,27 +213,36 @@ class _CausalMaskMemo:
 
     def classify(self, mask, wait=True):
         """``"causal"``, a window width, False, or None (still running and ``wait`` is False)."""
+        return self._scan(mask).poll(wait)
+
+    def facts(self, mask, wait=True):
+        """``(verdict, ends)`` of ``_MaskVerdict``, or None (still running and ``wait`` is False)."""
+        return self._scan(mask).facts(wait)
+
+    def _scan(self, mask):
+        """The entry of ``mask`` ``[mask_b, 1, sq, sk]``, started now if there is none."""
         hit = self._entry(mask)
         if hit is not None:
-            return hit.poll(wait)
+            return hit
         key, storage = self._key(mask)
         if mask.is_cuda:
-            record = _masked_ext.classify_mask(mask)
+            record, ends = _masked_ext.scan_mask(mask)
             entry = _MaskVerdict(storage, mask._version)
             slot = self._result_slot(entry)
             with torch.cuda.device(mask.device):  # copy and event on the mask's device and stream
                 slot.copy_(record, non_blocking=True)
                 event = torch.cuda.Event()
                 event.record()
-            entry.pending = (slot, event)
+            entry.pending = (slot, event, ends, mask.numel())
         else:
-            entry = _MaskVerdict(storage, mask._version, verdict=self._classify_on_host(mask))
+            square = mask.shape[-1] == mask.shape[-2]
+            entry = _MaskVerdict(storage, mask._version, verdict=self._classify_on_host(mask) if square else False)
         if len(self._entries) >= self._limit:
             self._entries = {k: v for k, v in self._entries.items() if v.storage() is not None}
             if len(self._entries) >= self._limit:
                 self._entries.clear()
         self._entries[key] = entry
-        return entry.poll(wait)
+        return entry
 
     def is_plain_causal(self, mask, wait=True):
         verdict = self.classify(mask, wait)
@@ -319,16 +347,16 @@ class ScaledMaskedSoftmaxBias(torch.autograd.Function):
     ``ScaledUpperTriangMaskedSoftmaxBias``."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, bias, scale, slopes=None):
+    def forward(ctx, inputs, mask, bias, scale, slopes=None, row_end=None):
         scale = _fp32(scale)
         ctx.bias_shape = bias.shape
-        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale, slopes), scale)
+        return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale, slopes, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
         grads = _masked_ext.backward(output_grads, probs, scale)
-        return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None, None
+        return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None, None, None
 
 
 class ScaledMaskedSoftmaxAlibi(torch.autograd.Function):
@@ -339,14 +367,14 @@ class ScaledMaskedSoftmaxAlibi(torch.autograd.Function):
     megatron/model/transformer.py:529-534).  Gradient with respect to ``inputs`` only."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, slopes, scale):
+    def forward(ctx, inputs, mask, slopes, scale, row_end=None):
         scale = _fp32(scale)
-        return _remember(ctx, _masked_ext.forward_alibi(inputs, mask, slopes, scale), scale)
+        return _remember(ctx, _masked_ext.forward_alibi(inputs, mask, slopes, scale, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _masked_ext.backward(output_grads, probs, scale), None, None, None
+        return _masked_ext.backward(output_grads, probs, scale), None, None, None, None
 
 
 class ScaledSlidingWindowSoftmax(torch.autograd.Function):
@@ -373,18 +401,20 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
 
     ``inputs``: ``[b, np, sq, sk]`` fp16/bf16; ``mask``: ``[1 or b, 1, sq, sk]`` bool or
     uint8, non-zero = masked, shared by all heads.  Reference:
-    megatron/model/fused_softmax.py:56-83.
+    megatron/model/fused_softmax.py:56-83.  ``row_end`` (optional, an addition): where every mask
+    row's visible keys end, as ``scaled_masked_softmax_cuda.scan_mask`` finds it -- the forward
+    kernel then fetches nothing behind that point.
     """
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale):
+    def forward(ctx, inputs, mask, scale, row_end=None):
         scale = _fp32(scale)
-        return _remember(ctx, _masked_ext.forward(inputs, mask, scale), scale)
+        return _remember(ctx, _masked_ext.forward(inputs, mask, scale, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _masked_ext.backward(output_grads, probs, scale), None, None
+        return _masked_ext.backward(output_grads, probs, scale), None, None, None
 
 
 class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
@@ -426,11 +456,11 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     ``[1 or b, np, sq, sk]``, differentiable) and ``slopes`` (optional, ALiBi) add to the scores."""
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, p, bias=None, slopes=None):
+    def forward(ctx, inputs, mask, scale, p, bias=None, slopes=None, row_end=None):
         scale = _fp32(scale)
         seed, offset, state = _rng.take_philox_state(inputs.device)
         probs, dropped = _masked_ext.forward_dropout(
-            inputs, mask, scale, p, seed, offset, state, bias=bias, slopes=slopes)
+            inputs, mask, scale, p, seed, offset, state, bias=bias, slopes=slopes, row_end=row_end)
         _remember(ctx, probs, scale)
         ctx.dropout = (p, seed, offset, state)
         ctx.bias_shape = None if bias is None else bias.shape
@@ -441,7 +471,7 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         probs, scale = _recall(ctx)
         grads = _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout)
         wants_bias = ctx.bias_shape is not None and ctx.needs_input_grad[4]
-        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None), None
+        return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None), None, None
 
 
 class SoftmaxFusionTypes(enum.Enum):
@@ -460,18 +490,25 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     scale: multiplier applied before the softmax, or None.
     causal_mask_check (not in the reference): ``"lazy"`` (default) | ``"verify"`` | ``"trust"`` -- how
         the upper_triang fusion treats the mask it is given; see the module text.
+    skip_hidden_tails (not in the reference, default True): a call that the mask-tensor kernel serves
+        tells it where every row's visible keys end, once the scan of the mask has found that this
+        spares a sixteenth of the keys or more (the padding of a batch of sequences of different
+        lengths): the kernel then fetches nothing behind those points.  The scan is the one of
+        ``causal_mask_check`` -- once per mask, never waited for under ``"lazy"``, never made under
+        ``"trust"`` --, and the result is the same bit for bit.
 
     Reference: megatron/model/fused_softmax.py:92-205.
     """
 
     def __init__(self, input_in_fp16, input_in_bf16, fusion_type, mask_func, softmax_in_fp32, scale,
-                 causal_mask_check="lazy"):
+                 causal_mask_check="lazy", skip_hidden_tails=True):
         super().__init__()
         assert fusion_type in list(SoftmaxFusionTypes), f"Invalid fusion type {fusion_type}"
         assert scale is None or softmax_in_fp32, "softmax should be in fp32 when scaled"
         assert causal_mask_check in ("verify", "lazy", "trust"), f"Invalid causal_mask_check {causal_mask_check}"
         # how upper_triang fusion makes sure that the mask is the plain triangle (see the module text)
         self.causal_mask_check = causal_mask_check
+        self.skip_hidden_tails = skip_hidden_tails
 
         self.input_in_fp16 = input_in_fp16
         self.input_in_bf16 = input_in_bf16
@@ -482,7 +519,7 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         self.mask_func = mask_func
         self.softmax_in_fp32 = softmax_in_fp32
         self.scale = scale
-        self._last_mask = None  # (weak reference to the mask of the previous call, its version, its verdict)
+        self._last_mask = None  # (weak reference to the mask of the previous call, its version, (verdict, ends))
         if self.fusion:
             load_fused_kernels()  # ImportError here, not at the first forward
 
@@ -525,17 +562,18 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         if alibi_slopes is not None:
             assert sq == sk or sq == 1, "assumption sq == sk unless at inference time with cache in layer_past with sq == 1"
         causal = self.mask_kind(mask, sq, sk) == "causal"
+        ends = None if causal else self.hidden_tails(mask, b, sq, sk)
         if dropout_p:
             if causal:
                 return ScaledUpperTriangMaskedSoftmaxDropout.apply(input, scale, dropout_p, alibi_slopes, bias)
-            return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p, bias, alibi_slopes)
+            return ScaledMaskedSoftmaxDropout.apply(input, mask, scale, dropout_p, bias, alibi_slopes, ends)
         if bias is not None:
             if causal:
                 return ScaledUpperTriangMaskedSoftmaxBias.apply(input, bias, scale, alibi_slopes)
-            return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale, alibi_slopes)
+            return ScaledMaskedSoftmaxBias.apply(input, mask, bias, scale, alibi_slopes, ends)
         if causal:
             return ScaledUpperTriangMaskedSoftmaxAlibi.apply(input, alibi_slopes, scale)
-        return ScaledMaskedSoftmaxAlibi.apply(input, mask, alibi_slopes, scale)
+        return ScaledMaskedSoftmaxAlibi.apply(input, mask, alibi_slopes, scale, ends)
 
     def is_kernel_available(self, mask, b, np, sq, sk):
         """Whether the fused branch serves this call.
@@ -597,10 +635,11 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
             return ScaledSlidingWindowSoftmax.apply(input, scale, kind)
         # general fusion, or a causal-fusion call whose mask is not (known to be) a causal one -- some
         # other pattern, a step against a key/value cache, a verdict still on its way: what the torch
-        # path computes, from the mask itself
+        # path computes, from the mask itself (and not from the hidden tails of its rows, if it has any)
+        ends = self.hidden_tails(mask, b, sq, sk)
         if not records:
-            return _masked_ext.forward(input, mask, _fp32(scale))
-        return ScaledMaskedSoftmax.apply(input, mask, scale)
+            return _masked_ext.forward(input, mask, _fp32(scale), row_end=ends)
+        return ScaledMaskedSoftmax.apply(input, mask, scale, ends)
 
     def mask_kind(self, mask, sq, sk):
         """What the upper_triang fusion knows about ``mask``: ``"causal"``, a sliding-window width, or
@@ -621,23 +660,37 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         before the capture keeps its verdict, any other is None."""
         if self.causal_mask_check == "trust":
             return "causal"
-        last = self._last_mask
-        if last is not None and last[0]() is mask and last[1] == mask._version:
-            verdict = last[2]  # the tensor object of the previous call, unchanged: no lookup
-        else:
-            verdict = self._classify_mask(mask)
-            if verdict is not None:
-                self._last_mask = (weakref.ref(mask), mask._version, verdict)
+        facts = self._mask_facts(mask)
+        verdict = None if facts is None else facts[0]
         return None if verdict is False else verdict  # (a window of width 0 is a verdict too)
 
-    def _classify_mask(self, mask):
-        """The memo's answer: a verdict, False for any other mask, None while it is on its way."""
-        if (mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != mask.shape[3]
-                or mask.dtype not in (torch.bool, torch.uint8)):
-            return False
+    def hidden_tails(self, mask, b, sq, sk):
+        """The ``row_end`` hint for a call that the mask-tensor kernel serves, or None: switched off,
+        ``"trust"`` (the mask is never read), a mask in another layout than ``[1 or b, 1, sq, sk]``
+        on the GPU, a mask that hides less than a sixteenth of its keys behind its rows' last visible
+        ones, or a scan that has not arrived yet."""
+        if not self.skip_hidden_tails or self.causal_mask_check == "trust":
+            return None
+        if not (mask.is_cuda and self._mask_fits_the_mask_kernel(mask, b, sq, sk)):
+            return None
+        facts = self._mask_facts(mask)
+        return None if facts is None else facts[1]
+
+    def _mask_facts(self, mask):
+        """The memo's answer: ``(verdict, ends)`` -- the verdict False for a mask that is not a causal
+        one --, or None while it is on its way."""
+        last = self._last_mask
+        if last is not None and last[0]() is mask and last[1] == mask._version:
+            return last[2]  # the tensor object of the previous call, unchanged: no lookup
+        if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
+            return (False, None)
         if mask.is_cuda and torch.cuda.is_current_stream_capturing():
-            return _causal_memo.lookup(mask, wait=None)
-        return _causal_memo.classify(mask, wait=self.causal_mask_check == "verify")
+            facts = _causal_memo.lookup_facts(mask, wait=None)
+        else:
+            facts = _causal_memo.facts(mask, wait=self.causal_mask_check == "verify")
+        if facts is not None:
+            self._last_mask = (weakref.ref(mask), mask._version, facts)
+        return facts
 
     def mask_is_plain_causal(self, mask):
         """True if the causal kernel may serve ``mask``; see ``classify_mask``."""

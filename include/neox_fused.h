@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define NEOX_FUSED_ABI_VERSION 3
+#define NEOX_FUSED_ABI_VERSION 4
 
 typedef enum neox_dtype {
     NEOX_F16 = 0,  /* IEEE binary16 */
@@ -220,6 +220,40 @@ int neox_sliding_window_softmax_bwd(void* dx, const void* dy, const void* y, flo
  *   megatron/model/fused_softmax.py:173-179, megatron/utils.py:67-80 (the masks it recognises)
  */
 int neox_mask_classify(int32_t* record, const uint8_t* mask, int32_t mask_b, int32_t sq, int32_t sk, void* stream);
+
+/*
+ * The same pass over a mask tensor [mask_b, 1, sq, sk] of any shape, which also notes where the
+ * visible keys of every row end: row_end[r] (int32 [mask_b * sq], device memory) = last visible key
+ * + 1, 0 for a row without a visible key.  `record` takes eight int32 (8-byte aligned): [0..3] as
+ * neox_mask_classify writes them (record[0] = 1 for a mask that is not square), [4], [5] the low and
+ * the high half of the 64-bit sum of sk - row_end[r] over the rows with a visible key -- the keys
+ * that neox_masked_softmax_ends_fwd does not fetch --, [6], [7] zero.
+ * No counterpart in the reference: its mask-tensor kernel reads every score and mask byte
+ *   megatron/fused_kernels/scaled_masked_softmax.h:123-233
+ */
+int neox_mask_scan(int32_t* record, int32_t* row_end, const uint8_t* mask, int32_t mask_b, int32_t sq, int32_t sk,
+                   void* stream);
+
+/*
+ * Mask-tensor softmax forward that is told where the visible keys of every mask row end and fetches
+ * neither scores nor mask bytes (nor bias) behind that point: row_end[r], int32 [mask_b * sq] as
+ * neox_mask_scan writes it, promises that every key j >= row_end[r] of mask row r is hidden, whatever
+ * the mask byte says; 0 (or a value >= sk, or row_end == NULL) promises nothing for that row.  The
+ * result is that of the plain entry points, bit for bit: y = softmax over the visible keys, exact
+ * zeros elsewhere, a fully hidden row uniform 1/sk.  One entry point for every feature set:
+ * alibi_slopes and bias (with bias_b) are optional as in neox_masked_softmax_bias_fwd; y_drop == NULL
+ * means no dropout (p, seed, offset and device_state are ignored), otherwise the call is
+ * neox_masked_softmax_dropout_fwd with the hint.  The backward pass is the plain one.
+ * Replaces, for masks whose rows end early (the padding of a batch of sequences of different
+ * lengths),
+ *   megatron/model/fused_softmax.py:56-83 (ScaledMaskedSoftmax.forward)
+ *   megatron/fused_kernels/scaled_masked_softmax.h:123-233
+ */
+int neox_masked_softmax_ends_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask, const int32_t* row_end,
+                                 const float* alibi_slopes, const void* bias, int32_t bias_b, float scale, float p,
+                                 uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                 int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                 int32_t dtype, void* stream);
 
 /*
  * Rows-per-block figure the reference's dispatcher predicate consumes; kept for

@@ -353,11 +353,13 @@ def test_public_names_and_signatures_match_the_reference_modules():
     def params(fn):
         return list(inspect.signature(fn).parameters)
 
-    # the reference's positional parameters, plus one optional keyword that defaults to checking without waiting
+    # the reference's positional parameters, plus two optional keywords: checking without waiting, and
+    # not fetching what lies behind a row's last visible key (which changes no result)
     assert params(FusedScaleMaskSoftmax.__init__) == [
         "self", "input_in_fp16", "input_in_bf16", "fusion_type", "mask_func", "softmax_in_fp32", "scale",
-        "causal_mask_check"]
+        "causal_mask_check", "skip_hidden_tails"]
     assert inspect.signature(FusedScaleMaskSoftmax.__init__).parameters["causal_mask_check"].default == "lazy"
+    assert inspect.signature(FusedScaleMaskSoftmax.__init__).parameters["skip_hidden_tails"].default is True
     # the reference's positional parameters, plus three optional additions that default to "off"
     assert params(FusedScaleMaskSoftmax.forward) == ["self", "input", "mask", "alibi_slopes", "dropout_p", "bias"]
     assert inspect.signature(FusedScaleMaskSoftmax.forward).parameters["bias"].default is None
@@ -366,7 +368,8 @@ def test_public_names_and_signatures_match_the_reference_modules():
     assert params(FusedScaleMaskSoftmax.is_kernel_available) == ["self", "mask", "b", "np", "sq", "sk"]
     assert params(FusedScaleMaskSoftmax.get_batch_per_block) == ["sq", "sk", "b", "np"]
     assert params(fused_softmax.ScaledUpperTriangMaskedSoftmax.forward) == ["ctx", "inputs", "scale"]
-    assert params(fused_softmax.ScaledMaskedSoftmax.forward) == ["ctx", "inputs", "mask", "scale"]
+    assert params(fused_softmax.ScaledMaskedSoftmax.forward) == ["ctx", "inputs", "mask", "scale", "row_end"]
+    assert inspect.signature(fused_softmax.ScaledMaskedSoftmax.forward).parameters["row_end"].default is None
     assert [e.name for e in SoftmaxFusionTypes] == ["upper_triang", "general", "none"]
     assert [e.value for e in SoftmaxFusionTypes] == [1, 2, 3]
     pe = positional_embeddings
