@@ -27,7 +27,8 @@ The LAST line of stdout is one compact ASCII JSON object (under 6 KB):
 * min_pct_hbm_peak_over_configs -- the lowest % of HBM peak over those rows.
 
 --studies adds the measurements around the table (fused dropout, bias and ALiBi variants, sliding-window
-masks, other head sizes, ragged lengths, rows staged in LDS with every feature, a scan over the row lengths,
+masks, masks whose rows end early, other head sizes, ragged lengths, rows staged in LDS with every feature,
+a scan over the row lengths,
 the unfused torch branches on this GPU,
 the Python modules against the C-ABI, a plain copy) and writes them to the
 JSON file STUDIES_PATH names; none of them runs by default and none enters the line.
@@ -848,6 +849,60 @@ def run_studies(c):
                 ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
                 del s_
             out["evaluation_lengths"] = ragged
+    # The mask-tensor forward pass told where every row's visible keys end (neox_mask_scan,
+    # neox_masked_softmax_ends_fwd) against the plain one, same buffers, same masks: configs[1] with its
+    # padding mask (lengths 256..1024), a batch padded to 4096 keys, and a causal mask given as a tensor.
+    # Bytes: as for the plain pass (every score in, every probability out, the mask once), so that the
+    # two rows of a pair compare by time.
+    if want("ends"):
+        with section("ends"):
+            ends_rows = []
+
+            def pair(name, Bb, H, q_, n, dt, sc, mask_, nsets, nl):
+                sets_ = []
+                for i in range(nsets):
+                    x_ = torch.empty(Bb, H, q_, n, dtype=dt, device=dev).normal_(0.0, 8.0, generator=gen(1400 + i))
+                    sets_.append({"x": x_, "y": torch.empty_like(x_)})
+                record = torch.empty(8, dtype=torch.int32, device=dev)
+                row_end = torch.empty(mask_.shape[0] * q_, dtype=torch.int32, device=dev)
+                mb_ = mask_.shape[0]
+
+                def scan(_):
+                    ok(lib.neox_mask_scan(record.data_ptr(), row_end.data_ptr(), mask_.data_ptr(), mb_, q_, n, stream))
+
+                def plain(t):
+                    ok(lib.neox_masked_softmax_fwd(t["y"].data_ptr(), t["x"].data_ptr(), mask_.data_ptr(), sc, Bb, H, q_, n, mb_,
+                                                   code[dt], stream))
+
+                def hinted(t):
+                    ok(lib.neox_masked_softmax_ends_fwd(None, t["y"].data_ptr(), t["x"].data_ptr(), mask_.data_ptr(),
+                                                        row_end.data_ptr(), None, None, 0, sc, 0.0, 0, 0, None,
+                                                        Bb, H, q_, n, mb_, code[dt], stream))
+
+                scan(None)
+                plain(sets_[0])
+                want_y = sets_[0]["y"].clone()
+                hinted(sets_[0])
+                torch.cuda.synchronize()
+                tail = (int(record[4]) & 0xFFFFFFFF) | ((int(record[5]) & 0xFFFFFFFF) << 32)
+                nbytes = Bb * H * q_ * n * 4 + mask_.numel()
+                r0 = row(f"{name}: neox_masked_softmax_fwd", nbytes, *time_launches(plain, sets_, nl))
+                r1 = row(f"{name}: neox_masked_softmax_ends_fwd", nbytes, *time_launches(hinted, sets_, nl))
+                r1["bit_equal_to_the_plain_pass"] = bool(torch.equal(sets_[0]["y"], want_y))
+                r1["keys_behind_the_rows_ends_pct"] = round(100.0 * tail / mask_.numel(), 1)
+                r2 = row(f"{name}: neox_mask_scan (once per mask)", mask_.numel(), *time_launches(scan, [None], nl))
+                ends_rows.extend([r0, r1, r2])
+
+            lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(1401))
+            pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
+            pair("cfg2 padded fwd [8,16,1024,1024] fp16", b, heads, sq, sk, dtype, scale, pad, 6, 100)
+            lens = torch.randint(1024, 4097, (4,), device=dev, generator=gen(1402))
+            pad = (torch.arange(4096, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(4, 1, 4096, 4096).contiguous()
+            pair("padded fwd [4,16,4096,4096] bf16", 4, 16, 4096, 4096, torch.bfloat16, 0.125, pad, 2, 30)
+            if not args.quick:
+                pair("causal mask as a tensor [1,32,8192,8192] bf16", 1, 32, 8192, 8192, torch.bfloat16, 128 ** -0.5,
+                     causal_mask(8192), 2, 10)
+            out["rows_that_end_early"] = ends_rows
     # Rows beyond the register budget (staged in LDS) with every feature: [2, 4, sq, sk] bf16, 1 GiB per
     # tensor, three buffer sets taken in turn, a padding mask that hides the last tenth of every row;
     # sk = 36864 (two blocks share a CU), 65536 (a block has a CU to itself) and their ragged neighbours.
