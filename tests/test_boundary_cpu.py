@@ -86,6 +86,25 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     assert b"mask batch dim" in lib.neox_fused_last_error()
     assert lib.neox_masked_softmax_bwd(p, p, p, 1.0, 0, 8, F16, None) == -3
     assert lib.neox_masked_softmax_bwd(p, p, p, 1.0, 8, 8, 7, None) == -2
+    # the mask scan and the forward pass that takes its row ends
+    assert lib.neox_mask_scan(None, p, p, 1, 8, 8, None) == -1
+    assert lib.neox_mask_scan(p, None, p, 1, 8, 8, None) == -1
+    assert lib.neox_mask_scan(p, p, p, 0, 8, 8, None) == -3
+    assert lib.neox_mask_scan(p, p, p, 1, 8, 0, None) == -3
+    assert lib.neox_mask_scan(p + 4, p, p, 1, 8, 8, None) == -5  # the record holds a 64-bit count
+    assert lib.neox_mask_scan(p, p + 2, p, 1, 8, 8, None) == -5
+    ends = lib.neox_masked_softmax_ends_fwd
+    assert ends(None, None, p, p, p, None, None, 0, 1.0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -1
+    assert ends(None, p, p, None, p, None, None, 0, 1.0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -1
+    assert ends(None, p, p, p, p + 2, None, None, 0, 1.0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -5
+    assert ends(None, p, p, p, p, None, None, 0, 1.0, 0.0, 0, 0, None, 2, 2, 8, 8, 3, F16, None) == -3
+    assert ends(None, p, p, p, p, None, None, 0, 1.0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F32, None) == -2
+    assert ends(p, p, p, p, p, None, None, 0, 1.0, 0.5, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -4  # y_drop aliases y
+    assert ends(p + 256, p, p, p, p, None, None, 0, 1.0, 1.5, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -3
+    assert b"dropout probability" in lib.neox_fused_last_error()
+    # without y_drop the dropout arguments are not looked at
+    assert ends(None, p, p, p, p, None, p, 3, 1.0, 1.5, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -3
+    assert b"bias batch dim" in lib.neox_fused_last_error()
     st = (ctypes.c_int64 * 3)(64, 32, 8)
     neg = (ctypes.c_int64 * 3)(64, -32, 8)
     rope = lib.neox_rope_apply
