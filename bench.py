@@ -849,8 +849,8 @@ def run_studies(c):
                 ragged.append(softmax_extras(r, s_[0]["x"][:2], s_[0]["y"][:2], causal_mask(n), sc, dt, B))
                 del s_
             out["evaluation_lengths"] = ragged
-    # The mask-tensor forward pass told where every row's visible keys end (neox_mask_scan,
-    # neox_masked_softmax_ends_fwd) against the plain one, same buffers, same masks: configs[1] with its
+    # The mask-tensor passes told where every row's visible keys end (neox_mask_scan,
+    # neox_masked_softmax_ends_fwd/_bwd) against the plain ones, same buffers, same masks: configs[1] with its
     # padding mask (lengths 256..1024), a batch padded to 4096 keys, and a causal mask given as a tensor.
     # Bytes: as for the plain pass (every score in, every probability out, the mask once), so that the
     # two rows of a pair compare by time.
@@ -862,7 +862,8 @@ def run_studies(c):
                 sets_ = []
                 for i in range(nsets):
                     x_ = torch.empty(Bb, H, q_, n, dtype=dt, device=dev).normal_(0.0, 8.0, generator=gen(1400 + i))
-                    sets_.append({"x": x_, "y": torch.empty_like(x_)})
+                    sets_.append({"x": x_, "y": torch.empty_like(x_), "dx": torch.empty_like(x_),
+                                  "g": torch.empty_like(x_).normal_(0.0, 1.0, generator=gen(1450 + i))})
                 record = torch.empty(8, dtype=torch.int32, device=dev)
                 row_end = torch.empty(mask_.shape[0] * q_, dtype=torch.int32, device=dev)
                 mb_ = mask_.shape[0]
@@ -879,11 +880,25 @@ def run_studies(c):
                                                         row_end.data_ptr(), None, None, 0, sc, 0.0, 0, 0, None,
                                                         Bb, H, q_, n, mb_, code[dt], stream))
 
+                def plain_bwd(t):
+                    ok(lib.neox_masked_softmax_bwd(t["dx"].data_ptr(), t["g"].data_ptr(), t["y"].data_ptr(), sc, Bb * H * q_, n,
+                                                   code[dt], stream))
+
+                def hinted_bwd(t):
+                    ok(lib.neox_masked_softmax_ends_bwd(t["dx"].data_ptr(), t["g"].data_ptr(), t["y"].data_ptr(), row_end.data_ptr(),
+                                                        sc, 0, 0.0, 0, 0, None, Bb, H, q_, n, mb_, code[dt], stream))
+
                 scan(None)
                 plain(sets_[0])
                 want_y = sets_[0]["y"].clone()
+                plain_bwd(sets_[0])
+                want_dx = sets_[0]["dx"].clone()
                 hinted(sets_[0])
+                hinted_bwd(sets_[0])
                 torch.cuda.synchronize()
+                same_dx = bool(torch.equal(sets_[0]["dx"], want_dx))
+                for t in sets_[1:]:
+                    plain(t)  # probabilities for the backward launches
                 tail = (int(record[4]) & 0xFFFFFFFF) | ((int(record[5]) & 0xFFFFFFFF) << 32)
                 nbytes = Bb * H * q_ * n * 4 + mask_.numel()
                 r0 = row(f"{name}: neox_masked_softmax_fwd", nbytes, *time_launches(plain, sets_, nl))
@@ -891,7 +906,11 @@ def run_studies(c):
                 r1["bit_equal_to_the_plain_pass"] = bool(torch.equal(sets_[0]["y"], want_y))
                 r1["keys_behind_the_rows_ends_pct"] = round(100.0 * tail / mask_.numel(), 1)
                 r2 = row(f"{name}: neox_mask_scan (once per mask)", mask_.numel(), *time_launches(scan, [None], nl))
-                ends_rows.extend([r0, r1, r2])
+                bbytes = Bb * H * q_ * n * 6
+                r3 = row(f"{name}: neox_masked_softmax_bwd", bbytes, *time_launches(plain_bwd, sets_, nl))
+                r4 = row(f"{name}: neox_masked_softmax_ends_bwd", bbytes, *time_launches(hinted_bwd, sets_, nl))
+                r4["bit_equal_to_the_plain_pass"] = same_dx
+                ends_rows.extend([r0, r1, r3, r4, r2])
 
             lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(1401))
             pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()

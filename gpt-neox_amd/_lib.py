@@ -68,6 +68,10 @@ SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _f32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
          _vp],
     ),
+    "neox_masked_softmax_ends_bwd": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _f32, _i32, _f32, _u64, _u64, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp],
+    ),
     "neox_mask_scan": (ctypes.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _vp]),
     "neox_masked_softmax_dropout_bwd": (
         ctypes.c_int, [_vp, _vp, _vp, _f32, _f32, _u64, _u64, _vp, _i64, _i32, _i32, _vp]

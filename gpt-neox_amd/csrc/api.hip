@@ -142,6 +142,16 @@ struct SoftmaxCall {
         a.bias_bytes = fits32((uint64_t)bias_b * (uint64_t)np * (uint64_t)a.sq * (uint64_t)a.sk * 2u);
         features |= kBias;
     }
+    // which mask row [mask_b, 1, sq, .] a score row belongs to, for a call that brings no mask tensor
+    void mask_rows(int b, int np, int mask_b) {
+        if (status) return;
+        if (mask_b != 1 && mask_b != b) {
+            status = fail(NEOX_ERR_BAD_SHAPE, "%s: mask batch dim %d must be 1 or b=%d", what, mask_b, b);
+            return;
+        }
+        a.rows_per_mask_batch = (uint32_t)((int64_t)np * a.sq);
+        a.mask_bcast = (mask_b == 1 && b != 1) ? 1 : 0;
+    }
     // where the visible keys of every mask row end, int32 [mask_b * sq]; null = no hint
     void row_ends(const int32_t* ends) {
         if (status || !ends) return;
@@ -309,6 +319,20 @@ int neox_masked_softmax_ends_fwd(void* y_drop, void* y, const void* x, const uin
     if (c.status) return c.status;
     c.forward(y, x, scale);
     return c.launch(false, Mask::Bytes, stream);
+}
+
+int neox_masked_softmax_ends_bwd(void* dx, const void* dy, const void* y, const int32_t* row_end, float scale,
+                                 int32_t dropout, float p, uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                 int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                 int32_t dtype, void* stream) {
+    SoftmaxCall c("neox_masked_softmax_ends_bwd", dtype, {dx, dy, y});
+    c.head_rows(b, np, sq, sk);
+    c.mask_rows(b, np, mask_b);
+    c.row_ends(row_end);
+    if (dropout) c.dropout(p, seed, offset, device_state);
+    if (c.status) return c.status;
+    c.backward(dx, dy, y, scale);
+    return c.launch(true, Mask::None, stream);
 }
 
 int neox_masked_softmax_fwd(void* y, const void* x, const uint8_t* mask, float scale, int32_t b,

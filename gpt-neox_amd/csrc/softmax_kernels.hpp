@@ -48,8 +48,10 @@ struct SoftmaxArgs {
     uint32_t units_per_piece;
     uint32_t affine_blocks;        // leading blocks that take part: a multiple of 8
     int32_t window;                // kBand kernels: row i sees the keys max(0, i - window) .. i
-    // Mask-tensor forward, optional: per mask row [mask_b * sq], the number of leading keys that can be
-    // visible -- every key from there on is hidden whatever its mask byte says; 0 = the whole row
+    // Mask-tensor forward and full-row backward, optional: per mask row [mask_b * sq], the number of
+    // leading keys that can be visible -- every key from there on is hidden whatever its mask byte
+    // says (backward: its probability is zero); 0 = the whole row.  Needs sq, rows_per_mask_batch
+    // and mask_bcast.
     const int32_t* row_end;
 };
 
@@ -253,9 +255,10 @@ __device__ __forceinline__ RowPos locate(uint32_t row, const SoftmaxArgs& a) {
     p.row = p.store ? row : a.rows - 1;
     p.i = p.row % (uint32_t)a.sq;
     p.len = (MASK == Mask::Causal) ? min((int)p.i + 1, a.sk) : a.sk;
-    if constexpr (MASK == Mask::Bytes) {
+    if constexpr (MASK != Mask::Causal) {
         // a row whose tail is known to be hidden ends there, like a causal row on its diagonal: the
-        // tail's scores and mask bytes are never fetched (one scalar load, the address is row-uniform)
+        // tail's scores and mask bytes (backward: its probabilities, all zero, and its gradient) are
+        // never fetched (one scalar load, the address is row-uniform)
         if (a.row_end != nullptr) {
             const uint32_t mb = a.mask_bcast ? 0u : p.row / a.rows_per_mask_batch;
             const int end = a.row_end[(size_t)mb * a.sq + p.i];
@@ -919,6 +922,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
     u32x4 rg[R][C], rp[R][C];
     int len[R];
     constexpr bool kSkip = kSkipHidden && MASK == Mask::None && !kRag;
+    const bool hinted = MASK == Mask::None && a.row_end != nullptr;  // uniform over the launch
     const uint32_t i0 = row0 % (uint32_t)a.sq;  // wave-uniform
 #pragma unroll
     for (int p = 0; p < R; ++p) {
@@ -926,15 +930,27 @@ __global__ __launch_bounds__(256) void softmax_bwd_packed_kernel(SoftmaxArgs a) 
         const uint32_t i = wrap_row(i0 + lr, (uint32_t)a.sq);
         len[p] = (MASK == Mask::Causal) ? min((int)i + 1, sk) : sk;
         if (lr >= rows_here) len[p] = 0;
+        if constexpr (MASK == Mask::None) {
+            // the row is known to end early (see SoftmaxArgs::row_end): neither tensor is fetched behind that
+            if (hinted && lr < rows_here) {
+                const uint32_t row = row0 + lr;
+                const uint32_t mb = a.mask_bcast ? 0u : row / a.rows_per_mask_batch;
+                const int end = a.row_end[(size_t)mb * a.sq + i];
+                if (end > 0 && end < sk) len[p] = end;
+            }
+        }
 #pragma unroll
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
             rp[p][c] = packed_ld<kLdNt>(by, (lr * sk + col) * 2u, col < len[p]);
             if constexpr (!kSkip) rg[p][c] = packed_ld<kLdNt>(bg, (lr * sk + col) * 2u, col < len[p]);
+            else if (hinted) rg[p][c] = packed_ld<kLdNt>(bg, (lr * sk + col) * 2u, col < len[p]);
         }
     }
-    if constexpr (kSkip) {
-        // full rows (after a mask-tensor forward): no gradient for a lane whose 8 probabilities are all zero
+    if (kSkip && !hinted) {
+        // full rows (after a mask-tensor forward): no gradient for a lane whose 8 probabilities are all
+        // zero -- unless the rows' ends are known, which spares both tensors without making one load
+        // wait for the other
 #pragma unroll
         for (int p = 0; p < R; ++p) {
             const uint32_t lr = p * RPP + grp;

@@ -133,9 +133,34 @@ def forward_bias(input, mask, bias, scale_factor, slopes=None, row_end=None):
     return softmax_results
 
 
-def backward(output_grads, softmax_results, scale_factor):
-    """Returns d(input), written into ``output_grads`` itself when it is contiguous."""
+def _backward_ends(output_grads, softmax_results, row_end, scale_factor, dropout=None):
+    """The backward pass with the hint ``row_end`` ``[mask_b * sq]`` (see :func:`scan_mask`): nothing is
+    fetched behind a row's end, where the probabilities are zero.  ``dropout``: ``(p, seed, offset,
+    state)`` of the forward call or None.  Arguments already checked."""
+    b, np_, sq, sk = output_grads.shape
+    if row_end.dtype != torch.int32 or row_end.dim() != 1 or row_end.numel() not in (sq, b * sq) \
+            or row_end.device != output_grads.device:
+        raise RuntimeError("row_end must be an int32 tensor [mask_b * sq] on the gradient's device")
+    if not row_end.is_contiguous():
+        row_end = row_end.contiguous()
+    if output_grads.numel() == 0:
+        return output_grads
+    p, seed, offset, state = dropout if dropout is not None else (0.0, 0, 0, None)
+    grads = output_grads.data_ptr()
+    with _guard(output_grads):
+        _check(_lib_handle().neox_masked_softmax_ends_bwd(
+            grads, grads, softmax_results.data_ptr(), row_end.data_ptr(), float(scale_factor),
+            0 if dropout is None else 1, float(p), int(seed), int(offset), _state_ptr(state),
+            b, np_, sq, sk, row_end.numel() // sq, _code(output_grads.dtype), _stream(output_grads)))
+    return output_grads
+
+
+def backward(output_grads, softmax_results, scale_factor, row_end=None):
+    """Returns d(input), written into ``output_grads`` itself when it is contiguous.  ``row_end``
+    (optional, an addition): the hint of :func:`scan_mask` for the mask of the forward call."""
     output_grads, softmax_results = _grads(output_grads, softmax_results, (4,))
+    if row_end is not None:
+        return _backward_ends(output_grads, softmax_results, row_end, scale_factor)
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads
@@ -183,10 +208,13 @@ def forward_dropout(input, mask, scale_factor, p, seed, offset, state=None, bias
     return softmax_results, dropped
 
 
-def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset, state=None):
+def backward_dropout(output_grads, softmax_results, scale_factor, p, seed, offset, state=None, row_end=None):
     """d(input) from the gradient of ``dropped``; written into ``output_grads`` itself when
-    that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call."""
+    that tensor is contiguous.  ``(p, seed, offset)`` are those of the forward call; ``row_end``
+    (optional) as in :func:`backward`."""
     output_grads, softmax_results = _grads(output_grads, softmax_results, (4,))
+    if row_end is not None:
+        return _backward_ends(output_grads, softmax_results, row_end, scale_factor, (p, seed, offset, state))
     b, np_, sq, sk = output_grads.shape
     if output_grads.numel() == 0:
         return output_grads

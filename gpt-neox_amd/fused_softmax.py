@@ -350,12 +350,13 @@ class ScaledMaskedSoftmaxBias(torch.autograd.Function):
     def forward(ctx, inputs, mask, bias, scale, slopes=None, row_end=None):
         scale = _fp32(scale)
         ctx.bias_shape = bias.shape
+        ctx.row_end = row_end
         return _remember(ctx, _masked_ext.forward_bias(inputs, mask, bias, scale, slopes, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        grads = _masked_ext.backward(output_grads, probs, scale)
+        grads = _masked_ext.backward(output_grads, probs, scale, row_end=ctx.row_end)
         return grads, None, (_bias_gradient(grads, ctx.bias_shape) if ctx.needs_input_grad[2] else None), None, None, None
 
 
@@ -369,12 +370,13 @@ class ScaledMaskedSoftmaxAlibi(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inputs, mask, slopes, scale, row_end=None):
         scale = _fp32(scale)
+        ctx.row_end = row_end
         return _remember(ctx, _masked_ext.forward_alibi(inputs, mask, slopes, scale, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _masked_ext.backward(output_grads, probs, scale), None, None, None, None
+        return _masked_ext.backward(output_grads, probs, scale, row_end=ctx.row_end), None, None, None, None
 
 
 class ScaledSlidingWindowSoftmax(torch.autograd.Function):
@@ -409,12 +411,13 @@ class ScaledMaskedSoftmax(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inputs, mask, scale, row_end=None):
         scale = _fp32(scale)
+        ctx.row_end = row_end
         return _remember(ctx, _masked_ext.forward(inputs, mask, scale, row_end=row_end), scale)
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        return _masked_ext.backward(output_grads, probs, scale), None, None, None
+        return _masked_ext.backward(output_grads, probs, scale, row_end=ctx.row_end), None, None, None
 
 
 class ScaledUpperTriangMaskedSoftmaxDropout(torch.autograd.Function):
@@ -464,12 +467,13 @@ class ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         _remember(ctx, probs, scale)
         ctx.dropout = (p, seed, offset, state)
         ctx.bias_shape = None if bias is None else bias.shape
+        ctx.row_end = row_end
         return dropped
 
     @staticmethod
     def backward(ctx, output_grads):
         probs, scale = _recall(ctx)
-        grads = _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout)
+        grads = _masked_ext.backward_dropout(output_grads, probs, scale, *ctx.dropout, row_end=ctx.row_end)
         wants_bias = ctx.bias_shape is not None and ctx.needs_input_grad[4]
         return grads, None, None, None, (_bias_gradient(grads, ctx.bias_shape) if wants_bias else None), None, None
 

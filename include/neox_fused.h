@@ -243,7 +243,8 @@ int neox_mask_scan(int32_t* record, int32_t* row_end, const uint8_t* mask, int32
  * zeros elsewhere, a fully hidden row uniform 1/sk.  One entry point for every feature set:
  * alibi_slopes and bias (with bias_b) are optional as in neox_masked_softmax_bias_fwd; y_drop == NULL
  * means no dropout (p, seed, offset and device_state are ignored), otherwise the call is
- * neox_masked_softmax_dropout_fwd with the hint.  The backward pass is the plain one.
+ * neox_masked_softmax_dropout_fwd with the hint.  The backward pass is the plain one, or
+ * neox_masked_softmax_ends_bwd.
  * Replaces, for masks whose rows end early (the padding of a batch of sequences of different
  * lengths),
  *   megatron/model/fused_softmax.py:56-83 (ScaledMaskedSoftmax.forward)
@@ -252,6 +253,21 @@ int neox_mask_scan(int32_t* record, int32_t* row_end, const uint8_t* mask, int32
 int neox_masked_softmax_ends_fwd(void* y_drop, void* y, const void* x, const uint8_t* mask, const int32_t* row_end,
                                  const float* alibi_slopes, const void* bias, int32_t bias_b, float scale, float p,
                                  uint64_t seed, uint64_t offset, const uint64_t* device_state,
+                                 int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
+                                 int32_t dtype, void* stream);
+
+/*
+ * The backward pass of the mask-tensor softmax with the same hint: behind row_end[r] the probabilities
+ * are zero, so neither they nor the incoming gradient are fetched there, and dx is zero.  The result is
+ * that of neox_masked_softmax_bwd -- or, with dropout != 0, of neox_masked_softmax_dropout_bwd with
+ * (p, seed, offset, device_state) of the forward call -- bit for bit.  [b, np, sq, sk] and mask_b say
+ * which entry of row_end belongs to a row; dx may alias dy.
+ * Replaces, for masks whose rows end early,
+ *   megatron/model/fused_softmax.py:56-83 (ScaledMaskedSoftmax.backward)
+ *   megatron/fused_kernels/scaled_masked_softmax.h:240-335
+ */
+int neox_masked_softmax_ends_bwd(void* dx, const void* dy, const void* y, const int32_t* row_end, float scale,
+                                 int32_t dropout, float p, uint64_t seed, uint64_t offset, const uint64_t* device_state,
                                  int32_t b, int32_t np, int32_t sq, int32_t sk, int32_t mask_b,
                                  int32_t dtype, void* stream);
 

@@ -105,6 +105,15 @@ def test_argument_errors_are_reported_without_touching_the_gpu():
     # without y_drop the dropout arguments are not looked at
     assert ends(None, p, p, p, p, None, p, 3, 1.0, 1.5, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -3
     assert b"bias batch dim" in lib.neox_fused_last_error()
+    endsb = lib.neox_masked_softmax_ends_bwd
+    assert endsb(p, None, p, p, 1.0, 0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -1
+    assert endsb(p, p, p, p + 2, 1.0, 0, 0.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -5
+    assert endsb(p, p, p, p, 1.0, 0, 0.0, 0, 0, None, 2, 2, 8, 8, 3, F16, None) == -3
+    assert b"mask batch dim" in lib.neox_fused_last_error()
+    assert endsb(p, p, p, p, 1.0, 0, 7.0, 0, 0, None, 2, 2, 8, 0, 2, F16, None) == -3  # p is not looked at
+    assert b"sk=0" in lib.neox_fused_last_error()
+    assert endsb(p, p, p, p, 1.0, 1, 7.0, 0, 0, None, 2, 2, 8, 8, 2, F16, None) == -3
+    assert b"dropout probability" in lib.neox_fused_last_error()
     st = (ctypes.c_int64 * 3)(64, 32, 8)
     neg = (ctypes.c_int64 * 3)(64, -32, 8)
     rope = lib.neox_rope_apply

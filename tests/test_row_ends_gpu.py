@@ -1,11 +1,11 @@
-"""The hint that tells the mask-tensor forward kernels where every row's visible keys end
-(neox_mask_scan, neox_masked_softmax_ends_fwd), through the C-ABI.
+"""The hint that tells the mask-tensor kernels where every row's visible keys end
+(neox_mask_scan, neox_masked_softmax_ends_fwd, neox_masked_softmax_ends_bwd), through the C-ABI.
 
 What is pinned: the scan against plain torch (last visible key + 1 per mask row, the number of
-keys behind those points, the causal verdict in the first four words); the hinted forward pass
-bit-equal to the plain one for every kernel family, mask pattern and feature set -- it computes the
-same numbers in the same order and only fetches less --, so it inherits the plain pass's parity with
-the oracle (checked once more here against the fp32 expression); keys behind a row's end count as
+keys behind those points, the causal verdict in the first four words); the hinted forward and
+backward passes bit-equal to the plain ones for every kernel family, mask pattern and feature set --
+they compute the same numbers in the same order and only fetch less --, so they inherit the plain
+passes' parity with the oracle (checked once more here against the fp32 expression); keys behind a row's end count as
 hidden whatever their mask bytes say; and the Python module passing the hint along by itself, without
 a host synchronisation, once it has seen that a mask hides enough.
 """
@@ -113,6 +113,40 @@ def test_every_feature_set_takes_the_hint(device, shape, dtype):
         y, dropped = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, row_end=row_end, **extra)
         y0, dropped0 = masked_ext.forward_dropout(x, mask, scale, p, seed, offset, **extra)
         assert torch.equal(y, y0) and torch.equal(dropped, dropped0)
+
+
+BWD_SHAPES = [(2, 3, 9, 40), (2, 2, 8, 384), (2, 2, 16, 512), (3, 2, 8, 1024), (2, 2, 6, 1536), (2, 2, 8, 2048),
+              (1, 2, 6, 4096), (2, 1, 4, 8192), (1, 2, 3, 20000), (2, 1, 3, 33000), (1, 1, 3, 50008), (2, 2, 5, 1001),
+              (1, 2, 3, 9001), (2, 2, 4, 5)]
+
+
+@pytest.mark.parametrize("kind", ["padding", "random tail"])
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+def test_hinted_backward_equals_the_plain_one(device, shape, kind):
+    b, heads, sq, sk = shape
+    dtype = DTYPES[(sk + len(kind)) % 2]
+    mask = masks(kind, b, sq, sk, device, 3 * sk + sq)
+    _, row_end = masked_ext.scan_mask(mask)
+    x = torch.empty(shape, dtype=dtype, device=device).normal_(0.0, 4.0, generator=gen(device, sk))
+    g = torch.empty(shape, dtype=dtype, device=device).normal_(0.0, 1.0, generator=gen(device, sk + 1))
+    y = masked_ext.forward(x, mask, 0.25)
+    plain = masked_ext.backward(g.clone(), y, 0.25)
+    buf = g.clone()
+    hinted = masked_ext.backward(buf, y, 0.25, row_end=row_end)
+    assert hinted.data_ptr() == buf.data_ptr()  # in place, like the plain pass
+    assert torch.equal(hinted, plain)
+    hidden = mask.expand(shape) & ~mask.all(-1, keepdim=True).expand(shape)
+    assert (hinted[hidden] == 0).all()
+    p, seed, offset = 0.25, 17, 8
+    yd, _ = masked_ext.forward_dropout(x, mask, 0.25, p, seed, offset)
+    assert torch.equal(masked_ext.backward_dropout(g.clone(), yd, 0.25, p, seed, offset, row_end=row_end),
+                       masked_ext.backward_dropout(g.clone(), yd, 0.25, p, seed, offset))
+    # the mask of the first sample for all of them
+    _, end1 = masked_ext.scan_mask(mask[:1])
+    y1 = masked_ext.forward(x, mask[:1], 0.25)
+    assert torch.equal(masked_ext.backward(g.clone(), y1, 0.25, row_end=end1), masked_ext.backward(g.clone(), y1, 0.25))
+    with pytest.raises(RuntimeError, match="row_end"):
+        masked_ext.backward(g.clone(), y, 0.25, row_end=row_end[:-1])
 
 
 def test_keys_behind_a_rows_end_count_as_hidden(device):
