@@ -646,12 +646,19 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         return ScaledMaskedSoftmax.apply(input, mask, scale, ends)
 
     def mask_kind(self, mask, sq, sk):
-        """What the upper_triang fusion knows about ``mask``: ``"causal"``, a sliding-window width, or
-        None -- use the mask tensor (general fusion, ``sq != sk``, any other pattern, or a
-        classification that has not arrived yet).  See ``classify_mask``."""
-        if not self.upper_triang_mask_fusion or sq != sk:
+        """What the module knows about ``mask``: ``"causal"``, a sliding-window width, or None -- use
+        the mask tensor (``sq != sk``, any other pattern, or a classification that has not arrived
+        yet).  See ``classify_mask``.  The general fusion asks too: GPT-NeoX hands it the same causal
+        masks (``scaled_masked_softmax_fusion``), and a mask that has been read and found causal is
+        served by the kernels that read no mask -- but nothing is taken on trust there, since its
+        masks may be anything."""
+        if sq != sk:
             return None
-        return self.classify_mask(mask)
+        if self.upper_triang_mask_fusion:
+            return self.classify_mask(mask)
+        if self.general_mask_fusion and self.causal_mask_check != "trust":
+            return self.classify_mask(mask)
+        return None
 
     def classify_mask(self, mask):
         """``"causal"`` -- the mask hides exactly the keys ``j > i``, or ``causal_mask_check`` is

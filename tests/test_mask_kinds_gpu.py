@@ -245,10 +245,17 @@ def test_module_serves_sliding_window_masks_with_the_window_kernel(device):
     xs = scores((1, 2, 200, 200), dtype, device, 5)
     assert mod.mask_kind(small, 200, 200) == 17
     assert torch.equal(mod(xs, small), masked_ext.forward(xs, small, 0.25))
-    # general fusion never classifies: the mask tensor is used as it is
+    # general fusion gets the same masks from GPT-NeoX (scaled_masked_softmax_fusion) and uses what the scan
+    # has found -- the same result by the kernel that reads no mask -- but takes nothing on trust
     gen_mod = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.25)
-    assert gen_mod.mask_kind(window, s, s) is None
-    assert torch.equal(gen_mod(x, window), masked_ext.forward(x, window, 0.25))
+    assert gen_mod.mask_kind(window, s, s) == w
+    yg = gen_mod(x, window)
+    assert torch.equal(yg, y.detach())
+    assert max_err(yg, masked_ext.forward(x, window, 0.25)) <= 2.0 ** -8  # a unit in the last place of bf16 at most
+    trusting = FusedScaleMaskSoftmax(False, True, SoftmaxFusionTypes.general, R.gpt2_attention_mask_func, True, 0.25,
+                                     causal_mask_check="trust")
+    assert trusting.mask_kind(window, s, s) is None
+    assert torch.equal(trusting(x, window), masked_ext.forward(x, window, 0.25))
 
 
 def test_default_module_never_synchronises_the_host(device, monkeypatch):
