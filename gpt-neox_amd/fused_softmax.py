@@ -31,7 +31,11 @@ Deliberate differences from the reference:
   run the mask-tensor kernel, which is right for any mask --, ``"verify"`` waits for that answer
   (one host synchronisation per new mask), and ``"trust"`` restores the reference's behaviour of
   never reading the mask (megatron/model/fused_softmax.py:173-179).  A causal-fusion call with ``sq != sk`` (a step
-  against a key/value cache, where the reference asserts) also runs the mask-tensor kernel;
+  against a key/value cache, where the reference asserts) also runs the mask-tensor kernel.  The
+  general fusion uses the same verdicts for square masks (never on trust), and whatever call the
+  mask-tensor kernel serves tells it where every mask row's visible keys end once the same scan has
+  found that worthwhile (``skip_hidden_tails``): the padding of a batch is then neither fetched nor
+  computed, with the same bits as before;
 * masked scores are excluded, so their probability is exactly 0 as in the torch
   path (the reference's padded kernel fills -10000), and a fully masked row is
   uniform ``1/sk`` as in the torch path;
