@@ -683,13 +683,17 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
         """The ``row_end`` hint for a call that the mask-tensor kernel serves, or None: switched off,
         ``"trust"`` (the mask is never read), a mask in another layout than ``[1 or b, 1, sq, sk]``
         on the GPU, a mask that hides less than a sixteenth of its keys behind its rows' last visible
-        ones, or a scan that has not arrived yet."""
+        ones, a scan that has not arrived yet, or a HIP graph being captured."""
         if not self.skip_hidden_tails or self.causal_mask_check == "trust":
             return None
         if not (mask.is_cuda and self._mask_fits_the_mask_kernel(mask, b, sq, sk)):
             return None
         facts = self._mask_facts(mask)
-        return None if facts is None else facts[1]
+        if facts is None or facts[1] is None:
+            return None
+        # the hint lives in the memo, which may drop it when many masks have passed: a HIP graph that
+        # recorded its address could outlive it, so captured launches go without
+        return None if torch.cuda.is_current_stream_capturing() else facts[1]
 
     def _mask_facts(self, mask):
         """The memo's answer: ``(verdict, ends)`` -- the verdict False for a mask that is not a causal

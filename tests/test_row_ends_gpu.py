@@ -267,3 +267,30 @@ def test_causal_fusion_uses_the_hint_for_masks_that_are_not_causal(device, monke
     assert m.mask_kind(causal, s, s) == "causal"
     m(x, causal)
     assert seen["hinted"] == 1
+
+
+def test_launches_recorded_into_a_hip_graph_go_without_the_hint(device, monkeypatch):
+    # the hint lives in the module's memo and a graph could outlive it: captured launches use the plain pass
+    b, heads, s = 2, 2, 1024
+    x = torch.randn(b, heads, s, s, device=device).bfloat16()
+    mask = masks("padding", b, s, s, device, 11)
+    m = module(SoftmaxFusionTypes.general, "verify")
+    seen = calls_with_hint(monkeypatch)
+    want = m(x, mask)
+    assert seen["hinted"] == 1 and m.hidden_tails(mask, b, s, s) is not None
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            assert m.hidden_tails(mask, b, s, s) is None
+            out = m(x, mask)
+    torch.cuda.synchronize()
+    assert seen["hinted"] == 1
+    for _ in range(3):
+        out.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    assert torch.equal(m(x, mask), want) and seen["hinted"] == 2
