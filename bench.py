@@ -915,6 +915,9 @@ def run_studies(c):
             lens = torch.randint(256, sk + 1, (b,), device=dev, generator=gen(1401))
             pad = (torch.arange(sk, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(b, 1, sq, sk).contiguous()
             pair("cfg2 padded fwd [8,16,1024,1024] fp16", b, heads, sq, sk, dtype, scale, pad, 6, 100)
+            lens = torch.randint(64, 513, (32,), device=dev, generator=gen(1403))
+            pad = (torch.arange(512, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(32, 1, 512, 512).contiguous()
+            pair("padded fwd [32,12,512,512] fp16", 32, 12, 512, 512, torch.float16, 0.125, pad, 6, 100)
             lens = torch.randint(1024, 4097, (4,), device=dev, generator=gen(1402))
             pad = (torch.arange(4096, device=dev)[None, None, None, :] >= lens[:, None, None, None]).expand(4, 1, 4096, 4096).contiguous()
             pair("padded fwd [4,16,4096,4096] bf16", 4, 16, 4096, 4096, torch.bfloat16, 0.125, pad, 2, 30)

@@ -816,6 +816,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_packed_kernel(SoftmaxArgs a) 
         for (int c = 0; c < C; ++c) {
             const int col = col0 + c * kChunk;
             bool active = col < len[p];
+            // (SoftmaxArgs::row_end is not looked at here: it spared nothing more and cost a load per row)
             if constexpr (MASK == Mask::Bytes && kSkipHidden && !kRag) active = active && !all_hidden(mk[p][c]);
             raw[p][c] = packed_ld<kLdNt>(rx, (lr * sk + col) * 2u, active);
             if constexpr ((FLAGS & kBias) != 0) {
