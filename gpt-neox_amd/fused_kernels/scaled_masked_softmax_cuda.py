@@ -271,6 +271,11 @@ def scan_mask(mask):
     return record, row_end
 
 
+def launch_stream(tensor):
+    """The raw handle of the stream a call on ``tensor`` is launched on now."""
+    return _stream(tensor)
+
+
 def hidden_tail_keys(record):
     """The number of keys that the ``row_end`` hint of :func:`scan_mask` saves: the sum over the
     mask rows of ``sk - row_end`` (rows without a visible key not counted), from the eight numbers

@@ -100,7 +100,8 @@ class _MaskVerdict:
     any other mask; ``ends``: where every row's visible keys end (the ``row_end`` hint of the
     mask-tensor kernels, a device tensor) if that saves a sixteenth of the keys or more, else None.
     Both are None while the device-side scan is still running (then ``pending`` holds the pinned
-    result slot, the event that follows the copy, the hint and the number of keys of the mask)."""
+    result slot, the event that follows the copy, the hint, the number of keys of the mask and the
+    stream the scan runs on)."""
 
     __slots__ = ("storage", "version", "verdict", "ends", "pending")
 
@@ -115,7 +116,7 @@ class _MaskVerdict:
         """The verdict if it is known by now.  ``wait``: True blocks until it is, False asks the
         event, None does not touch the event at all (for use while a HIP graph is captured)."""
         if self.verdict is None and self.pending is not None and wait is not None:
-            slot, event, ends, keys = self.pending
+            slot, event, ends, keys, _ = self.pending
             if wait:
                 event.synchronize()
             if wait or event.query():
@@ -132,6 +133,13 @@ class _MaskVerdict:
     def facts(self, wait):
         """``(verdict, ends)``, or None while they are on their way."""
         return None if self.poll(wait) is None else (self.verdict, self.ends)
+
+    def early_ends(self, stream):
+        """The hint of a scan that is still on its way, for a launch on the stream the scan runs on: the
+        launch follows the scan there and finds the array filled, whatever the host knows by then."""
+        if self.pending is None or self.pending[4] != stream:
+            return None
+        return self.pending[2]
 
 
 class _CausalMaskMemo:
@@ -183,6 +191,11 @@ class _CausalMaskMemo:
         """``(verdict, ends)`` likewise."""
         hit = self._entry(mask)
         return None if hit is None else hit.facts(wait)
+
+    def early_ends(self, mask):
+        """See ``_MaskVerdict.early_ends``; None for a mask without a scan on its way."""
+        hit = self._entry(mask)
+        return None if hit is None else hit.early_ends(_masked_ext.launch_stream(mask))
 
     def _result_slot(self, entry):
         """Eight pinned host words for the record of ``entry``.  The slots are handed out in turn; an
@@ -237,7 +250,7 @@ class _CausalMaskMemo:
                 slot.copy_(record, non_blocking=True)
                 event = torch.cuda.Event()
                 event.record()
-            entry.pending = (slot, event, ends, mask.numel())
+            entry.pending = (slot, event, ends, mask.numel(), _masked_ext.launch_stream(mask))
         else:
             square = mask.shape[-1] == mask.shape[-2]
             entry = _MaskVerdict(storage, mask._version, verdict=self._classify_on_host(mask) if square else False)
@@ -499,9 +512,9 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     causal_mask_check (not in the reference): ``"lazy"`` (default) | ``"verify"`` | ``"trust"`` -- how
         the upper_triang fusion treats the mask it is given; see the module text.
     skip_hidden_tails (not in the reference, default True): a call that the mask-tensor kernel serves
-        tells it where every row's visible keys end, once the scan of the mask has found that this
-        spares a sixteenth of the keys or more (the padding of a batch of sequences of different
-        lengths): the kernel then fetches nothing behind those points.  The scan is the one of
+        tells it where every row's visible keys end, unless the scan of the mask has found that this
+        spares less than a sixteenth of the keys (the padding of a batch of sequences of different
+        lengths is more): the kernel then fetches nothing behind those points.  The scan is the one of
         ``causal_mask_check`` -- once per mask, never waited for under ``"lazy"``, never made under
         ``"trust"`` --, and the result is the same bit for bit.
 
@@ -682,18 +695,25 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
     def hidden_tails(self, mask, b, sq, sk):
         """The ``row_end`` hint for a call that the mask-tensor kernel serves, or None: switched off,
         ``"trust"`` (the mask is never read), a mask in another layout than ``[1 or b, 1, sq, sk]``
-        on the GPU, a mask that hides less than a sixteenth of its keys behind its rows' last visible
-        ones, a scan that has not arrived yet, or a HIP graph being captured."""
+        on the GPU, a mask known to hide less than a sixteenth of its keys behind its rows' last
+        visible ones, or a HIP graph being captured.  While the scan of a mask is still on its way
+        the hint is passed already, to launches on the scan's stream."""
         if not self.skip_hidden_tails or self.causal_mask_check == "trust":
             return None
         if not (mask.is_cuda and self._mask_fits_the_mask_kernel(mask, b, sq, sk)):
             return None
         facts = self._mask_facts(mask)
-        if facts is None or facts[1] is None:
+        if facts is not None and facts[1] is None:
             return None
         # the hint lives in the memo, which may drop it when many masks have passed: a HIP graph that
         # recorded its address could outlive it, so captured launches go without
-        return None if torch.cuda.is_current_stream_capturing() else facts[1]
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        if facts is None:
+            # the scan is still on its way: a launch on its stream comes after it and may use what it
+            # writes -- the first call with a fresh mask skips the hidden tails already
+            return _causal_memo.early_ends(mask)
+        return facts[1]
 
     def _mask_facts(self, mask):
         """The memo's answer: ``(verdict, ends)`` -- the verdict False for a mask that is not a causal

@@ -294,3 +294,27 @@ def test_launches_recorded_into_a_hip_graph_go_without_the_hint(device, monkeypa
         torch.cuda.synchronize()
         assert torch.equal(out, want)
     assert torch.equal(m(x, mask), want) and seen["hinted"] == 2
+
+
+def test_first_call_with_a_fresh_mask_uses_the_scan_that_is_still_on_its_way(device, monkeypatch):
+    # lazy: nobody waits for the scan's record, but a launch on the scan's stream follows it and finds
+    # the rows' ends in device memory -- a fresh causal mask costs its upper triangle not even once
+    b, heads, s = 1, 2, 2048
+    x = torch.randn(b, heads, s, s, device=device).bfloat16()
+    m = module(SoftmaxFusionTypes.upper_triang, "lazy")
+    seen = calls_with_hint(monkeypatch)
+    want = masked_ext.forward(x, R.get_attn_mask(s, device), 0.5)
+    for _ in range(3):
+        fresh = R.get_attn_mask(s, device)
+        before = seen["hinted"]
+        y = m(x, fresh)
+        kind = m.mask_kind(fresh, s, s)
+        assert seen["hinted"] == before + 1 or kind == "causal"  # (unless the record has arrived already)
+        assert torch.equal(y, want)
+    # on another stream the scan's array may not be ready: no hint there until the record has arrived
+    fresh = R.get_attn_mask(s, device)
+    m(x, fresh)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert m.hidden_tails(fresh, b, s, s) is None or m.mask_kind(fresh, s, s) is not None
+    torch.cuda.synchronize()
