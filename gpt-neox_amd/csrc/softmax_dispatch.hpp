@@ -14,9 +14,9 @@
 //   chunks <= 32   16 waves per row, 1024-thread block               (sk <= 16384)
 //                  forward, in the lower 3/4 of each of these three ranges (7/8 of the last):
 //                  half as many waves with 3 (4) chunks each; causal backward likewise at
-//                  8193-12288 columns; mask-tensor forward at 513-768 and 1025-1536 columns and
-//                  causal forward at 1025-1408: packed kernel, two rows of two chunks or one row
-//                  of three chunks per wave
+//                  8193-12288 columns; mask-tensor forward at 513-2048 columns (unless the call
+//                  knows where its rows end) and causal forward at 1025-1408: packed kernel, two
+//                  rows of two chunks or one row of three or four chunks per wave
 //   chunks <= 64   16 waves per row with 3 or 4 chunks per wave      (sk <= 32768)
 //   longer rows    staged in LDS, one 1024-thread block per row: in half of a CU's LDS, two
 //                  blocks per CU (sk <= 40448), or in all of it       (sk <= 81408)
@@ -179,15 +179,23 @@ static std::optional<hipError_t> dispatch_aligned(const SoftmaxArgs& a, bool vec
     }
     if (chunks == 1) return dispatch_short_rows<T, M, BWD, EXTRA>(a, st);
     if constexpr (!BWD && M == Mask::Bytes) {
-        // mask-tensor forward, 513-768 columns: the packed kernel with two rows of two chunks per wave
-        // keeps four accesses per tensor in flight where the row kernel's second chunk is mostly empty
-        // (-17 % at 520-640 columns, -8 % at 768, +1 % at 896; the causal forward loses 2-10 % with it);
-        // 1025-1536 columns: one row of three chunks per wave instead of two waves with four slots
-        // (-9 % at 1032 and 1152 columns, -5 % at 1280, -1 % at 1536; four chunks: +2...4 %); with
-        // dropout folded in both steps gain 4-11 %
+        // mask-tensor forward, 513-2048 columns: the packed kernel -- two rows of two chunks, or one row of
+        // three or four chunks per wave -- keeps four accesses per tensor in flight and fetches no score of
+        // a lane whose keys are all hidden.  Against the row kernels (two waves with four chunk slots from
+        // 1025 columns on): -17 % at 520-640 columns, -8 % at 768, -9 % at 1032 and 1152, -5 % at 1280, -1 %
+        // at 1536 whatever the mask; at 769-1024 and 1537-2048 columns -5...-19 % under padding and causal
+        // masks and +0...3 % under masks that hide nothing or hide at random.  With dropout folded in
+        // the steps up to 1536 columns gain 4-11 %.  A call that knows where its rows end
+        // (SoftmaxArgs::row_end, which the packed kernels do not look at) takes the row kernel at two
+        // chunks, which ends the row there without waiting for the mask bytes and sums in the same order
+        // (-16 % at 640 columns, -3...-7 % at 1024 against the packed kernel); at three and four chunks it
+        // measured -3...+9 % and would sum in another order, so those stay with the packed kernel.
         const bool fits32 = a.mask_bytes != 0 && (a.bias == nullptr || a.bias_bytes != 0);
-        if (chunks == 2 && a.sk <= 768 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
-        if (chunks == 3 && fits32) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
+        if (fits32) {
+            if (chunks == 2 && a.row_end == nullptr) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 2, 2>(a, st);
+            if (chunks == 3) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 3>(a, st);
+            if (chunks == 4) return launch_packed_shape<T, M, BWD, EXTRA, kWave, 1, 4>(a, st);
+        }
     }
     if constexpr (!BWD && M == Mask::Causal) {
         // causal forward, 1025-1408 columns: one row of three chunks per wave instead of two waves with

@@ -49,9 +49,9 @@ struct SoftmaxArgs {
     uint32_t affine_blocks;        // leading blocks that take part: a multiple of 8
     int32_t window;                // kBand kernels: row i sees the keys max(0, i - window) .. i
     // Mask-tensor forward and full-row backward, optional: per mask row [mask_b * sq], the number of
-    // leading keys that can be visible -- every key from there on is hidden whatever its mask byte
-    // says (backward: its probability is zero); 0 = the whole row.  Needs sq, rows_per_mask_batch
-    // and mask_bcast.
+    // leading keys that can be visible -- the caller's promise that the mask hides every key from
+    // there on (backward: that its probability is zero), which a kernel may use or not; 0 = the
+    // whole row.  Needs sq, rows_per_mask_batch and mask_bcast.
     const int32_t* row_end;
 };
 

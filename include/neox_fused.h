@@ -235,10 +235,12 @@ int neox_mask_scan(int32_t* record, int32_t* row_end, const uint8_t* mask, int32
                    void* stream);
 
 /*
- * Mask-tensor softmax forward that is told where the visible keys of every mask row end and fetches
- * neither scores nor mask bytes (nor bias) behind that point: row_end[r], int32 [mask_b * sq] as
- * neox_mask_scan writes it, promises that every key j >= row_end[r] of mask row r is hidden, whatever
- * the mask byte says; 0 (or a value >= sk, or row_end == NULL) promises nothing for that row.  The
+ * Mask-tensor softmax forward that is told where the visible keys of every mask row end and need
+ * fetch neither scores nor mask bytes (nor bias) behind that point: row_end[r], int32 [mask_b * sq] as
+ * neox_mask_scan writes it, is the caller's promise that the mask hides every key j >= row_end[r] of
+ * mask row r; 0 (or a value >= sk, or row_end == NULL) promises nothing for that row.  A kernel may use
+ * the promise or read the mask bytes (rows of up to 512 columns and of 1025 to 2048 skip hidden keys
+ * from the bytes themselves), so a false promise gives an unspecified mixture of the two.  The
  * result is that of the plain entry points, bit for bit: y = softmax over the visible keys, exact
  * zeros elsewhere, a fully hidden row uniform 1/sk.  One entry point for every feature set:
  * alibi_slopes and bias (with bias_b) are optional as in neox_masked_softmax_bias_fwd; y_drop == NULL

@@ -5,8 +5,8 @@ What is pinned: the scan against plain torch (last visible key + 1 per mask row,
 keys behind those points, the causal verdict in the first four words); the hinted forward and
 backward passes bit-equal to the plain ones for every kernel family, mask pattern and feature set --
 they compute the same numbers in the same order and only fetch less --, so they inherit the plain
-passes' parity with the oracle (checked once more here against the fp32 expression); keys behind a row's end count as
-hidden whatever their mask bytes say; and the Python module passing the hint along by itself, without
+passes' parity with the oracle (checked once more here against the fp32 expression); ends given by the caller instead of
+the scan; and the Python module passing the hint along by itself, without
 a host synchronisation, once it has seen that a mask hides enough.
 """
 import pytest
@@ -149,18 +149,23 @@ def test_hinted_backward_equals_the_plain_one(device, shape, kind):
         masked_ext.backward(g.clone(), y, 0.25, row_end=row_end[:-1])
 
 
-def test_keys_behind_a_rows_end_count_as_hidden(device):
-    # the hint is a promise of the caller: a shorter end than the mask's hides more
-    b, heads, sq, sk = 2, 2, 6, 2048
-    x = torch.empty((b, heads, sq, sk), dtype=torch.bfloat16, device=device).normal_(0.0, 4.0, generator=gen(device, 1))
-    mask = torch.zeros(b, 1, sq, sk, dtype=torch.bool, device=device)
-    ends = torch.tensor([2048, 1000, 513, 512, 8, 1] * b, dtype=torch.int32, device=device)
-    y = masked_ext.forward(x, mask, 0.5, row_end=ends)
-    hidden = torch.arange(sk, device=device).view(1, 1, 1, sk) >= ends.view(b, 1, sq, 1)
-    assert torch.equal(y, masked_ext.forward(x, hidden, 0.5))
-    # 0 and values beyond sk promise nothing
-    none = torch.tensor([0, sk, sk + 5, -3, 0, 2**31 - 1] * b, dtype=torch.int32, device=device)
-    assert torch.equal(masked_ext.forward(x, mask, 0.5, row_end=none), masked_ext.forward(x, mask, 0.5))
+def test_row_ends_given_by_the_caller(device):
+    # the hint is a promise of the caller -- every key at or behind a row's end is masked in the mask
+    # tensor too -- which a kernel may use or not: ends that the caller knows (here: the lengths a padding
+    # mask was built from) serve like those of the scan, and 0 or a value beyond sk promises nothing
+    b, heads, sq = 2, 2, 6
+    for sk in (1024, 2048, 8192):
+        x = torch.empty((b, heads, sq, sk), dtype=torch.bfloat16, device=device).normal_(0.0, 4.0, generator=gen(device, 1))
+        ends = torch.tensor([sk, 1000, 513, 512, 8, 1] * b, dtype=torch.int32, device=device)
+        hidden = torch.arange(sk, device=device).view(1, 1, 1, sk) >= ends.view(b, 1, sq, 1)
+        want = masked_ext.forward(x, hidden, 0.5)
+        assert torch.equal(masked_ext.forward(x, hidden, 0.5, row_end=ends), want)
+        longer = (ends + 3).clamp(max=sk)  # a weaker promise is still a true one
+        assert torch.equal(masked_ext.forward(x, hidden, 0.5, row_end=longer), want)
+        none = torch.tensor([0, sk, sk + 5, -3, 0, 2**31 - 1] * b, dtype=torch.int32, device=device)
+        assert torch.equal(masked_ext.forward(x, hidden, 0.5, row_end=none), want)
+        g = torch.randn_like(x)
+        assert torch.equal(masked_ext.backward(g.clone(), want, 0.5, row_end=longer), masked_ext.backward(g.clone(), want, 0.5))
 
 
 def test_row_end_of_the_wrong_kind_is_refused(device):
