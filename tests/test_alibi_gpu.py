@@ -59,7 +59,7 @@ def oracle(x, mask, slopes, scale, bias=None):
     return R.softmax_fp32(t, mask, scale)
 
 
-# [b, np, sq, sk]: packed kernels (<= 512 columns; 513-768 and 1025-1536 with a mask tensor), one to
+# [b, np, sq, sk]: packed kernels (<= 512 columns; 513-2048 with a mask tensor), one to
 # sixteen waves per row, ragged rows (sk % 8 != 0), the element-wise kernels (sk < 8), rows staged in LDS (sk > 32768),
 # and one-query decode steps
 MASKED_ALIBI_SHAPES = [(2, 3, 8, 8), (1, 4, 40, 40), (2, 2, 136, 136), (1, 6, 512, 512), (1, 2, 640, 640), (2, 2, 1000, 1000),

@@ -1,6 +1,6 @@
 """Kernel instantiations that only unusual calls reach, each against the oracle (through the C-ABI).
 
-* rows that the packed kernels take (at most 512 columns; 513-768 and 1025-1536 with a mask tensor)
+* rows that the packed kernels take (at most 512 columns; 513-2048 with a mask tensor)
   whose mask or bias tensor is larger than a 32-bit buffer range (4 GiB): the row kernels with a
   64-bit address per row instead;
 * packed kernels on tensors beyond 4 GiB;
@@ -57,7 +57,7 @@ def sample_rows(n, device, seed):
 # softmax: short rows with tensors beyond 4 GiB
 # ---------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("sk", [512, 511, 640, 1536])  # aligned / ragged short rows; the packed kernels' longer rows
+@pytest.mark.parametrize("sk", [512, 511, 640, 1536, 2048])  # aligned / ragged short rows; the packed kernels' longer rows
 def test_rows_with_a_mask_tensor_beyond_4_gib(device, sk, dtype):
     sq = FOUR_GIB // sk + 16
     assert sq * sk > FOUR_GIB
