@@ -103,20 +103,21 @@ class _MaskVerdict:
     result slot, the event that follows the copy, the hint, the number of keys of the mask and the
     stream the scan runs on)."""
 
-    __slots__ = ("storage", "version", "verdict", "ends", "pending")
+    __slots__ = ("storage", "version", "verdict", "ends", "stream", "pending")
 
     def __init__(self, storage, version, verdict=None, pending=None):
         self.storage = weakref.ref(storage)
         self.version = version
         self.verdict = verdict
         self.ends = None
+        self.stream = None  # the stream the scan ran on, whose allocator pool holds ``ends``
         self.pending = pending
 
     def poll(self, wait):
         """The verdict if it is known by now.  ``wait``: True blocks until it is, False asks the
         event, None does not touch the event at all (for use while a HIP graph is captured)."""
         if self.verdict is None and self.pending is not None and wait is not None:
-            slot, event, ends, keys, _ = self.pending
+            slot, event, ends, keys, self.stream = self.pending
             if wait:
                 event.synchronize()
             if wait or event.query():
@@ -131,8 +132,8 @@ class _MaskVerdict:
         return self.verdict
 
     def facts(self, wait):
-        """``(verdict, ends)``, or None while they are on their way."""
-        return None if self.poll(wait) is None else (self.verdict, self.ends)
+        """``(verdict, ends, stream of the scan)``, or None while they are on their way."""
+        return None if self.poll(wait) is None else (self.verdict, self.ends, self.stream)
 
     def early_ends(self, stream):
         """The hint of a scan that is still on its way, for a launch on the stream the scan runs on: the
@@ -188,7 +189,7 @@ class _CausalMaskMemo:
         return None if hit is None else hit.poll(wait)
 
     def lookup_facts(self, mask, wait=False):
-        """``(verdict, ends)`` likewise."""
+        """``(verdict, ends, stream)`` likewise."""
         hit = self._entry(mask)
         return None if hit is None else hit.facts(wait)
 
@@ -233,7 +234,7 @@ class _CausalMaskMemo:
         return self._scan(mask).poll(wait)
 
     def facts(self, mask, wait=True):
-        """``(verdict, ends)`` of ``_MaskVerdict``, or None (still running and ``wait`` is False)."""
+        """``(verdict, ends, stream)`` of ``_MaskVerdict``, or None (still running and ``wait`` is False)."""
         return self._scan(mask).facts(wait)
 
     def _scan(self, mask):
@@ -713,16 +714,21 @@ class FusedScaleMaskSoftmax(torch.nn.Module):
             # the scan is still on its way: a launch on its stream comes after it and may use what it
             # writes -- the first call with a fresh mask skips the hidden tails already
             return _causal_memo.early_ends(mask)
-        return facts[1]
+        ends = facts[1]
+        if facts[2] != _masked_ext.launch_stream(mask):
+            # a launch on another stream than the one whose pool the array came from: the allocator
+            # must not hand the block on before this launch is through, should the memo drop it
+            ends.record_stream(torch.cuda.current_stream(mask.device))
+        return ends
 
     def _mask_facts(self, mask):
-        """The memo's answer: ``(verdict, ends)`` -- the verdict False for a mask that is not a causal
-        one --, or None while it is on its way."""
+        """The memo's answer: ``(verdict, ends, stream)`` -- the verdict False for a mask that is not a
+        causal one --, or None while it is on its way."""
         last = self._last_mask
         if last is not None and last[0]() is mask and last[1] == mask._version:
             return last[2]  # the tensor object of the previous call, unchanged: no lookup
         if mask.dim() != 4 or mask.shape[1] != 1 or mask.dtype not in (torch.bool, torch.uint8):
-            return (False, None)
+            return (False, None, None)
         if mask.is_cuda and torch.cuda.is_current_stream_capturing():
             facts = _causal_memo.lookup_facts(mask, wait=None)
         else:

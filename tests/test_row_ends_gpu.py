@@ -323,3 +323,19 @@ def test_first_call_with_a_fresh_mask_uses_the_scan_that_is_still_on_its_way(dev
     with torch.cuda.stream(side):
         assert m.hidden_tails(fresh, b, s, s) is None or m.mask_kind(fresh, s, s) is not None
     torch.cuda.synchronize()
+
+
+def test_hint_on_another_stream_than_the_scans(device, monkeypatch):
+    b, heads, s = 2, 2, 1024
+    x = torch.randn(b, heads, s, s, device=device).bfloat16()
+    mask = masks("padding", b, s, s, device, 13)
+    m = module(SoftmaxFusionTypes.general, "verify")
+    seen = calls_with_hint(monkeypatch)
+    want = m(x, mask)  # scanned on the default stream
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            assert torch.equal(m(x, mask), want)
+    side.synchronize()
+    assert seen["hinted"] == 4
