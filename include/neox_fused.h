@@ -26,6 +26,15 @@
 extern "C" {
 #endif
 
+/*
+ * ABI versions.  A version is bumped when an entry point is added or its parameter list changes; the
+ * Python binding refuses a library of another version.
+ *   4  + neox_mask_scan, neox_masked_softmax_ends_fwd, neox_masked_softmax_ends_bwd
+ *   3  + neox_masked_softmax_alibi_fwd, neox_sliding_window_softmax_fwd/_bwd, neox_mask_classify;
+ *      neox_*_softmax_bias_fwd and neox_masked_softmax_dropout_fwd take ALiBi slopes too
+ *   2  + the dropout, bias and ALiBi entry points, neox_rope_apply_freqs
+ *   1  the four softmax entry points, neox_rope_apply, neox_get_batch_per_block
+ */
 #define NEOX_FUSED_ABI_VERSION 4
 
 typedef enum neox_dtype {
